@@ -1,0 +1,277 @@
+"""ctypes binding of the CPU oracle (liboracle.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by the smoke check and by the CPU-baseline leg of
+bench.py.  The shipped package never imports this module.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "liboracle.so")
+
+
+def build(force=False):
+    srcs = [os.path.join(_HERE, f) for f in ("oracle_pr.c", "oracle_gcn.c", "Makefile")]
+    stale = (not os.path.exists(_SO)) or any(os.path.getmtime(s) > os.path.getmtime(_SO) for s in srcs)
+    if force or stale:
+        subprocess.check_call(["make", "-C", _HERE, "-B", "liboracle.so"], stdout=subprocess.DEVNULL)
+    return _SO
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        _lib = C.CDLL(_SO)
+        _lib.orc_cross_entropy.restype = C.c_float
+        _lib.orc_accuracy.restype = C.c_float
+        _lib.orc_gcn_forward_backward.restype = C.c_float
+        _lib.orc_go_pr_create.restype = C.c_void_p
+        _lib.orc_go_pr_peval.restype = C.c_int64
+        _lib.orc_go_pr_inceval.restype = C.c_int64
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _i32(a):
+    return np.ascontiguousarray(a, dtype=np.int32)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+# ---------------------------------------------------------------- PageRank
+def build_graph(global_n, u, v):
+    """Local relabel + stable out-edge CSR. Returns (n_local, g2l, l2g, index, dst)."""
+    u, v = _i32(u), _i32(v)
+    E = len(u)
+    g2l = np.empty(global_n, np.int32)
+    l2g = np.empty(global_n, np.int32)
+    index = np.empty(global_n + 1, np.int32)
+    dst = np.empty(max(E, 1), np.int32)
+    n = lib().orc_build_graph(C.c_int(global_n), C.c_int(E), _p(u), _p(v), _p(g2l), _p(l2g), _p(index), _p(dst))
+    return n, g2l, l2g[:n].copy(), index[: n + 1].copy(), dst[:E].copy()
+
+
+def pr_pull_f64(row_ptr, col_idx, inv_outdeg, alpha, iters, nthreads=0):
+    row_ptr = np.ascontiguousarray(row_ptr, np.int64)
+    col_idx = _i32(col_idx)
+    inv_outdeg = np.ascontiguousarray(inv_outdeg, np.float64)
+    n = len(row_ptr) - 1
+    out = np.empty(n, np.float64)
+    lib().orc_pr_pull_f64(C.c_int64(n), _p(row_ptr), _p(col_idx), _p(inv_outdeg), C.c_double(alpha),
+                          C.c_int(iters), _p(out), C.c_int(nthreads))
+    return out
+
+
+class PushState:
+    """State of the delta-push restatement of pr.cu (dtype float32 = the reference's, or float64)."""
+
+    def __init__(self, index, dst, outdeg, nglobal, dtype=np.float32, mirror2worker=None):
+        self.index, self.dst, self.outdeg = _i32(index), _i32(dst), _i32(outdeg)
+        self.n = len(self.index) - 1
+        self.nglobal = int(nglobal)
+        self.dtype = np.dtype(dtype)
+        self.suf = "f32" if self.dtype == np.float32 else "f64"
+        self.ct = C.c_float if self.dtype == np.float32 else C.c_double
+        self.m2w = _i32(mirror2worker) if mirror2worker is not None else np.full(self.n, -1, np.int32)
+        self.pr = np.zeros(self.n, self.dtype)
+        self.acc = np.zeros(self.n, self.dtype)
+        self.diff = np.zeros(self.n, self.dtype)
+        self.gacc = np.zeros(1, self.dtype)
+        self.gdiff = np.zeros(1, self.dtype)
+        self.active = np.zeros(self.n, np.int32)
+
+    def peval(self):
+        f = getattr(lib(), "orc_pr_push_peval_" + self.suf)
+        return f(C.c_int(self.n), C.c_int(self.nglobal), _p(self.index), _p(self.dst), _p(self.outdeg),
+                 _p(self.m2w), _p(self.pr), _p(self.acc), _p(self.diff), _p(self.gacc), _p(self.gdiff),
+                 _p(self.active))
+
+    def inceval(self, alpha=0.85, eps=1e-6):
+        f = getattr(lib(), "orc_pr_push_inceval_" + self.suf)
+        return f(C.c_int(self.n), C.c_int(self.nglobal), _p(self.index), _p(self.dst), _p(self.outdeg),
+                 _p(self.m2w), self.ct(alpha), self.ct(eps), _p(self.pr), _p(self.acc), _p(self.diff),
+                 _p(self.gacc), _p(self.gdiff), _p(self.active))
+
+
+class GoPR:
+    """Map-based restatement of the Go CPU 'pr' job."""
+
+    def __init__(self, u, v, targets_num):
+        self.u, self.v, self.tn = _i32(u), _i32(v), _i32(targets_num)
+        self.h = C.c_void_p(lib().orc_go_pr_create(C.c_int(len(self.u)), _p(self.u), _p(self.v), _p(self.tn)))
+
+    def peval(self):
+        return lib().orc_go_pr_peval(self.h)
+
+    def inceval(self, alpha=0.85, eps=0.01):
+        me = C.c_float(0)
+        it = lib().orc_go_pr_inceval(self.h, C.c_float(alpha), C.c_float(eps), C.byref(me))
+        return it, me.value
+
+    def read(self):
+        n = lib().orc_go_pr_num_nodes(self.h)
+        ids = np.empty(n, np.int32)
+        pr = np.empty(n, np.float32)
+        lib().orc_go_pr_read(self.h, _p(ids), _p(pr))
+        return ids, pr
+
+    def close(self):
+        if self.h:
+            lib().orc_go_pr_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        self.close()
+
+
+# ---------------------------------------------------------------- GCN
+def edge_values(rp, ci, in_deg, out_deg):
+    rp, ci, in_deg, out_deg = _i32(rp), _i32(ci), _i32(in_deg), _i32(out_deg)
+    val = np.empty(len(ci), np.float32)
+    lib().orc_edge_values(C.c_int(len(rp) - 1), _p(rp), _p(ci), _p(in_deg), _p(out_deg), _p(val))
+    return val
+
+
+def csr_transpose(n_rows, n_cols, rp, ci, v=None):
+    rp, ci = _i32(rp), _i32(ci)
+    v = None if v is None else _f32(v)
+    rpT = np.empty(n_cols + 1, np.int32)
+    ciT = np.empty(len(ci), np.int32)
+    vT = None if v is None else np.empty(len(ci), np.float32)
+    lib().orc_csr_transpose(C.c_int(n_rows), C.c_int(n_cols), _p(rp), _p(ci), _p(v), _p(rpT), _p(ciT), _p(vT))
+    return rpT, ciT, vT
+
+
+def spmm_f32(rp, ci, val, B):
+    rp, ci, val, B = _i32(rp), _i32(ci), _f32(val), _f32(B)
+    n, K = len(rp) - 1, B.shape[1]
+    out = np.empty((n, K), np.float32)
+    lib().orc_spmm_f32(C.c_int(n), _p(rp), _p(ci), _p(val), _p(B), C.c_int(K), _p(out), C.c_int(K), C.c_int(K))
+    return out
+
+
+def spmm_f64acc(rp, ci, val, B):
+    rp, ci, val, B = _i32(rp), _i32(ci), _f32(val), _f32(B)
+    n, K = len(rp) - 1, B.shape[1]
+    out = np.empty((n, K), np.float64)
+    lib().orc_spmm_f64acc(C.c_int(n), _p(rp), _p(ci), _p(val), _p(B), C.c_int(K), _p(out), C.c_int(K), C.c_int(K))
+    return out
+
+
+def sgemm_f32(transA, transB, A, B, alpha=1.0, beta=0.0, Cin=None):
+    A, B = _f32(A), _f32(B)
+    M = A.shape[1] if transA else A.shape[0]
+    K = A.shape[0] if transA else A.shape[1]
+    N = B.shape[0] if transB else B.shape[1]
+    out = np.zeros((M, N), np.float32) if Cin is None else _f32(Cin).copy()
+    lib().orc_sgemm_f32(C.c_int(int(transA)), C.c_int(int(transB)), C.c_int(M), C.c_int(N), C.c_int(K),
+                        C.c_float(alpha), _p(A), C.c_int(A.shape[1]), _p(B), C.c_int(B.shape[1]),
+                        C.c_float(beta), _p(out), C.c_int(N))
+    return out
+
+
+def sgemm_f64acc(transA, transB, A, B):
+    A, B = _f32(A), _f32(B)
+    M = A.shape[1] if transA else A.shape[0]
+    K = A.shape[0] if transA else A.shape[1]
+    N = B.shape[0] if transB else B.shape[1]
+    out = np.empty((M, N), np.float64)
+    lib().orc_sgemm_f64acc(C.c_int(int(transA)), C.c_int(int(transB)), C.c_int(M), C.c_int(N), C.c_int(K),
+                           _p(A), C.c_int(A.shape[1]), _p(B), C.c_int(B.shape[1]), _p(out), C.c_int(N))
+    return out
+
+
+def relu_forward(x, training=True):
+    x = _f32(x).copy()
+    mask = np.zeros(x.size, np.uint8)
+    lib().orc_relu_forward(_p(x), _p(mask), C.c_int64(x.size), C.c_int(int(training)))
+    return x, mask.reshape(x.shape)
+
+
+def relu_backward(g, mask):
+    g = _f32(g).copy()
+    mask = np.ascontiguousarray(mask, np.uint8)
+    lib().orc_relu_backward(_p(g), _p(mask), C.c_int64(g.size))
+    return g
+
+
+def dropout_forward(x, keep, p):
+    x = _f32(x).copy()
+    keep = np.ascontiguousarray(keep, np.uint8)
+    lib().orc_dropout_forward(_p(x), _p(keep), C.c_int64(x.size), C.c_float(p))
+    return x
+
+
+def dropout_backward(g, keep, p):
+    g = _f32(g).copy()
+    keep = np.ascontiguousarray(keep, np.uint8)
+    lib().orc_dropout_backward(_p(g), _p(keep), C.c_int64(g.size), C.c_float(p))
+    return g
+
+
+def cross_entropy(logits, truth, training=True):
+    logits, truth = _f32(logits), _i32(truth)
+    n, c = logits.shape
+    grad = np.empty((n, c), np.float32) if training else None
+    cnt = C.c_int(0)
+    loss = lib().orc_cross_entropy(C.c_int(n), C.c_int(c), _p(logits), C.c_int(c), _p(truth), _p(grad),
+                                   C.c_int(c), C.byref(cnt))
+    return loss, grad, cnt.value
+
+
+def accuracy(logits, truth):
+    logits, truth = _f32(logits), _i32(truth)
+    n, c = logits.shape
+    return lib().orc_accuracy(C.c_int(n), C.c_int(c), _p(logits), C.c_int(c), _p(truth))
+
+
+def argmax(logits):
+    logits = _f32(logits)
+    n, c = logits.shape
+    out = np.empty(n, np.int32)
+    lib().orc_argmax(C.c_int(n), C.c_int(c), _p(logits), C.c_int(c), _p(out))
+    return out
+
+
+def adam_step(w, g, m, v, decay, weight_decay, lr, beta1, beta2, eps, step_count):
+    """In place on w, m, v (float32 arrays)."""
+    lib().orc_adam_step(_p(w), _p(_f32(g)), _p(m), _p(v), C.c_int64(w.size), C.c_int(int(decay)),
+                        C.c_float(weight_decay), C.c_float(lr), C.c_float(beta1), C.c_float(beta2),
+                        C.c_float(eps), C.c_int(step_count))
+
+
+def sgd_step(w, g, lr):
+    lib().orc_sgd_step(_p(w), _p(_f32(g)), C.c_int64(w.size), C.c_float(lr))
+
+
+def gcn_forward_backward(rp, ci, v, rpT, ciT, vT, X, W1, W2, truth, keep1=None, p_drop=0.5):
+    """Returns dict(loss, Z, H1, dW1, dW2, dT1)."""
+    rp, ci, v = _i32(rp), _i32(ci), _f32(v)
+    rpT, ciT, vT = _i32(rpT), _i32(ciT), _f32(vT)
+    X, W1, W2, truth = _f32(X), _f32(W1), _f32(W2), _i32(truth)
+    n, in_dim = X.shape
+    hidden, classes = W1.shape[1], W2.shape[1]
+    keep1 = None if keep1 is None else np.ascontiguousarray(keep1, np.uint8)
+    Z = np.empty((n, classes), np.float32)
+    H1 = np.empty((n, hidden), np.float32)
+    dW1 = np.empty((in_dim, hidden), np.float32)
+    dW2 = np.empty((hidden, classes), np.float32)
+    dT1 = np.empty((n, hidden), np.float32)
+    loss = lib().orc_gcn_forward_backward(
+        C.c_int(n), C.c_int(in_dim), C.c_int(hidden), C.c_int(classes), _p(rp), _p(ci), _p(v), _p(rpT),
+        _p(ciT), _p(vT), _p(X), _p(W1), _p(W2), _p(truth), _p(keep1), C.c_float(p_drop), _p(Z), _p(H1),
+        _p(dW1), _p(dW2), _p(dT1))
+    return dict(loss=loss, Z=Z, H1=H1, dW1=dW1, dW2=dW2, dT1=dT1)
