@@ -1,0 +1,116 @@
+"""ctypes loader for csrc/libdrone_hip.so.  Fails loudly when the library is missing."""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "csrc", "libdrone_hip.so")
+
+
+class DroneError(RuntimeError):
+    pass
+
+
+def library_path():
+    return _SO
+
+
+class Response(C.Structure):
+    """DRONE/src/cuda/algorithm/common.h:23-27"""
+    _fields_ = [("Mirror2MasterSendSize", C.c_int), ("Mirror2MasterRecvSize", C.c_int),
+                ("Master2MirrorSendSize", C.c_int), ("Master2MirrorRecvSize", C.c_int),
+                ("VisitedSize", C.c_int), ("LocalVertexSize", C.c_int),
+                ("CalTime", C.c_float), ("SendTime", C.c_float)]
+
+    def IsEmpty(self):
+        """DRONE/src/tools/cuda_convert.go:47-52"""
+        return (self.Mirror2MasterSendSize == 0 and self.Mirror2MasterRecvSize == 0 and
+                self.Master2MirrorSendSize == 0 and self.Master2MirrorRecvSize == 0)
+
+
+class Graph(C.Structure):
+    """DRONE/src/cuda/graph.h:16-38 (+ ext)"""
+    _fields_ = [("Global2Local", C.c_void_p), ("Local2Global", C.c_void_p),
+                ("MasterWorkerIndex", C.c_void_p), ("Master2Workers", C.c_void_p),
+                ("MasterSize", C.c_int), ("MirrorWorkerSize", C.c_int),
+                ("Mirror2Worker", C.c_void_p), ("MirrorSize", C.c_int),
+                ("index", C.c_void_p), ("dst", C.c_void_p), ("edgeLen", C.c_void_p),
+                ("localVertexSize", C.POINTER(C.c_int)), ("globalVertexSize", C.POINTER(C.c_int)),
+                ("edgeSize", C.POINTER(C.c_int)),
+                ("gridSize", C.c_int), ("blockSize", C.c_int),
+                ("active", C.c_void_p), ("updateByMessage", C.c_void_p),
+                ("GID", C.c_int), ("ext", C.c_void_p)]
+
+
+class Comm(C.Structure):
+    """DRONE/src/cuda/graph.h:40-43"""
+    _fields_ = [("comm", C.c_void_p), ("s", C.c_void_p)]
+
+
+class PRValues(C.Structure):
+    """DRONE/src/cuda/algorithm/pr.h:7-16 (+ ext)"""
+    _fields_ = [("sendID", C.c_void_p), ("recvID", C.c_void_p),
+                ("sendDiff", C.c_void_p), ("recvDiff", C.c_void_p),
+                ("prValue", C.c_void_p), ("accValue", C.c_void_p), ("diffValue", C.c_void_p),
+                ("globalAcc", C.c_void_p), ("globalDiff", C.c_void_p),
+                ("outDegree", C.c_void_p), ("ext", C.c_void_p)]
+
+
+_lib = None
+
+_I, _I64, _U64, _D, _F, _P = C.c_int, C.c_int64, C.c_uint64, C.c_double, C.c_float, C.c_void_p
+
+# name -> (restype, argtypes); every symbol include/drone_hip.h declares
+SIGNATURES = {
+    "drone_last_error": (_I, []),
+    "drone_last_error_string": (C.c_char_p, []),
+    "drone_version": (C.c_char_p, []),
+    "build_graph": (C.POINTER(Graph), [_I, _I, _P, _P, _I, _I, C.POINTER(Comm)]),
+    "getLocalVertexSize": (_I, [C.POINTER(Graph)]),
+    "getGlobalVertexSize": (_I, [C.POINTER(Graph)]),
+    "addMasterRoute": (None, [C.POINTER(Graph), _P, _P, _P, _I, _I]),
+    "addMirrorRoute": (None, [C.POINTER(Graph), _P, _P, _I]),
+    "loadOutDegree": (None, [C.POINTER(Graph), C.POINTER(PRValues), _P]),
+    "PR_PEVal": (Response, [C.POINTER(Graph), C.POINTER(PRValues), _I, _I, C.POINTER(Comm)]),
+    "PR_IncEVal": (Response, [C.POINTER(Graph), C.POINTER(PRValues), _I, _I, C.POINTER(Comm)]),
+    "drone_graph_destroy": (None, [C.POINTER(Graph)]),
+    "drone_pr_values_destroy": (None, [C.POINTER(Graph), C.POINTER(PRValues)]),
+    "drone_pr_plan_create": (_I, [C.POINTER(_P), _I64, _I64, _P, _P, _P, _P]),
+    "drone_pr_plan_destroy": (_I, [_P]),
+    "drone_pr_run_f64": (_I, [_P, _D, _I, _P, _P]),
+    "drone_pr_profile_enable": (_I, [_P, _I]),
+    "drone_pr_profile_read": (_I, [_P, C.POINTER(_I), C.POINTER(_D), C.POINTER(_D), C.POINTER(_D)]),
+    "drone_pr_bytes_per_iteration": (_I64, [_I64, _I64]),
+    "drone_pr_run_graph_f64": (_I, [C.POINTER(Graph), C.POINTER(PRValues), _D, _I, _P]),
+    "drone_rmat_edges": (_I, [_I, _I64, _D, _D, _D, _U64, _I64, _P, _P]),
+    "drone_fill_uniform_f32": (_I, [_P, _I64, _U64, _F, _F]),
+    "drone_fill_normal_f32": (_I, [_P, _I64, _U64]),
+    "drone_fill_randint_i32": (_I, [_P, _I64, _U64, C.c_int32]),
+    "drone_timer_create": (_I, [C.POINTER(_P)]),
+    "drone_timer_start": (_I, [_P, _P]),
+    "drone_timer_stop": (_I, [_P, _P]),
+    "drone_timer_elapsed_ms": (_I, [_P, C.POINTER(_F)]),
+    "drone_timer_destroy": (_I, [_P]),
+    "drone_device_synchronize": (_I, []),
+}
+
+
+def lib():
+    """The loaded library with typed entry points.  Raises DroneError when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            raise DroneError(
+                f"{_SO} is missing: build it with `make -C drone_amd/csrc` (or __graft_entry__.build()). "
+                "There is no CPU fallback.")
+        handle = C.CDLL(_SO)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise DroneError(f"libdrone_hip error {rc}: {lib().drone_last_error_string().decode()}")

@@ -1,0 +1,230 @@
+// fp64 pull PageRank over an in-edge CSR (int64 row_ptr, int32 col_idx) on gfx950.
+//
+// Iteration k (normalised form of DRONE/src/cuda/algorithm/pr.cu:51-87 with eps = 0):
+//   r_k[v] = (1-a)/N + a * ( sum_{u->v} c_{k-1}[u] + d_{k-1}/N ),   c[u] = r[u]*inv_outdeg[u],
+//   d = sum of r over vertices with inv_outdeg == 0.
+// The aggregation kernel gathers c_{k-1}, and its row epilogue writes c_k (and r_k on the last
+// iteration) and accumulates d_k, so one iteration touches: row_ptr 8N, col_idx 4E, gather source 8N,
+// inv_outdeg 8N, c_k 8N  =  4E + 32N bytes.
+#include "relabel.h"
+#include "spmv_merge.h"
+
+namespace drone {
+
+constexpr int kPrIpt = 8;  // items per lane; tile = 2048 merge items, 24.6 KB of LDS
+
+struct PrF64Epi {
+    const double *__restrict__ c_in;   // gather source
+    const double *__restrict__ inv;    // inverse out-degree, 0 for dangling
+    double *__restrict__ c_out;        // next gather source
+    double *__restrict__ r_out;        // ranks in the caller's vertex order, written when non-null
+    const int32_t *__restrict__ order; // internal id -> caller's id
+    const double *__restrict__ dang;   // device scalar: dangling mass of the previous ranks
+    double alpha, inv_n;
+
+    __device__ __forceinline__ double load(int c) const { return c_in[c]; }
+    __device__ __forceinline__ void row(int r, double s, double &stat) const
+    {
+        const double base = (1.0 - alpha) * inv_n + alpha * dang[0] * inv_n;
+        const double rn = base + alpha * s;
+        const double iv = inv[r];
+        c_out[r] = rn * iv;
+        if (r_out) r_out[order[r]] = rn;
+        if (iv == 0.0) stat += rn;
+    }
+    __device__ __forceinline__ void fix(int r, double carry, double &stat) const
+    {
+        const double add = alpha * carry;
+        const double iv = inv[r];
+        c_out[r] += add * iv;
+        if (r_out) r_out[order[r]] += add;
+        if (iv == 0.0) stat += add;
+    }
+};
+
+// c_0 = inv_outdeg / N ; partial count of dangling vertices per block.
+__global__ __launch_bounds__(kSpmvBlock) void pr_f64_init_kernel(int64_t n, const double *__restrict__ inv,
+                                                                 double inv_n, double *__restrict__ c0,
+                                                                 double *__restrict__ block_stat)
+{
+    __shared__ double s_red[kSpmvBlock / kWave];
+    double stat = 0.0;
+    for (int64_t i = (int64_t)blockIdx.x * kSpmvBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kSpmvBlock) {
+        const double iv = inv[i];
+        c0[i] = iv * inv_n;
+        if (iv == 0.0) stat += inv_n;
+    }
+    const double total = block_sum_256(stat, s_red);
+    if (threadIdx.x == 0) block_stat[blockIdx.x] = total;
+}
+
+__global__ void pr_f64_uniform_kernel(int64_t n, double inv_n, double *__restrict__ r)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        r[i] = inv_n;
+}
+
+}  // namespace drone
+
+using namespace drone;
+
+struct drone_pr_plan {
+    int device = 0;
+    int64_t n = 0, nnz = 0;
+    const double *inv_user = nullptr;  // caller's inverse out-degree, caller's vertex order
+    Relabel rl;                        // hot-first copy of the CSR; all work vectors use its id space
+    double *inv = nullptr;             // inverse out-degree in internal order
+    MergeTiling mt;
+    MergeScratch ms;
+    double *c[2] = {nullptr, nullptr};
+    double *dang = nullptr;  // device scalar
+    int init_blocks = 0;
+    // profiling
+    int prof_cap = 0, prof_n = 0;
+    hipEvent_t *ev0 = nullptr, *ev1 = nullptr;
+};
+
+extern "C" int64_t drone_pr_bytes_per_iteration(int64_t n, int64_t nnz) { return 4 * nnz + 32 * n + 8; }
+
+extern "C" int drone_pr_plan_create(drone_pr_plan **out, int64_t n, int64_t nnz, const int64_t *row_ptr,
+                                    const int32_t *col_idx, const double *inv_outdeg, drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(out != nullptr, "plan pointer");
+    DRONE_REQUIRE(n > 0 && n < INT32_MAX, "vertex count must be in [1, 2^31-2]");
+    DRONE_REQUIRE(nnz >= 0, "nnz");
+    DRONE_REQUIRE(row_ptr && inv_outdeg && (col_idx || nnz == 0), "null CSR array");
+    drone_pr_plan *p = new drone_pr_plan();
+    DRONE_HIP_TRY(hipGetDevice(&p->device));
+    p->n = n;
+    p->nnz = nnz;
+    p->inv_user = inv_outdeg;
+    hipStream_t s = as_stream(stream);
+    int rc = relabel_create(&p->rl, n, nnz, row_ptr, col_idx, s);
+    if (rc != DRONE_OK) { delete p; return rc; }
+    rc = merge_tiling_create<int64_t>(&p->mt, n, nnz, p->rl.row_ptr, kSpmvBlock * kPrIpt, s);
+    if (rc != DRONE_OK) { drone_pr_plan_destroy(p); return rc; }
+    rc = merge_scratch_create(&p->ms, p->mt, sizeof(double));
+    if (rc != DRONE_OK) { drone_pr_plan_destroy(p); return rc; }
+    DRONE_HIP_TRY(hipMalloc(&p->c[0], sizeof(double) * (size_t)n));
+    DRONE_HIP_TRY(hipMalloc(&p->c[1], sizeof(double) * (size_t)n));
+    DRONE_HIP_TRY(hipMalloc(&p->dang, sizeof(double)));
+    DRONE_HIP_TRY(hipMalloc(&p->inv, sizeof(double) * (size_t)n));
+    // the init kernel parks its block partials in block_stat: never more blocks than it holds
+    int ib = (int)ceil_div(n, kSpmvBlock * 8);
+    const int fb = fixup_blocks(p->mt.num_tiles);
+    p->init_blocks = ib < fb ? ib : fb;
+    if (p->init_blocks < 1) p->init_blocks = 1;
+    DRONE_HIP_TRY(hipStreamSynchronize(s));
+    *out = p;
+    return DRONE_OK;
+}
+
+extern "C" int drone_pr_plan_destroy(drone_pr_plan *p)
+{
+    if (!p) return DRONE_OK;
+    merge_tiling_destroy(&p->mt);
+    merge_scratch_destroy(&p->ms);
+    relabel_destroy(&p->rl);
+    if (p->inv) (void)hipFree(p->inv);
+    if (p->c[0]) (void)hipFree(p->c[0]);
+    if (p->c[1]) (void)hipFree(p->c[1]);
+    if (p->dang) (void)hipFree(p->dang);
+    for (int i = 0; i < p->prof_cap; ++i) {
+        (void)hipEventDestroy(p->ev0[i]);
+        (void)hipEventDestroy(p->ev1[i]);
+    }
+    delete[] p->ev0;
+    delete[] p->ev1;
+    delete p;
+    return DRONE_OK;
+}
+
+extern "C" int drone_pr_profile_enable(drone_pr_plan *p, int max_launches)
+{
+    clear_error();
+    DRONE_REQUIRE(p != nullptr && max_launches >= 0 && max_launches <= (1 << 20), "profile size");
+    for (int i = 0; i < p->prof_cap; ++i) {
+        (void)hipEventDestroy(p->ev0[i]);
+        (void)hipEventDestroy(p->ev1[i]);
+    }
+    delete[] p->ev0;
+    delete[] p->ev1;
+    p->ev0 = p->ev1 = nullptr;
+    p->prof_cap = p->prof_n = 0;
+    if (max_launches == 0) return DRONE_OK;
+    p->ev0 = new hipEvent_t[max_launches];
+    p->ev1 = new hipEvent_t[max_launches];
+    for (int i = 0; i < max_launches; ++i) {
+        DRONE_HIP_TRY(hipEventCreate(&p->ev0[i]));
+        DRONE_HIP_TRY(hipEventCreate(&p->ev1[i]));
+        p->prof_cap = i + 1;
+    }
+    return DRONE_OK;
+}
+
+extern "C" int drone_pr_profile_read(drone_pr_plan *p, int *launches, double *mean_ms, double *min_ms,
+                                     double *max_ms)
+{
+    clear_error();
+    DRONE_REQUIRE(p != nullptr, "plan");
+    double sum = 0.0, mn = 1e300, mx = 0.0;
+    for (int i = 0; i < p->prof_n; ++i) {
+        float ms = 0.0f;
+        DRONE_HIP_TRY(hipEventSynchronize(p->ev1[i]));
+        DRONE_HIP_TRY(hipEventElapsedTime(&ms, p->ev0[i], p->ev1[i]));
+        sum += ms;
+        if (ms < mn) mn = ms;
+        if (ms > mx) mx = ms;
+    }
+    if (launches) *launches = p->prof_n;
+    if (mean_ms) *mean_ms = p->prof_n ? sum / p->prof_n : 0.0;
+    if (min_ms) *min_ms = p->prof_n ? mn : 0.0;
+    if (max_ms) *max_ms = mx;
+    p->prof_n = 0;
+    return DRONE_OK;
+}
+
+extern "C" int drone_pr_run_f64(drone_pr_plan *p, double alpha, int iters, double *rank_out,
+                                drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(p != nullptr && rank_out != nullptr, "null argument");
+    DRONE_REQUIRE(iters >= 0, "iteration count");
+    DRONE_REQUIRE(alpha >= 0.0 && alpha <= 1.0, "alpha must be in [0,1]");
+    hipStream_t s = as_stream(stream);
+    const double inv_n = 1.0 / (double)p->n;
+    if (iters == 0) {
+        pr_f64_uniform_kernel<<<1024, 256, 0, s>>>(p->n, inv_n, rank_out);
+        DRONE_HIP_TRY(hipGetLastError());
+        return DRONE_OK;
+    }
+    // the caller may have refreshed inv_outdeg since the plan was made: re-read it every run (8N bytes)
+    { int rc = relabel_gather_f64(p->rl, p->inv_user, p->inv, s); if (rc != DRONE_OK) return rc; }
+    pr_f64_init_kernel<<<p->init_blocks, kSpmvBlock, 0, s>>>(p->n, p->inv, inv_n, p->c[0], p->ms.block_stat);
+    reduce_stat_kernel<0><<<1, kSpmvBlock, 0, s>>>(p->ms.block_stat, p->init_blocks, p->dang);
+    for (int it = 0; it < iters; ++it) {
+        PrF64Epi epi;
+        epi.c_in = p->c[it & 1];
+        epi.c_out = p->c[(it + 1) & 1];
+        epi.inv = p->inv;
+        epi.r_out = (it == iters - 1) ? rank_out : nullptr;
+        epi.dang = p->dang;
+        epi.order = p->rl.order;
+        epi.alpha = alpha;
+        epi.inv_n = inv_n;
+        const bool prof = p->prof_n < p->prof_cap;
+        double *carry = static_cast<double *>(p->ms.tile_carry);
+        if (prof) DRONE_HIP_TRY(hipEventRecord(p->ev0[p->prof_n], s));
+        spmv_merge_kernel<double, int64_t, kPrIpt, PrF64Epi><<<p->mt.num_tiles, kSpmvBlock, 0, s>>>(
+            p->n, p->nnz, p->mt.tile_row, p->rl.row_ptr, p->rl.col, epi, carry, p->ms.tile_stat);
+        if (prof) DRONE_HIP_TRY(hipEventRecord(p->ev1[p->prof_n++], s));
+        const int fb = fixup_blocks(p->mt.num_tiles);
+        spmv_fixup_kernel<double, PrF64Epi><<<fb, kSpmvBlock, 0, s>>>(
+            p->mt.num_tiles, p->mt.tile_row, p->mt.walk_len, carry, p->ms.tile_stat, epi, p->ms.block_stat);
+        // dang is read by the kernels above and overwritten here, in stream order
+        reduce_stat_kernel<0><<<1, kSpmvBlock, 0, s>>>(p->ms.block_stat, fb, p->dang);
+    }
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}

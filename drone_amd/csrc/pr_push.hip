@@ -1,0 +1,324 @@
+// PR_PEVal / PR_IncEVal / loadOutDegree with the reference's float delta-push semantics
+// (DRONE/src/cuda/algorithm/pr.cu:14-37, 51-87, 430-448, 490-515), computed without atomics:
+// a vertex kernel decides what every vertex pushes this superstep (push[u] = delta/outdeg, or 0 when
+// the change is below eps), and the merge-path aggregation pulls diff[v] = sum of push[u] over the
+// in-edges of v together with the number of non-zero pushes, which gives g->active and VisitedSize.
+#include <chrono>
+
+#include "graph_ext.h"
+
+using namespace drone;
+
+namespace {
+
+constexpr float kEps = 1e-6f;    // pr.cu:11
+constexpr float kAlpha = 0.85f;  // pr.cu:12
+constexpr int kPushIpt = 8;
+
+struct PushEpi {
+    const float *__restrict__ push;
+    float *__restrict__ diff;
+    int *__restrict__ active;
+
+    __device__ __forceinline__ PushF2 load(int c) const
+    {
+        const float v = push[c];
+        return PushF2{v, v != 0.0f ? 1.0f : 0.0f};
+    }
+    __device__ __forceinline__ void row(int r, PushF2 s, double &stat) const
+    {
+        diff[r] = s.s;
+        const int a = s.c != 0.0f;
+        active[r] = a;
+        stat += a;
+    }
+    __device__ __forceinline__ void fix(int r, PushF2 carry, double &stat) const
+    {
+        diff[r] += carry.s;
+        if (carry.c != 0.0f && active[r] == 0) {
+            active[r] = 1;
+            stat += 1.0;
+        }
+    }
+};
+
+// pr.cu:490-500
+__global__ void set_out_degree_kernel(int *local_out, const int *global_out, const int *l2g, int n)
+{
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
+        local_out[i] = global_out[l2g[i]];
+}
+
+// pr.cu:14-37 without the edge loop: pr = 1, acc = 0, push = 1/outdeg; dangling masters add
+// 1/Nglobal to the global diff (block partials, summed in a fixed order afterwards).
+__global__ __launch_bounds__(kSpmvBlock) void pr_init_vertex_kernel(
+    int n, int nglobal, const int *__restrict__ outdeg, const int *__restrict__ m2w, float *__restrict__ pr,
+    float *__restrict__ acc, float *__restrict__ push, int *__restrict__ update_by_message,
+    double *__restrict__ block_part)
+{
+    __shared__ double s_red[kSpmvBlock / kWave];
+    double part = 0.0;
+    for (int id = blockIdx.x * kSpmvBlock + threadIdx.x; id < n; id += gridDim.x * kSpmvBlock) {
+        acc[id] = 0.0f;
+        pr[id] = 1.0f;
+        update_by_message[id] = 0;
+        const int od = outdeg[id];
+        float p = 0.0f;
+        if (od == 0) {
+            if (m2w[id] == -1) part += (double)(1.0f / (float)nglobal);
+        } else {
+            p = 1.0f / (float)od;
+        }
+        push[id] = p;
+    }
+    const double total = block_sum_256(part, s_red);
+    if (threadIdx.x == 0) block_part[blockIdx.x] = total;
+}
+
+// pr.cu:430-448 (thread 0): globalAcc += globalDiff; globalDiff = 0
+__global__ void pr_fold_global_kernel(float *global_acc, float *global_diff)
+{
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        *global_acc += *global_diff;
+        *global_diff = 0.0f;
+    }
+}
+
+// pr.cu:430-448 (per vertex) fused with pr.cu:51-87 without the edge loop.
+__global__ __launch_bounds__(kSpmvBlock) void pr_increment_vertex_kernel(
+    int n, int nglobal, const int *__restrict__ outdeg, const int *__restrict__ m2w, float *__restrict__ pr,
+    float *__restrict__ acc, const float *__restrict__ diff, const float *__restrict__ global_acc,
+    float *__restrict__ push, int *__restrict__ update_by_message, double *__restrict__ block_part)
+{
+    __shared__ double s_red[kSpmvBlock / kWave];
+    const float ga = *global_acc;
+    double part = 0.0;
+    for (int id = blockIdx.x * kSpmvBlock + threadIdx.x; id < n; id += gridDim.x * kSpmvBlock) {
+        update_by_message[id] = 0;
+        const float a = acc[id] + diff[id];
+        acc[id] = a;
+        const float old = pr[id];
+        const float p = kAlpha * (a + ga) + (1 - kAlpha);
+        float d = p - old;
+        if (d < 0) d = -d;
+        float out = 0.0f;
+        if (!(d < kEps)) {
+            const int od = outdeg[id];
+            if (od == 0) {
+                if (m2w[id] == -1) part += (double)((p - old) / (float)nglobal);
+            } else {
+                out = (p - old) / (float)od;
+            }
+            pr[id] = p;
+        }
+        push[id] = out;
+    }
+    const double total = block_sum_256(part, s_red);
+    if (threadIdx.x == 0) block_part[blockIdx.x] = total;
+}
+
+// globalDiff += (float) sum of block partials, fixed order
+__global__ __launch_bounds__(kSpmvBlock) void pr_add_global_diff_kernel(const double *__restrict__ part, int count,
+                                                                        float *__restrict__ global_diff)
+{
+    __shared__ double s_red[kSpmvBlock / kWave];
+    double v = 0.0;
+    for (int k = threadIdx.x; k < count; k += kSpmvBlock) v += part[k];
+    const double total = block_sum_256(v, s_red);
+    if (threadIdx.x == 0) *global_diff += (float)total;
+}
+
+double seconds_since(std::chrono::steady_clock::time_point t0)
+{
+    return std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+}
+
+void ensure_push_ready(Graph *g)
+{
+    GraphExt *x = static_cast<GraphExt *>(g->ext);
+    if (x->push_ready) return;
+    if (merge_tiling_create<int>(&x->mt, x->n, x->edges, x->in_index, kSpmvBlock * kPushIpt, nullptr) != DRONE_OK ||
+        merge_scratch_create(&x->ms, x->mt, sizeof(PushF2)) != DRONE_OK) {
+        printf("Failed: %s\n", drone_last_error_string());
+        exit(EXIT_FAILURE);
+    }
+    x->push_ready = true;
+}
+
+int aggregate_push(Graph *g, PRValues *values, hipStream_t s)
+{
+    GraphExt *x = static_cast<GraphExt *>(g->ext);
+    PRExt *px = static_cast<PRExt *>(values->ext);
+    PushEpi epi{px->push, values->diffValue, g->active};
+    spmv_merge_launch<PushF2, int, kPushIpt, PushEpi>(x->mt, x->ms, x->in_index, x->in_src, epi, px->stat, s);
+    DRONE_HIP_OR_DIE(hipGetLastError());
+    double visited = 0.0;
+    DRONE_HIP_OR_DIE(hipMemcpyAsync(&visited, px->stat, sizeof(double), hipMemcpyDeviceToHost, s));
+    DRONE_HIP_OR_DIE(hipStreamSynchronize(s));
+    return (int)visited;
+}
+
+}  // namespace
+
+void drone::graph_ext_release(GraphExt *x)
+{
+    if (x->in_index) (void)hipFree(x->in_index);
+    if (x->in_src) (void)hipFree(x->in_src);
+    merge_tiling_destroy(&x->mt);
+    merge_scratch_destroy(&x->ms);
+    if (x->plan64) (void)drone_pr_plan_destroy(x->plan64);
+    if (x->row_ptr64) (void)hipFree(x->row_ptr64);
+    if (x->inv64) (void)hipFree(x->inv64);
+    if (x->rank64) (void)hipFree(x->rank64);
+    *x = GraphExt{};
+}
+
+extern "C" void loadOutDegree(Graph *g, PRValues *values, int *globalOutDegree)
+{
+    clear_error();
+    DRONE_HIP_OR_DIE(hipSetDevice(g->GID));
+    const int nglobal = *g->globalVertexSize, n = *g->localVertexSize;
+    DRONE_HIP_OR_DIE(hipMalloc(&values->outDegree, sizeof(int) * (size_t)(n ? n : 1)));
+    int *d_global = nullptr;
+    DRONE_HIP_OR_DIE(hipMalloc(&d_global, sizeof(int) * (size_t)(nglobal ? nglobal : 1)));
+    DRONE_HIP_OR_DIE(hipMemcpy(d_global, globalOutDegree, sizeof(int) * (size_t)nglobal, hipMemcpyHostToDevice));
+    set_out_degree_kernel<<<1024, 256>>>(values->outDegree, d_global, g->Local2Global, n);
+    DRONE_HIP_OR_DIE(hipDeviceSynchronize());
+    (void)hipFree(d_global);
+}
+
+extern "C" Response PR_PEVal(Graph *g, PRValues *values, int workerId, int workerNum, Comm *comm)
+{
+    (void)workerId; (void)workerNum;
+    clear_error();
+    const auto t0 = std::chrono::steady_clock::now();
+    DRONE_HIP_OR_DIE(hipSetDevice(g->GID));
+    hipStream_t s = comm ? static_cast<hipStream_t>(comm->s) : nullptr;
+    Response res = {};
+    const int n = getLocalVertexSize(g), nglobal = getGlobalVertexSize(g);
+    const size_t cnt = (size_t)(n ? n : 1);
+    if (values->outDegree == nullptr) {
+        set_error(DRONE_ERR_INVALID, "PR_PEVal: loadOutDegree has not been called");
+        printf("Failed: PR_PEVal before loadOutDegree\n");
+        exit(EXIT_FAILURE);
+    }
+    ensure_push_ready(g);
+    // pr.cu:383-389: the state vectors are allocated by this call
+    if (!g->active) DRONE_HIP_OR_DIE(hipMalloc(&g->active, sizeof(int) * cnt));
+    if (!g->updateByMessage) DRONE_HIP_OR_DIE(hipMalloc(&g->updateByMessage, sizeof(int) * cnt));
+    if (!values->ext) {
+        DRONE_HIP_OR_DIE(hipMalloc(&values->prValue, sizeof(float) * cnt));
+        DRONE_HIP_OR_DIE(hipMalloc(&values->accValue, sizeof(float) * cnt));
+        DRONE_HIP_OR_DIE(hipMalloc(&values->diffValue, sizeof(float) * cnt));
+        DRONE_HIP_OR_DIE(hipMalloc(&values->globalDiff, sizeof(float)));
+        DRONE_HIP_OR_DIE(hipMalloc(&values->globalAcc, sizeof(float)));
+        PRExt *px = new PRExt();
+        DRONE_HIP_OR_DIE(hipMalloc(&px->push, sizeof(float) * cnt));
+        DRONE_HIP_OR_DIE(hipMalloc(&px->stat, sizeof(double)));
+        px->vertex_blocks = (int)ceil_div(cnt, kSpmvBlock * 4);
+        if (px->vertex_blocks > 4096) px->vertex_blocks = 4096;
+        DRONE_HIP_OR_DIE(hipMalloc(&px->block_part, sizeof(double) * (size_t)px->vertex_blocks));
+        values->ext = px;
+        // exchange staging (pr.cu:402-405) has no use with one subgraph: left null
+    }
+    PRExt *px = static_cast<PRExt *>(values->ext);
+    DRONE_HIP_OR_DIE(hipMemsetAsync(values->globalDiff, 0, sizeof(float), s));
+    DRONE_HIP_OR_DIE(hipMemsetAsync(values->globalAcc, 0, sizeof(float), s));
+    pr_init_vertex_kernel<<<px->vertex_blocks, kSpmvBlock, 0, s>>>(n, nglobal, values->outDegree, g->Mirror2Worker,
+                                                                  values->prValue, values->accValue, px->push,
+                                                                  g->updateByMessage, px->block_part);
+    pr_add_global_diff_kernel<<<1, kSpmvBlock, 0, s>>>(px->block_part, px->vertex_blocks, values->globalDiff);
+    res.VisitedSize = aggregate_push(g, values, s);
+    res.LocalVertexSize = n;
+    res.CalTime = (float)seconds_since(t0);
+    res.SendTime = 0.0f;  // one subgraph: nothing to exchange (pr.cu:415-421 moves zero elements)
+    return res;
+}
+
+extern "C" Response PR_IncEVal(Graph *g, PRValues *values, int workerId, int workerNum, Comm *comm)
+{
+    (void)workerId; (void)workerNum;
+    clear_error();
+    const auto t0 = std::chrono::steady_clock::now();
+    DRONE_HIP_OR_DIE(hipSetDevice(g->GID));
+    hipStream_t s = comm ? static_cast<hipStream_t>(comm->s) : nullptr;
+    Response res = {};
+    if (!values->ext) {
+        set_error(DRONE_ERR_INVALID, "PR_IncEVal: PR_PEVal has not been called");
+        printf("Failed: PR_IncEVal before PR_PEVal\n");
+        exit(EXIT_FAILURE);
+    }
+    PRExt *px = static_cast<PRExt *>(values->ext);
+    const int n = getLocalVertexSize(g), nglobal = getGlobalVertexSize(g);
+    pr_fold_global_kernel<<<1, 64, 0, s>>>(values->globalAcc, values->globalDiff);
+    pr_increment_vertex_kernel<<<px->vertex_blocks, kSpmvBlock, 0, s>>>(
+        n, nglobal, values->outDegree, g->Mirror2Worker, values->prValue, values->accValue, values->diffValue,
+        values->globalAcc, px->push, g->updateByMessage, px->block_part);
+    pr_add_global_diff_kernel<<<1, kSpmvBlock, 0, s>>>(px->block_part, px->vertex_blocks, values->globalDiff);
+    res.VisitedSize = aggregate_push(g, values, s);
+    res.LocalVertexSize = n;
+    res.CalTime = (float)seconds_since(t0);
+    res.SendTime = 0.0f;
+    return res;
+}
+
+extern "C" void drone_pr_values_destroy(Graph *g, PRValues *values)
+{
+    if (!values) return;
+    if (g) (void)hipSetDevice(g->GID);
+    PRExt *px = static_cast<PRExt *>(values->ext);
+    if (px) {
+        (void)hipFree(px->push);
+        (void)hipFree(px->stat);
+        (void)hipFree(px->block_part);
+        delete px;
+    }
+    if (values->prValue) (void)hipFree(values->prValue);
+    if (values->accValue) (void)hipFree(values->accValue);
+    if (values->diffValue) (void)hipFree(values->diffValue);
+    if (values->globalAcc) (void)hipFree(values->globalAcc);
+    if (values->globalDiff) (void)hipFree(values->globalDiff);
+    if (values->outDegree) (void)hipFree(values->outDegree);
+    *values = PRValues{};
+}
+
+// ---- fp64 pull run driven from the Graph ----------------------------------------------------------
+namespace {
+
+__global__ void widen_row_ptr_kernel(const int *in, int64_t *out, int count)
+{
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < count; i += gridDim.x * blockDim.x) out[i] = in[i];
+}
+
+__global__ void inverse_out_degree_kernel(const int *outdeg, double *inv, int n)
+{
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+        const int d = outdeg[i];
+        inv[i] = d > 0 ? 1.0 / (double)d : 0.0;
+    }
+}
+
+}  // namespace
+
+extern "C" int drone_pr_run_graph_f64(Graph *g, PRValues *values, double alpha, int iters, double *rank_out)
+{
+    clear_error();
+    DRONE_REQUIRE(g && g->ext && values && rank_out, "null argument");
+    DRONE_REQUIRE(values->outDegree != nullptr, "loadOutDegree has not been called");
+    DRONE_HIP_TRY(hipSetDevice(g->GID));
+    GraphExt *x = static_cast<GraphExt *>(g->ext);
+    DRONE_REQUIRE(x->n > 0, "empty graph");
+    if (!x->plan64) {
+        DRONE_HIP_TRY(hipMalloc(&x->row_ptr64, sizeof(int64_t) * ((size_t)x->n + 1)));
+        DRONE_HIP_TRY(hipMalloc(&x->inv64, sizeof(double) * (size_t)x->n));
+        DRONE_HIP_TRY(hipMalloc(&x->rank64, sizeof(double) * (size_t)x->n));
+        widen_row_ptr_kernel<<<1024, 256>>>(x->in_index, x->row_ptr64, x->n + 1);
+        int rc = drone_pr_plan_create(&x->plan64, x->n, x->edges, x->row_ptr64, x->in_src, x->inv64, nullptr);
+        if (rc != DRONE_OK) return rc;
+    }
+    inverse_out_degree_kernel<<<1024, 256>>>(values->outDegree, x->inv64, x->n);
+    int rc = drone_pr_run_f64(x->plan64, alpha, iters, x->rank64, nullptr);
+    if (rc != DRONE_OK) return rc;
+    DRONE_HIP_TRY(hipMemcpy(rank_out, x->rank64, sizeof(double) * (size_t)x->n, hipMemcpyDeviceToHost));
+    return DRONE_OK;
+}

@@ -1,0 +1,28 @@
+// Hot-first vertex relabelling for the pull aggregation.
+//
+// Every gather of an 8-byte value moves a whole 128-byte line from L2 (or beyond) into the CU, so the
+// cost of the gather stream is set by how many distinct lines it touches, not by its bytes.  Sorting
+// vertices by how often they are gathered (their count in col_idx, i.e. out-degree) packs the popular
+// sources into few lines that stay cache resident.  The plan keeps a relabelled copy of the CSR; rows
+// use the same id space because an iteration's output is the next iteration's gather source.
+#pragma once
+#include "common.h"
+
+namespace drone {
+
+struct Relabel {
+    int64_t n = 0, nnz = 0;
+    int32_t *order = nullptr;    // device [n]: new id -> old id
+    int64_t *row_ptr = nullptr;  // device [n+1]: relabelled CSR offsets
+    int32_t *col = nullptr;      // device [nnz]: relabelled sources, row order kept
+};
+
+// Builds the relabelled CSR from (row_ptr, col) on `stream`.  All temporaries are freed before return.
+int relabel_create(Relabel *rl, int64_t n, int64_t nnz, const int64_t *row_ptr, const int32_t *col,
+                   hipStream_t stream);
+void relabel_destroy(Relabel *rl);
+
+// out[i] = in[order[i]]
+int relabel_gather_f64(const Relabel &rl, const double *in, double *out, hipStream_t stream);
+
+}  // namespace drone

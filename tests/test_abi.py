@@ -1,0 +1,107 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every function include/drone_hip.h declares,
+the Python mirror binds each of them, struct layouts match the reference's, and host-only entry points
+(generators, argument validation) behave.  No GPU work happens here."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from drone_amd import _lib, rmat
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "drone_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"typedef struct \w+ \{.*?\} \w+;", "", text, flags=re.S)
+    text = re.sub(r"enum \w+ \{.*?\};", "", text, flags=re.S)
+    names = re.findall(r"\b([A-Za-z_]\w*)\s*\([^;{]*\)\s*;", text)
+    return sorted(set(names))
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_functions()
+    assert "build_graph" in names and "PR_IncEVal" in names and "drone_pr_run_f64" in names
+    handle = C.CDLL(_lib.library_path())
+    missing = [n for n in names if not hasattr(handle, n)]
+    assert not missing, f"declared in drone_hip.h but not exported: {missing}"
+
+
+def test_python_mirror_binds_every_declared_symbol():
+    assert sorted(_lib.SIGNATURES) == declared_functions()
+    _lib.lib()
+
+
+def test_struct_layouts_match_reference():
+    # common.h:23-27: 6 int + 2 float, returned by value over cgo
+    assert C.sizeof(_lib.Response) == 32
+    assert _lib.Response.VisitedSize.offset == 16 and _lib.Response.CalTime.offset == 24
+    # graph.h:40-43: two pointers
+    assert C.sizeof(_lib.Comm) == 16
+    # graph.h:16-38 field offsets on LP64 (ext appended after GID)
+    g = _lib.Graph
+    assert (g.Global2Local.offset, g.Local2Global.offset, g.MasterWorkerIndex.offset, g.Master2Workers.offset) == (0, 8, 16, 24)
+    assert (g.MasterSize.offset, g.MirrorWorkerSize.offset, g.Mirror2Worker.offset, g.MirrorSize.offset) == (32, 36, 40, 48)
+    assert (g.index.offset, g.dst.offset, g.edgeLen.offset) == (56, 64, 72)
+    assert (g.localVertexSize.offset, g.globalVertexSize.offset, g.edgeSize.offset) == (80, 88, 96)
+    assert (g.gridSize.offset, g.blockSize.offset, g.active.offset, g.updateByMessage.offset, g.GID.offset) == (104, 108, 112, 120, 128)
+    # pr.h:7-16: ten pointers, then ext
+    assert _lib.PRValues.outDegree.offset == 72 and _lib.PRValues.ext.offset == 80
+
+
+def test_version_and_error_channel():
+    L = _lib.lib()
+    assert b"gfx950" in L.drone_version()
+    # invalid arguments are rejected on the host before anything touches a device
+    rc = L.drone_rmat_edges(0, 10, 0.57, 0.19, 0.19, 1, 0, None, None)
+    assert rc == -1 and L.drone_last_error() == -1 and b"scale" in L.drone_last_error_string()
+    h = C.c_void_p()
+    assert L.drone_pr_plan_create(C.byref(h), 0, 0, None, None, None, None) == -1
+    assert L.drone_pr_bytes_per_iteration(10, 100) == 4 * 100 + 32 * 10 + 8
+
+
+def test_rmat_generator_is_a_pure_function_of_seed_and_index():
+    s, d = rmat.rmat_edges(10, 5000, seed=7)
+    s2, d2 = rmat.rmat_edges(10, 3000, seed=7, first_edge=2000)
+    np.testing.assert_array_equal(s[2000:], s2)
+    np.testing.assert_array_equal(d[2000:], d2)
+    s3, _ = rmat.rmat_edges(10, 5000, seed=8)
+    assert (s != s3).any()
+    assert s.max() < 1024 and d.max() < 1024
+
+
+def test_rmat_quadrant_probabilities():
+    # one level: the four quadrants appear with probabilities a, b, c, d
+    s, d = rmat.rmat_edges(1, 400000, a=0.57, b=0.19, c=0.19, seed=3)
+    q = np.bincount(s.astype(int) * 2 + d.astype(int), minlength=4) / 400000.0
+    np.testing.assert_allclose(q, [0.57, 0.19, 0.19, 0.05], atol=4e-3)
+
+
+@pytest.mark.parametrize("seed,expect", [(1, None)])
+def test_rmat_checksums_are_stable(seed, expect):
+    """Edge count and a 64-bit hash of the cleaned, sorted edge list for scale 10 with each benchmark seed:
+    the GPU box must generate exactly these graphs."""
+    import json
+    gold = json.load(open(os.path.join(ROOT, "tests", "golden", "rmat_checksums.json")))
+    for entry in gold:
+        s, d = rmat.rmat_edges(10, 1024 * entry["edge_factor"], a=entry["a"], b=entry["b"], c=entry["c"], seed=entry["seed"])
+        src, dst = rmat.clean_directed_np(s, d)
+        key = (dst.astype(np.uint64) << np.uint64(32)) | src.astype(np.uint64)
+        h = np.uint64(1469598103934665603)
+        with np.errstate(over="ignore"):
+            acc = np.bitwise_xor.reduce(key * np.uint64(1099511628211) + np.arange(len(key), dtype=np.uint64))
+        assert len(key) == entry["edges"]
+        assert int(acc ^ h) == entry["hash"]
+
+
+def test_fill_generators():
+    x = rmat.uniform_f32((1000, 7), seed=3)
+    assert x.min() >= -1 and x.max() < 1 and abs(x.mean()) < 0.05
+    y = rmat.normal_f32(200000, seed=4)
+    assert abs(y.mean()) < 0.01 and abs(y.std() - 1) < 0.01
+    z = rmat.randint_i32(100000, seed=5, bound=41)
+    assert z.min() == 0 and z.max() == 40
+    np.testing.assert_array_equal(rmat.uniform_f32(50, seed=3), x.ravel()[:50])

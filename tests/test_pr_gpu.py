@@ -1,0 +1,251 @@
+"""GPU parity of the PageRank path against the CPU oracle, through the C ABI.
+
+Tolerances: fp64 pull - per-vertex relative error <= 1e-9 after the fixed iteration count (the summation
+order differs from the oracle's, nothing else does); float delta-push - 2e-5 relative on pr (float sums in a
+different order than the oracle's serial stand-in for the reference's unordered atomics) and exact equality
+for everything integer (graph arrays, active flags, VisitedSize)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ALPHA = 0.85
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return torch
+
+
+def in_csr_np(n, src, dst):
+    src, dst = np.asarray(src, np.int64), np.asarray(dst, np.int64)
+    order = np.lexsort((src, dst))
+    s, d = src[order], dst[order]
+    rp = np.zeros(n + 1, np.int64)
+    rp[1:] = np.cumsum(np.bincount(d, minlength=n))
+    outdeg = np.bincount(src, minlength=n)
+    inv = np.where(outdeg > 0, 1.0 / np.maximum(outdeg, 1), 0.0)
+    return rp, s.astype(np.int32), inv
+
+
+def run_plan(torch, rp, ci, inv, iters, alpha=ALPHA):
+    from drone_amd.pagerank import PullPlanF64
+    plan = PullPlanF64(torch.from_numpy(rp).cuda(), torch.from_numpy(ci).cuda(), torch.from_numpy(inv).cuda())
+    out = plan.run(alpha, iters).cpu().numpy()
+    plan.close()
+    return out
+
+
+def assert_rel(got, ref, tol):
+    rel = np.abs(got - ref) / np.abs(ref)
+    assert rel.max() <= tol, f"max relative error {rel.max():.3e} at {rel.argmax()}"
+
+
+def small_cases():
+    rng = np.random.default_rng(11)
+    cases = {}
+    n = 17
+    cases["cycle"] = (n, np.arange(n), (np.arange(n) + 1) % n)
+    cases["single_vertex"] = (1, np.zeros(0, int), np.zeros(0, int))
+    cases["all_dangling"] = (300, np.zeros(0, int), np.zeros(0, int))
+    m = 9000                                 # hub row of 9000 in-edges: spans several 2048-item tiles
+    cases["in_star_hub"] = (m + 1, np.arange(1, m + 1), np.zeros(m, int))
+    cases["out_star_dangling_leaves"] = (m + 1, np.zeros(m, int), np.arange(1, m + 1))
+    # two long rows back to back followed by thousands of empty rows, then a dense tail
+    src = np.concatenate([np.arange(10, 5010), np.arange(20, 4020), rng.integers(0, 20000, 30000)])
+    dst = np.concatenate([np.full(5000, 3), np.full(4000, 4), rng.integers(15000, 20000, 30000)])
+    keep = src != dst
+    pairs = np.unique(np.stack([src[keep], dst[keep]], 1), axis=0)
+    cases["ragged"] = (20000, pairs[:, 0], pairs[:, 1])
+    # exactly one tile of items (n + nnz = 2048) and one more than a tile
+    for name, tot in (("one_tile_exact", 2048), ("one_tile_plus_one", 2049)):
+        nn = 512
+        e = tot - nn
+        s = rng.integers(0, nn, 4 * e)
+        d = rng.integers(0, nn, 4 * e)
+        k = s != d
+        pr = np.unique(np.stack([s[k], d[k]], 1), axis=0)
+        pr = pr[rng.permutation(len(pr))[:e]]
+        assert len(pr) == e
+        cases[name] = (nn, pr[:, 0], pr[:, 1])
+    return cases
+
+
+@pytest.mark.parametrize("name", list(small_cases()))
+@pytest.mark.parametrize("iters", [0, 1, 2, 20])
+def test_pull_f64_edge_cases(torch_cuda, oracle, name, iters):
+    n, src, dst = small_cases()[name]
+    rp, ci, inv = in_csr_np(n, src, dst)
+    got = run_plan(torch_cuda, rp, ci, inv, iters)
+    ref = oracle.pr_pull_f64(rp, ci, inv, ALPHA, iters)
+    assert_rel(got, ref, 1e-9)
+    assert abs(got.sum() - 1.0) < 1e-11
+
+
+@pytest.mark.parametrize("scale,ef,seed,iters", [(10, 16, 1, 20), (14, 16, 2, 50), (16, 16, 1, 20), (18, 8, 5, 10)])
+def test_pull_f64_rmat(torch_cuda, oracle, scale, ef, seed, iters):
+    """(16, 16, seed 1, 20 iterations) is the first benchmark configuration at full size."""
+    from drone_amd import rmat
+    x = rmat.pagerank_inputs_np(scale, ef, seed)
+    got = run_plan(torch_cuda, x["row_ptr"], x["col_idx"], x["inv_outdeg"], iters)
+    ref = oracle.pr_pull_f64(x["row_ptr"], x["col_idx"], x["inv_outdeg"], ALPHA, iters)
+    assert_rel(got, ref, 1e-9)
+    assert abs(got.sum() - 1.0) < 1e-11
+
+
+def test_pull_f64_other_alpha_and_rerun(torch_cuda, oracle):
+    from drone_amd import rmat
+    from drone_amd.pagerank import PullPlanF64
+    torch = torch_cuda
+    x = rmat.pagerank_inputs_np(12, 16, 9)
+    plan = PullPlanF64(torch.from_numpy(x["row_ptr"]).cuda(), torch.from_numpy(x["col_idx"]).cuda(),
+                       torch.from_numpy(x["inv_outdeg"]).cuda())
+    for alpha, iters in ((0.5, 7), (0.99, 3), (0.85, 7)):          # the same plan is reusable
+        got = plan.run(alpha, iters).cpu().numpy()
+        assert_rel(got, oracle.pr_pull_f64(x["row_ptr"], x["col_idx"], x["inv_outdeg"], alpha, iters), 1e-9)
+    a = plan.run(0.85, 7).cpu().numpy()
+    np.testing.assert_array_equal(a, got)                            # bitwise run-to-run determinism
+    plan.close()
+
+
+def test_pull_f64_torch_streams_and_tensor_devices(torch_cuda):
+    from drone_amd import rmat
+    from drone_amd.pagerank import PullPlanF64
+    torch = torch_cuda
+    x = rmat.pagerank_inputs_np(10, 16, 3)
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        rp, ci, inv = (torch.from_numpy(x[k]).cuda() for k in ("row_ptr", "col_idx", "inv_outdeg"))
+    s.synchronize()
+    plan = PullPlanF64(rp, ci, inv, stream=s.cuda_stream)
+    a = plan.run(0.85, 5)
+    s.synchronize()
+    plan0 = PullPlanF64(rp, ci, inv, stream=0)
+    b = plan0.run(0.85, 5)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    plan.close()
+    plan0.close()
+
+
+def test_pull_f64_full_size_properties(torch_cuda):
+    """Second benchmark configuration at full size (R-MAT scale 24, edge factor 16, seed 2): mass
+    conservation over 50 iterations and three iterations against an independent torch formulation
+    (the vendor's sparse CSR mat-vec in fp64), which the oracle would take minutes to produce."""
+    from drone_amd import rmat
+    from drone_amd.pagerank import PullPlanF64
+    torch = torch_cuda
+    x = rmat.pagerank_inputs_torch(24, 16, 2)
+    n = x["n"]
+    plan = PullPlanF64(x["row_ptr"], x["col_idx"], x["inv_outdeg"])
+    r50 = plan.run(ALPHA, 50)
+    assert abs(float(r50.sum()) - 1.0) < 1e-10
+    assert float(r50.min()) >= (1 - ALPHA) / n * (1 - 1e-12)
+    r3 = plan.run(ALPHA, 3)
+    A = torch.sparse_csr_tensor(x["row_ptr"], x["col_idx"].long(),
+                                torch.ones(x["nnz"], dtype=torch.float64, device="cuda"), size=(n, n))
+    r = torch.full((n,), 1.0 / n, dtype=torch.float64, device="cuda")
+    dang = x["inv_outdeg"] == 0
+    for _ in range(3):
+        c = r * x["inv_outdeg"]
+        s = torch.mv(A, c)
+        r = (1 - ALPHA) / n + ALPHA * (s + r[dang].sum() / n)
+    rel = ((r3 - r).abs() / r).max().item()
+    assert rel <= 1e-9, rel
+    plan.close()
+
+
+# ---------------------------------------------------------------- reference-compatible entry points
+def _edges(seed, scale=10, ef=8):
+    from drone_amd import rmat
+    s, d = rmat.rmat_edges(scale, (1 << scale) * ef, seed=seed)
+    src, dst = rmat.clean_directed_np(s, d)
+    rng = np.random.default_rng(seed)
+    p = rng.permutation(len(src))                     # arbitrary input order, as an edge file would have
+    gl = rng.permutation(1 << (scale + 1))[: 1 << scale]   # sparse global ids
+    return gl[src[p]].astype(np.int32), gl[dst[p]].astype(np.int32), 1 << (scale + 1)
+
+
+@pytest.mark.parametrize("seed", [1, 2])
+def test_build_graph_matches_reference_layout(torch_cuda, oracle, seed):
+    from drone_amd.pagerank import PRWorkerCUDA
+    u, v, gN = _edges(seed)
+    w = PRWorkerCUDA(gN, u, v)
+    n, g2l, l2g, index, dst = oracle.build_graph(gN, u, v)
+    got = w.graph_arrays()
+    assert w.n == n
+    np.testing.assert_array_equal(got["Global2Local"], g2l)
+    np.testing.assert_array_equal(got["Local2Global"], l2g)
+    np.testing.assert_array_equal(got["index"], index)
+    np.testing.assert_array_equal(got["dst"], dst)
+    g = w.g.contents
+    assert g.localVertexSize[0] == n and g.globalVertexSize[0] == gN and g.edgeSize[0] == len(u)
+    assert g.blockSize == 256 and g.gridSize == min((n - 1) // 256 + 1, 1024)
+    w.close()
+
+
+@pytest.mark.parametrize("seed,scale", [(1, 10), (3, 13)])
+def test_peval_inceval_against_push_oracle(torch_cuda, oracle, seed, scale):
+    from drone_amd.pagerank import PRWorkerCUDA
+    u, v, gN = _edges(seed, scale)
+    outdeg_global = np.bincount(u, minlength=gN).astype(np.int32)
+    w = PRWorkerCUDA(gN, u, v, outdeg_global)
+    n, g2l, l2g, index, dst = oracle.build_graph(gN, u, v)
+    st = oracle.PushState(index, dst, outdeg_global[l2g], gN)
+    res = w.peval()
+    assert res.VisitedSize == st.peval() and res.LocalVertexSize == n and res.IsEmpty()
+    s = w.state()
+    np.testing.assert_array_equal(s["outDegree"], outdeg_global[l2g])
+    np.testing.assert_array_equal(s["active"], st.active)
+    np.testing.assert_array_equal(s["pr"], st.pr)
+    np.testing.assert_allclose(s["diff"], st.diff, rtol=2e-5, atol=1e-7)
+    np.testing.assert_allclose(s["globalDiff"], st.gdiff[0], rtol=1e-5)
+    for k in range(1, 16):
+        res = w.incEval()
+        vis = st.inceval(alpha=0.85, eps=1e-6)
+        s = w.state()
+        if k <= 6:                      # before vertices start to freeze under eps the trajectories coincide
+            assert res.VisitedSize == vis
+            np.testing.assert_array_equal(s["active"], st.active)
+        np.testing.assert_allclose(s["pr"], st.pr, rtol=2e-5)
+        np.testing.assert_allclose(s["acc"], st.acc, rtol=2e-5, atol=1e-6)
+        np.testing.assert_allclose(s["globalAcc"], st.gacc[0], rtol=2e-5, atol=1e-7)
+    w.close()
+
+
+def test_push_path_converges_to_pull_ranks(torch_cuda, oracle):
+    """After enough supersteps the float delta-push state sits within the eps bound of the fp64 ranks."""
+    from drone_amd.pagerank import PRWorkerCUDA
+    u, v, gN = _edges(5, 11)
+    w = PRWorkerCUDA(gN, u, v)
+    w.peval()
+    for _ in range(80):
+        w.incEval()
+    pr = w.state()["pr"]
+    r = w.run_f64(0.85, 80) * gN          # the reference normalises by the GLOBAL vertex count
+    # pull over the local subgraph uses N_local; rescale: both are the same fixed point only when all
+    # global ids are present, so compare through the oracle on the local graph instead
+    n, g2l, l2g, index, dst = oracle.build_graph(gN, u, v)
+    rp, ci, inv = in_csr_np(n, np.repeat(np.arange(n), np.diff(index)), dst)
+    ref = oracle.pr_pull_f64(rp, ci, inv, 0.85, 80)
+    assert_rel(r / gN, ref, 1e-9)
+    w.close()
+    # float push state vs its own oracle after the same number of steps
+    st = oracle.PushState(index, dst, np.bincount(u, minlength=gN).astype(np.int32)[l2g], gN)
+    st.peval()
+    for _ in range(80):
+        st.inceval()
+    assert np.max(np.abs(pr - st.pr)) < 5 * 1e-6 * 0.85 / 0.15 + 1e-4
+
+
+def test_run_graph_f64_matches_oracle(torch_cuda, oracle):
+    from drone_amd.pagerank import PRWorkerCUDA
+    u, v, gN = _edges(7, 12)
+    w = PRWorkerCUDA(gN, u, v)
+    n, g2l, l2g, index, dst = oracle.build_graph(gN, u, v)
+    rp, ci, inv = in_csr_np(n, np.repeat(np.arange(n), np.diff(index)), dst)
+    for iters in (1, 20):
+        assert_rel(w.run_f64(0.85, iters), oracle.pr_pull_f64(rp, ci, inv, 0.85, iters), 1e-9)
+    w.close()
