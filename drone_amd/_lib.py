@@ -81,6 +81,23 @@ SIGNATURES = {
     "drone_pr_profile_read": (_I, [_P, C.POINTER(_I), C.POINTER(_D), C.POINTER(_D), C.POINTER(_D)]),
     "drone_pr_bytes_per_iteration": (_I64, [_I64, _I64]),
     "drone_pr_run_graph_f64": (_I, [C.POINTER(Graph), C.POINTER(PRValues), _D, _I, _P]),
+    "drone_gcn_edge_values": (_I, [_I, _P, _P, _P, _P, _P, _P]),
+    "drone_csr_transpose_f32": (_I, [_I, _I, _I64, _P, _P, _P, _P, _P, _P, _P]),
+    "drone_spmm_plan_create": (_I, [C.POINTER(_P), _I, _I64, _P, _I, _P]),
+    "drone_spmm_plan_destroy": (_I, [_P]),
+    "drone_spmm_csr_f32": (_I, [_P, _P, _P, _P, _P, _I, _P, _I, _I, _F, _F, _P]),
+    "drone_spmm_bytes": (_I64, [_I, _I64, _I]),
+    "drone_sgemm_rm_f32": (_I, [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P]),
+    "drone_sgemm_flops": (_I64, [_I, _I, _I]),
+    "drone_relu_forward_f32": (_I, [_P, _P, _I64, _I, _P]),
+    "drone_relu_backward_f32": (_I, [_P, _P, _I64, _P]),
+    "drone_dropout_mask": (_I, [_P, _I64, _U64, _U64, _F, _P]),
+    "drone_dropout_apply_f32": (_I, [_P, _P, _I64, _F, _P]),
+    "drone_cross_entropy_f32": (_I, [_I, _I, _P, _I, _P, _P, _I, _P, _P, _P]),
+    "drone_accuracy_f32": (_I, [_I, _I, _P, _I, _P, _P, _P, _P]),
+    "drone_sgd_step_f32": (_I, [_P, _P, _I64, _F, _P]),
+    "drone_adam_step_f32": (_I, [_P, _P, _P, _P, _I64, _I, _F, _F, _F, _F, _F, _I, _P]),
+    "drone_fill_f32": (_I, [_P, _I64, _F, _P]),
     "drone_rmat_edges": (_I, [_I, _I64, _D, _D, _D, _U64, _I64, _P, _P]),
     "drone_fill_uniform_f32": (_I, [_P, _I64, _U64, _F, _F]),
     "drone_fill_normal_f32": (_I, [_P, _I64, _U64]),

@@ -1,0 +1,246 @@
+// Row-major fp32 GEMM on the gfx950 matrix cores:  C(MxN) = alpha * op(A)(MxK) * op(B)(KxN) + beta * C.
+// Replaces the three cublasSgemm calls of cuda_gcn's CUDAMatmul (cuda_gcn/src/cuda/cuda_module.cu:25-38
+// forward, :72-85 input gradient, :92-105 weight gradient), which are tall-skinny: M or K is the vertex
+// count, the other dimensions are feature widths (41..602).
+//
+// Work-group = 256 lanes = 4 wavefronts computing a 128 x BN tile of C (BN = 128 or 64) with
+// v_mfma_f32_32x32x2_f32: every wavefront owns a (128/WM) x (BN/WN) sub-tile as 32x32 accumulators.
+// A and B tiles of depth 16 are staged through LDS k-major ([k][m], [k][n]) so that the lanes of one MFMA
+// operand read consecutive addresses; global loads are issued one tile ahead of the math.  Loads are plain
+// dword loads with bounds checks (arbitrary M, N, K and leading dimensions, no alignment demands); adjacent
+// lanes read adjacent addresses in whichever dimension is contiguous in memory.
+// A long reduction with a small output (the weight gradient: K = vertex count) is split over grid.z; the
+// partial tiles go to a scratch buffer and are summed in split order by a second kernel.
+#include <mutex>
+
+#include "common.h"
+
+namespace drone {
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 128;
+constexpr int BK = 16;
+constexpr int PAD = 4;
+
+// Loads a (BK x EXT) k-major tile of op(X) into registers: element (k, i) for k in [0,BK), i in [0,EXT).
+// K_CONTIG: memory holds X[i][k] (k contiguous) - lanes walk k fastest; else X[k][i] - lanes walk i fastest.
+template <int EXT, bool K_CONTIG>
+struct TileLoader {
+    static constexpr int PER = BK * EXT / 256;
+    float r[PER];
+    __device__ __forceinline__ void load(const float *__restrict__ X, int ld, int i0, int i_end, int k0, int k_end)
+    {
+        const int t = threadIdx.x;
+#pragma unroll
+        for (int p = 0; p < PER; ++p) {
+            int k, i;
+            if constexpr (K_CONTIG) { k = t % BK; i = t / BK + p * (256 / BK); }
+            else { i = t % EXT; k = t / EXT + p * (256 / EXT); }
+            const int gi = i0 + i, gk = k0 + k;
+            float v = 0.0f;
+            if (gi < i_end && gk < k_end) v = K_CONTIG ? X[(size_t)gi * ld + gk] : X[(size_t)gk * ld + gi];
+            r[p] = v;
+        }
+    }
+    __device__ __forceinline__ void store(float *s /* [BK][EXT+PAD] */) const
+    {
+        const int t = threadIdx.x;
+#pragma unroll
+        for (int p = 0; p < PER; ++p) {
+            int k, i;
+            if constexpr (K_CONTIG) { k = t % BK; i = t / BK + p * (256 / BK); }
+            else { i = t % EXT; k = t / EXT + p * (256 / EXT); }
+            s[k * (EXT + PAD) + i] = r[p];
+        }
+    }
+};
+
+// op(A) is M x K: TA=false -> A stored M x K (k contiguous); TA=true -> A stored K x M (m contiguous).
+// op(B) is K x N: TB=false -> B stored K x N (n contiguous); TB=true -> B stored N x K (k contiguous).
+template <int BN, bool TA, bool TB>
+__global__ __launch_bounds__(256) void sgemm_mfma_kernel(int M, int N, int K, float alpha, const float *__restrict__ A,
+                                                         int lda, const float *__restrict__ B, int ldb, float beta,
+                                                         float *__restrict__ C, int ldc, int k_chunk,
+                                                         float *__restrict__ partial)
+{
+    constexpr int WN = BN / 64;        // wavefronts along n (2 or 1)
+    constexpr int WM = 4 / WN;         // wavefronts along m
+    constexpr int TM = BM / WM / 32;   // 32x32 accumulators per wavefront along m (2 or 1)
+    constexpr int TN = 2;              // and along n (64 columns per wavefront)
+    __shared__ float sA[2][BK * (BM + PAD)];
+    __shared__ float sB[2][BK * (BN + PAD)];
+
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int kb = blockIdx.z * k_chunk;
+    const int ke = kb + k_chunk < K ? kb + k_chunk : K;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+    const int wm = wave / WN, wn = wave % WN;
+    const int lr = lane & 31, lk = lane >> 5;
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    TileLoader<BM, !TA> la;
+    TileLoader<BN, TB> lb;
+    la.load(A, lda, m0, M, kb, ke);
+    lb.load(B, ldb, n0, N, kb, ke);
+    la.store(sA[0]);
+    lb.store(sB[0]);
+    __syncthreads();
+
+    int buf = 0;
+    for (int k0 = kb; k0 < ke; k0 += BK) {
+        const bool more = k0 + BK < ke;
+        if (more) {
+            la.load(A, lda, m0, M, k0 + BK, ke);
+            lb.load(B, ldb, n0, N, k0 + BK, ke);
+        }
+        const float *a = sA[buf], *b = sB[buf];
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 2) {
+            float av[TM], bv[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) av[i] = a[(kk + lk) * (BM + PAD) + wm * (TM * 32) + i * 32 + lr];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) bv[j] = b[(kk + lk) * (BN + PAD) + wn * 64 + j * 32 + lr];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            la.store(sA[buf ^ 1]);
+            lb.store(sB[buf ^ 1]);
+        }
+        __syncthreads();
+        buf ^= 1;
+    }
+
+    // 32x32 accumulator layout: register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4, column l%32.
+    float *out = partial ? partial + (size_t)blockIdx.z * M * N : C;
+    const int ldo = partial ? N : ldc;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = m0 + wm * (TM * 32) + i * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
+                const int col = n0 + wn * 64 + j * 32 + lr;
+                if (row < M && col < N) {
+                    if (partial) {
+                        out[(size_t)row * ldo + col] = acc[i][j][v];
+                    } else {
+                        float r = alpha * acc[i][j][v];
+                        if (beta != 0.0f) r += beta * out[(size_t)row * ldo + col];
+                        out[(size_t)row * ldo + col] = r;
+                    }
+                }
+            }
+}
+
+// C = alpha * sum_z partial[z] + beta * C, z ascending
+__global__ void sgemm_reduce_kernel(int M, int N, int splits, const float *__restrict__ partial, float alpha,
+                                    float beta, float *__restrict__ C, int ldc)
+{
+    const int64_t total = (int64_t)M * N;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+        float s = 0.0f;
+        for (int z = 0; z < splits; ++z) s += partial[(size_t)z * total + idx];
+        const int row = (int)(idx / N), col = (int)(idx % N);
+        float r = alpha * s;
+        if (beta != 0.0f) r += beta * C[(size_t)row * ldc + col];
+        C[(size_t)row * ldc + col] = r;
+    }
+}
+
+// Grow-only scratch for split-K partials, one per device.  Calls that use it must not overlap on a device.
+std::mutex g_ws_mutex;
+float *g_ws[16] = {};
+size_t g_ws_bytes[16] = {};
+
+int workspace(size_t bytes, float **out)
+{
+    int dev = 0;
+    DRONE_HIP_TRY(hipGetDevice(&dev));
+    DRONE_REQUIRE(dev >= 0 && dev < 16, "device ordinal");
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    if (g_ws_bytes[dev] < bytes) {
+        if (g_ws[dev]) {
+            DRONE_HIP_TRY(hipDeviceSynchronize());
+            (void)hipFree(g_ws[dev]);
+            g_ws[dev] = nullptr;
+            g_ws_bytes[dev] = 0;
+        }
+        DRONE_HIP_TRY(hipMalloc(&g_ws[dev], bytes));
+        g_ws_bytes[dev] = bytes;
+    }
+    *out = g_ws[dev];
+    return DRONE_OK;
+}
+
+template <int BN>
+void launch(bool ta, bool tb, dim3 grid, hipStream_t s, int M, int N, int K, float alpha, const float *A, int lda,
+            const float *B, int ldb, float beta, float *C, int ldc, int k_chunk, float *partial)
+{
+    if (!ta && !tb) sgemm_mfma_kernel<BN, false, false><<<grid, 256, 0, s>>>(M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
+    else if (!ta && tb) sgemm_mfma_kernel<BN, false, true><<<grid, 256, 0, s>>>(M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
+    else if (ta && !tb) sgemm_mfma_kernel<BN, true, false><<<grid, 256, 0, s>>>(M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
+    else sgemm_mfma_kernel<BN, true, true><<<grid, 256, 0, s>>>(M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
+}
+
+}  // namespace
+}  // namespace drone
+
+using namespace drone;
+
+extern "C" int drone_sgemm_rm_f32(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,
+                                  const float *B, int ldb, float beta, float *C, int ldc, drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(M >= 0 && N >= 0 && K >= 0, "negative dimension");
+    DRONE_REQUIRE(ldc >= N, "ldc < N");
+    DRONE_REQUIRE(lda >= (transA ? M : K) && ldb >= (transB ? K : N), "leading dimension too small");
+    if (M == 0 || N == 0) return DRONE_OK;
+    DRONE_REQUIRE(C != nullptr && (K == 0 || (A && B)), "null operand");
+    hipStream_t s = as_stream(stream);
+    const bool narrow = N <= 64;
+    const int bn = narrow ? 64 : 128;
+    const int tiles = (int)(ceil_div(M, BM) * ceil_div(N, bn));
+    // split the reduction when the output has too few tiles to fill 256 CUs and K is long
+    int splits = 1;
+    if (tiles < 256 && K >= 4096) {
+        splits = (int)ceil_div(1024, tiles);
+        const int max_splits = (int)ceil_div(K, 512);
+        if (splits > max_splits) splits = max_splits;
+        if (splits > 512) splits = 512;
+    }
+    int k_chunk = (int)ceil_div(ceil_div(K > 0 ? K : 1, splits), BK) * BK;
+    splits = (int)ceil_div(K > 0 ? K : 1, k_chunk);
+    float *partial = nullptr;
+    if (splits > 1) {
+        int rc = workspace(sizeof(float) * (size_t)splits * M * N, &partial);
+        if (rc != DRONE_OK) return rc;
+    }
+    dim3 grid((unsigned)ceil_div(N, bn), (unsigned)ceil_div(M, BM), (unsigned)splits);
+    DRONE_REQUIRE(grid.y <= 65535u * 32u, "M too large for the launch grid");
+    if (narrow) launch<64>(transA != 0, transB != 0, grid, s, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
+    else launch<128>(transA != 0, transB != 0, grid, s, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
+    if (splits > 1) {
+        int blocks = (int)ceil_div((int64_t)M * N, 256);
+        if (blocks > 4096) blocks = 4096;
+        sgemm_reduce_kernel<<<blocks, 256, 0, s>>>(M, N, splits, partial, alpha, beta, C, ldc);
+    }
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
+extern "C" int64_t drone_sgemm_flops(int M, int N, int K) { return 2ll * M * N * K; }

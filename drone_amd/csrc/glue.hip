@@ -1,0 +1,325 @@
+// Element-wise and per-row kernels on the measured GCN step, semantics as in cuda_gcn/src/cuda/cuda_kernel.cu:
+// ReLU (:384-399), dropout with an explicit keep mask (:403-420), soft-max cross-entropy (:295-379 with the
+// host logic of cuda_module.cu:406-483), Adam (:450-460), plus SGD, accuracy (cuda_gcn.cu:226-246) and arg-max.
+#include <mutex>
+
+#include "common.h"
+
+namespace drone {
+namespace {
+
+constexpr int kThreads = 256;
+
+inline int grid_for(int64_t n, int per_thread = 4)
+{
+    int64_t b = ceil_div(n, (int64_t)kThreads * per_thread);
+    if (b < 1) b = 1;
+    if (b > 65536) b = 65536;
+    return (int)b;
+}
+
+__device__ __forceinline__ uint64_t splitmix64_dev(uint64_t x)
+{
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+
+__global__ void relu_forward_kernel(float *__restrict__ x, uint8_t *__restrict__ mask, int64_t n, int training)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        const bool keep = x[i] > 0;
+        if (training) mask[i] = keep;
+        if (!keep) x[i] = 0;
+    }
+}
+
+__global__ void relu_backward_kernel(float *__restrict__ g, const uint8_t *__restrict__ mask, int64_t n)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        if (!mask[i]) g[i] = 0;
+}
+
+// keep[i] = u(seed, step, i) >= p with u uniform in [0,1): a pure function of its arguments
+__global__ void dropout_mask_kernel(uint8_t *__restrict__ keep, int64_t n, uint64_t seed, uint64_t step, float p)
+{
+    const uint64_t key = splitmix64_dev(splitmix64_dev(seed) ^ (step * 0xD1342543DE82EF95ull));
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        const float u = (float)(splitmix64_dev(key + (uint64_t)i) >> 40) * (1.0f / 16777216.0f);
+        keep[i] = u >= p;
+    }
+}
+
+__global__ void dropout_apply_kernel(float *__restrict__ x, const uint8_t *__restrict__ keep, int64_t n, float scale)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        x[i] *= keep[i] ? scale : 0.0f;
+}
+
+// One wavefront per row.  grad = softmax - onehot on labelled rows, 0 elsewhere; the per-block loss sum and
+// labelled-row count go to block_loss / block_count.
+__global__ __launch_bounds__(kThreads) void cross_entropy_kernel(int n, int classes, const float *__restrict__ logits,
+                                                                 int ld, const int *__restrict__ truth,
+                                                                 float *__restrict__ grad, int ldg,
+                                                                 double *__restrict__ block_loss,
+                                                                 int *__restrict__ block_count)
+{
+    __shared__ double s_loss[kThreads / kWave];
+    __shared__ int s_cnt[kThreads / kWave];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    double loss = 0.0;
+    int cnt = 0;
+    for (int row = blockIdx.x * (kThreads / kWave) + wave; row < n; row += gridDim.x * (kThreads / kWave)) {
+        const float *z = logits + (size_t)row * ld;
+        const int t = truth[row];
+        if (t < 0) {
+            if (grad) for (int j = lane; j < classes; j += kWave) grad[(size_t)row * ldg + j] = 0.0f;
+            continue;
+        }
+        float mx = -INFINITY;
+        for (int j = lane; j < classes; j += kWave) mx = fmaxf(mx, z[j]);
+#pragma unroll
+        for (int m = kWave / 2; m > 0; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, kWave));
+        float sum = 0.0f;
+        for (int j = lane; j < classes; j += kWave) sum += expf(z[j] - mx);
+#pragma unroll
+        for (int m = kWave / 2; m > 0; m >>= 1) sum += __shfl_xor(sum, m, kWave);
+        if (grad)
+            for (int j = lane; j < classes; j += kWave) {
+                float g = expf(z[j] - mx) / sum;
+                if (j == t) g -= 1.0f;
+                grad[(size_t)row * ldg + j] = g;
+            }
+        if (lane == 0) {
+            loss += (double)(logf(sum) - (z[t] - mx));
+            cnt += 1;
+        }
+    }
+    if (lane == 0) { s_loss[wave] = loss; s_cnt[wave] = cnt; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double l = 0.0;
+        int c = 0;
+        for (int w = 0; w < kThreads / kWave; ++w) { l += s_loss[w]; c += s_cnt[w]; }
+        block_loss[blockIdx.x] = l;
+        block_count[blockIdx.x] = c;
+    }
+}
+
+// loss_out = sum(block_loss) / sum(block_count) (mean over labelled rows), count_out = sum(block_count)
+__global__ __launch_bounds__(kThreads) void cross_entropy_finish_kernel(int blocks, const double *__restrict__ block_loss,
+                                                                        const int *__restrict__ block_count,
+                                                                        float *__restrict__ loss_out,
+                                                                        int *__restrict__ count_out)
+{
+    __shared__ double s_l[kThreads];
+    __shared__ int s_c[kThreads];
+    double l = 0.0;
+    int c = 0;
+    for (int i = threadIdx.x; i < blocks; i += kThreads) { l += block_loss[i]; c += block_count[i]; }
+    s_l[threadIdx.x] = l;
+    s_c[threadIdx.x] = c;
+    __syncthreads();
+    for (int m = kThreads / 2; m > 0; m >>= 1) {
+        if (threadIdx.x < m) { s_l[threadIdx.x] += s_l[threadIdx.x + m]; s_c[threadIdx.x] += s_c[threadIdx.x + m]; }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        if (loss_out) *loss_out = (float)(s_l[0] / (double)s_c[0]);
+        if (count_out) *count_out = s_c[0];
+    }
+}
+
+// cuda_gcn.cu:226-246: a labelled row is wrong iff some logit is strictly greater than the true-class logit.
+// pred[row] = arg-max with ties to the lowest index (optional).  counts[0] += correct, counts[1] += labelled.
+__global__ __launch_bounds__(kThreads) void accuracy_kernel(int n, int classes, const float *__restrict__ logits, int ld,
+                                                            const int *__restrict__ truth, int *__restrict__ pred,
+                                                            int *__restrict__ counts)
+{
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    int correct = 0, total = 0;
+    for (int row = blockIdx.x * (kThreads / kWave) + wave; row < n; row += gridDim.x * (kThreads / kWave)) {
+        const float *z = logits + (size_t)row * ld;
+        float best = -INFINITY;
+        int arg = INT32_MAX;
+        for (int j = lane; j < classes; j += kWave) {
+            const float v = z[j];
+            if (v > best) { best = v; arg = j; }
+        }
+#pragma unroll
+        for (int m = kWave / 2; m > 0; m >>= 1) {
+            const float ob = __shfl_xor(best, m, kWave);
+            const int oa = __shfl_xor(arg, m, kWave);
+            if (ob > best || (ob == best && oa < arg)) { best = ob; arg = oa; }
+        }
+        if (lane == 0) {
+            if (pred) pred[row] = arg;
+            const int t = truth ? truth[row] : -1;
+            if (t >= 0) {
+                total++;
+                if (!(best > z[t])) correct++;
+            }
+        }
+    }
+    if (counts && lane == 0 && total) {
+        atomicAdd(&counts[0], correct);
+        atomicAdd(&counts[1], total);
+    }
+}
+
+__global__ void sgd_kernel(float *__restrict__ w, const float *__restrict__ g, int64_t n, float lr)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        w[i] -= lr * g[i];
+}
+
+// cuda_kernel.cu:450-460
+__global__ void adam_kernel(float *__restrict__ w, const float *__restrict__ grad, float *__restrict__ m,
+                            float *__restrict__ v, int64_t n, int decay, float weight_decay, float beta1, float beta2,
+                            float eps, float step_size)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        float g = grad[i];
+        if (decay) g += weight_decay * w[i];
+        const float mi = (float)(beta1 * m[i] + (1.0 - beta1) * g);
+        const float vi = (float)(beta2 * v[i] + (1.0 - beta2) * g * g);
+        m[i] = mi;
+        v[i] = vi;
+        w[i] -= step_size * mi / (sqrtf(vi) + eps);
+    }
+}
+
+__global__ void fill_f32_kernel(float *__restrict__ x, int64_t n, float value)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        x[i] = value;
+}
+
+// scratch for the cross-entropy block partials, one per device (grow-only)
+std::mutex g_mutex;
+void *g_ce_ws[16] = {};
+int g_ce_blocks[16] = {};
+
+}  // namespace
+}  // namespace drone
+
+using namespace drone;
+
+extern "C" int drone_relu_forward_f32(float *x, uint8_t *mask, int64_t n, int training, drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(n >= 0 && (n == 0 || x) && (!training || mask || n == 0), "null operand");
+    if (n == 0) return DRONE_OK;
+    relu_forward_kernel<<<grid_for(n), kThreads, 0, as_stream(stream)>>>(x, mask, n, training);
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
+extern "C" int drone_relu_backward_f32(float *grad, const uint8_t *mask, int64_t n, drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(n >= 0 && (n == 0 || (grad && mask)), "null operand");
+    if (n == 0) return DRONE_OK;
+    relu_backward_kernel<<<grid_for(n), kThreads, 0, as_stream(stream)>>>(grad, mask, n);
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
+extern "C" int drone_dropout_mask(uint8_t *keep, int64_t n, uint64_t seed, uint64_t step, float p, drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(n >= 0 && (n == 0 || keep) && p >= 0.0f && p < 1.0f, "mask / probability");
+    if (n == 0) return DRONE_OK;
+    dropout_mask_kernel<<<grid_for(n), kThreads, 0, as_stream(stream)>>>(keep, n, seed, step, p);
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
+// Forward and backward are the same scaling (cuda_kernel.cu:403-420): x *= keep ? 1/(1-p) : 0.
+extern "C" int drone_dropout_apply_f32(float *x, const uint8_t *keep, int64_t n, float p, drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(n >= 0 && (n == 0 || (x && keep)) && p >= 0.0f && p < 1.0f, "operand / probability");
+    if (n == 0) return DRONE_OK;
+    dropout_apply_kernel<<<grid_for(n), kThreads, 0, as_stream(stream)>>>(x, keep, n, 1 / (1 - p));
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
+extern "C" int drone_cross_entropy_f32(int n, int classes, const float *logits, int ld, const int *truth, float *grad,
+                                       int ldg, float *loss_out, int *count_out, drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(n > 0 && classes > 0 && logits && truth && ld >= classes, "operands");
+    DRONE_REQUIRE(grad == nullptr || ldg >= classes, "ldg < classes");
+    int dev = 0;
+    DRONE_HIP_TRY(hipGetDevice(&dev));
+    DRONE_REQUIRE(dev >= 0 && dev < 16, "device ordinal");
+    int blocks = (int)ceil_div(n, kThreads / kWave);
+    if (blocks > 2048) blocks = 2048;
+    void *ws = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        if (g_ce_blocks[dev] < 2048) {
+            DRONE_HIP_TRY(hipMalloc(&g_ce_ws[dev], 2048 * (sizeof(double) + sizeof(int))));
+            g_ce_blocks[dev] = 2048;
+        }
+        ws = g_ce_ws[dev];
+    }
+    double *bl = static_cast<double *>(ws);
+    int *bc = reinterpret_cast<int *>(bl + 2048);
+    hipStream_t s = as_stream(stream);
+    cross_entropy_kernel<<<blocks, kThreads, 0, s>>>(n, classes, logits, ld, truth, grad, ldg, bl, bc);
+    cross_entropy_finish_kernel<<<1, kThreads, 0, s>>>(blocks, bl, bc, loss_out, count_out);
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
+extern "C" int drone_accuracy_f32(int n, int classes, const float *logits, int ld, const int *truth, int *pred,
+                                  int *counts, drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(n > 0 && classes > 0 && logits && ld >= classes, "operands");
+    hipStream_t s = as_stream(stream);
+    int blocks = (int)ceil_div(n, kThreads / kWave);
+    if (blocks > 4096) blocks = 4096;
+    accuracy_kernel<<<blocks, kThreads, 0, s>>>(n, classes, logits, ld, truth, pred, counts);
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
+extern "C" int drone_sgd_step_f32(float *w, const float *g, int64_t n, float lr, drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(n >= 0 && (n == 0 || (w && g)), "null operand");
+    if (n == 0) return DRONE_OK;
+    sgd_kernel<<<grid_for(n), kThreads, 0, as_stream(stream)>>>(w, g, n, lr);
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
+// cuda_module.cu:590-600: step_count is the value after the increment.
+extern "C" int drone_adam_step_f32(float *w, const float *g, float *m, float *v, int64_t n, int decay,
+                                   float weight_decay, float lr, float beta1, float beta2, float eps, int step_count,
+                                   drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(n >= 0 && (n == 0 || (w && g && m && v)) && step_count >= 1, "operands");
+    if (n == 0) return DRONE_OK;
+    const float step_size = lr * sqrtf(1 - powf(beta2, (float)step_count)) / (1 - powf(beta1, (float)step_count));
+    adam_kernel<<<grid_for(n), kThreads, 0, as_stream(stream)>>>(w, g, m, v, n, decay, weight_decay, beta1, beta2, eps,
+                                                               step_size);
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
+extern "C" int drone_fill_f32(float *x, int64_t n, float value, drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(n >= 0 && (n == 0 || x), "null operand");
+    if (n == 0) return DRONE_OK;
+    fill_f32_kernel<<<grid_for(n), kThreads, 0, as_stream(stream)>>>(x, n, value);
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}

@@ -52,7 +52,7 @@ typedef struct Graph {
     int *MasterWorkerIndex; /* device [local+1]: master local id -> slice of Master2Workers    */
     int *Master2Workers;
     int MasterSize, MirrorWorkerSize;
-    int *Mirror2Worker; /* host-readable + device [local]: -1 unless the vertex is a mirror    */
+    int *Mirror2Worker; /* device [local]: -1 unless the vertex is a mirror                    */
     int MirrorSize;
     int *index;     /* device [local+1]: out-edge CSR offsets                                  */
     int *dst;       /* device [edgeSize]: out-edge CSR targets (local ids, input order kept)   */
@@ -121,9 +121,11 @@ void drone_pr_values_destroy(Graph *g, PRValues *values);
  * iteration (pr.cu:51-87 with eps = 0) normalised by N and written as a pull.                */
 typedef struct drone_pr_plan drone_pr_plan;
 
-/* Builds the merge-path tiling for the CSR and allocates the work vectors (the only allocations
- * of this path).  row_ptr [n+1], col_idx [nnz], inv_outdeg [n] stay owned by the caller and must
- * outlive the plan. */
+/* Builds, once per CSR: a hot-first relabelled copy of the CSR (vertices sorted by how often they
+ * are gathered, so that popular sources share cache lines), its merge-path tiling, and the work
+ * vectors - the only allocations of this path.  row_ptr [n+1] and col_idx [nnz] are read during this
+ * call only; inv_outdeg [n] is re-read at the start of every run and must outlive the plan.
+ * Results are returned in the caller's vertex order. */
 int drone_pr_plan_create(drone_pr_plan **plan, int64_t n, int64_t nnz, const int64_t *row_ptr,
                          const int32_t *col_idx, const double *inv_outdeg, drone_stream_t stream);
 int drone_pr_plan_destroy(drone_pr_plan *plan);
@@ -143,6 +145,69 @@ int64_t drone_pr_bytes_per_iteration(int64_t n, int64_t nnz);
 /* Same iteration driven from a Graph built by build_graph + loadOutDegree (local out-degrees are
  * taken from PRValues.outDegree).  rank_out: host [localVertexSize], normalised ranks. */
 int drone_pr_run_graph_f64(Graph *g, PRValues *values, double alpha, int iters, double *rank_out);
+
+/* ====================================================================================== */
+/* C. GCN layer kernels (replace the vendor calls and glue kernels of cuda_gcn's modules)   */
+/* ====================================================================================== */
+/* All dense operands are row-major fp32 with explicit leading dimensions (in elements); CSR arrays are
+ * int32 offsets / int32 columns / fp32 values, base 0 - the descriptors of cuda_module.cu:166-194.
+ * Calls are asynchronous on `stream`.  Apart from plan creation, the transpose (a set-up step) and
+ * grow-only scratch kept per device by drone_sgemm_rm_f32 (split reductions) and
+ * drone_cross_entropy_f32, nothing allocates; calls that use that scratch must not overlap on a device. */
+
+/* cuda_gcn/src/cuda/cuda_kernel.cu:145-155 (launched at cuda_module.cu:163):
+ * v[e(u->col)] = 1 / sqrtf(1.0 * out_deg[u] * in_deg[col]) for every entry of row u. */
+int drone_gcn_edge_values(int n, const int *rp, const int *ci, const int *in_deg, const int *out_deg,
+                          float *v, drone_stream_t stream);
+/* cusparseCsr2cscEx2(..., NUMERIC, ALG1) at cuda_module.cu:175-186: CSR of the transpose; row indices
+ * ascend within each output row.  v / vT may both be NULL (pattern only).  Synchronises `stream`. */
+int drone_csr_transpose_f32(int n_rows, int n_cols, int64_t nnz, const int *rp, const int *ci,
+                            const float *v, int *rpT, int *ciT, float *vT, drone_stream_t stream);
+/* Row classification for the SpMM of one CSR (rows with more than 4096 entries are split); holds the
+ * scratch for their partial rows, sized for feature widths up to max_k.  rp is read during the call. */
+typedef struct drone_spmm_plan drone_spmm_plan;
+int drone_spmm_plan_create(drone_spmm_plan **plan, int n_rows, int64_t nnz, const int *rp, int max_k,
+                           drone_stream_t stream);
+int drone_spmm_plan_destroy(drone_spmm_plan *plan);
+/* cusparseSpMM(NON_TRANSPOSE, NON_TRANSPOSE, alpha, A, B, beta, C, ALG_DEFAULT) at cuda_module.cu:245
+ * (forward: A = transposed CSR) and :335 (backward: A = original CSR):
+ * C[n_rows x K] = alpha * A * B + beta * C. */
+int drone_spmm_csr_f32(const drone_spmm_plan *plan, const int *rp, const int *ci, const float *v,
+                       const float *B, int ldb, float *C, int ldc, int K, float alpha, float beta,
+                       drone_stream_t stream);
+/* Algorithmic bytes of one SpMM: 4(n_rows+1) + 8 nnz + 8 n_rows K. */
+int64_t drone_spmm_bytes(int n_rows, int64_t nnz, int K);
+/* cublasSgemm at cuda_module.cu:25-38 (C = A*B), :72-85 (A.grad = C.grad*B^T: transB), :92-105
+ * (B.grad = A^T*C.grad: transA), written row-major: C(MxN) = alpha*op(A)(MxK)*op(B)(KxN) + beta*C.
+ * transA: A is stored K x M; transB: B is stored N x K. */
+int drone_sgemm_rm_f32(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,
+                       const float *B, int ldb, float beta, float *C, int ldc, drone_stream_t stream);
+int64_t drone_sgemm_flops(int M, int N, int K);
+/* cuda_kernel.cu:384-392 / :394-399: in-place ReLU with a byte mask recorded when training. */
+int drone_relu_forward_f32(float *x, uint8_t *mask, int64_t n, int training, drone_stream_t stream);
+int drone_relu_backward_f32(float *grad, const uint8_t *mask, int64_t n, drone_stream_t stream);
+/* cuda_kernel.cu:403-420 with the keep-mask explicit (the reference draws it from cuRAND states that
+ * cannot be reproduced): keep[i] = u(seed, step, i) >= p, then x *= keep ? 1/(1-p) : 0 for both the
+ * forward activations and the backward gradients. */
+int drone_dropout_mask(uint8_t *keep, int64_t n, uint64_t seed, uint64_t step, float p, drone_stream_t stream);
+int drone_dropout_apply_f32(float *x, const uint8_t *keep, int64_t n, float p, drone_stream_t stream);
+/* cuda_kernel.cu:295-379 + cuda_module.cu:406-483.  truth[i] < 0 = unlabelled.  grad (optional) receives
+ * softmax - onehot on labelled rows and 0 elsewhere - a SUM-reduced gradient (count_grad = 1 in the
+ * reference); *loss_out (device) = mean loss over labelled rows, *count_out (device) = their number. */
+int drone_cross_entropy_f32(int n, int classes, const float *logits, int ld, const int *truth, float *grad,
+                            int ldg, float *loss_out, int *count_out, drone_stream_t stream);
+/* cuda_gcn.cu:226-246: a labelled row is correct unless some logit is strictly greater than the true-class
+ * logit.  counts[0] += correct, counts[1] += labelled (device ints, zeroed by the caller); pred (optional)
+ * receives the arg-max with ties to the lowest index. */
+int drone_accuracy_f32(int n, int classes, const float *logits, int ld, const int *truth, int *pred,
+                       int *counts, drone_stream_t stream);
+/* w -= lr * g (the optimiser the benchmark configuration names). */
+int drone_sgd_step_f32(float *w, const float *g, int64_t n, float lr, drone_stream_t stream);
+/* cuda_module.cu:590-600 + cuda_kernel.cu:450-460; step_count is the value after the increment. */
+int drone_adam_step_f32(float *w, const float *g, float *m, float *v, int64_t n, int decay,
+                        float weight_decay, float lr, float beta1, float beta2, float eps, int step_count,
+                        drone_stream_t stream);
+int drone_fill_f32(float *x, int64_t n, float value, drone_stream_t stream);
 
 /* ====================================================================================== */
 /* D. Utilities                                                                           */

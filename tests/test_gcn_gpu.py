@@ -1,0 +1,260 @@
+"""GPU parity of the GCN kernels (SpMM, CSR transpose, edge values, MFMA GEMM, glue) against the CPU oracle,
+through the C ABI.  Tolerance for floating point: 1e-4 relative to the fp64-accumulated oracle value, measured
+against the row's scale (|A|·|B| accumulated), since fp32 summation order differs; integer results and
+masks are exact; arg-max predictions must be identical."""
+import json
+import os
+
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+@pytest.fixture(scope="module")
+def T():
+    import torch
+    assert torch.cuda.is_available()
+    return torch
+
+
+def dev(T, a):
+    return T.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def rel_err(got, ref64, scale64):
+    """max |got - ref| / scale, scale = sum |a||b| per output (>= |ref|), floored to avoid 0/0."""
+    return float(np.max(np.abs(got.astype(np.float64) - ref64) / np.maximum(scale64, 1e-30)))
+
+
+def random_csr(seed, n_rows, n_cols, density, hub=None):
+    rng = np.random.default_rng(seed)
+    m = sp.random(n_rows, n_cols, density=density, random_state=np.random.RandomState(seed), format="lil",
+                  dtype=np.float32)
+    if hub is not None:                       # one very long row to force the split path
+        cols = rng.choice(n_cols, size=hub, replace=False)
+        m[3, cols] = rng.uniform(-1, 1, hub).astype(np.float32)
+    m = m.tocsr()
+    m.sort_indices()
+    m.data = rng.uniform(-1, 1, m.nnz).astype(np.float32)
+    return m
+
+
+def run_spmm(T, m, B, K=None, ld_pad=0, alpha=1.0, beta=0.0, C0=None):
+    from drone_amd import gcn
+    rp, ci, v = dev(T, m.indptr.astype(np.int32)), dev(T, m.indices.astype(np.int32)), dev(T, m.data)
+    K = B.shape[1] if K is None else K
+    Bd = T.zeros((B.shape[0], K + ld_pad), dtype=T.float32, device="cuda")
+    Bd[:, :K] = dev(T, B)
+    out = T.full((m.shape[0], K + ld_pad), 7.0, dtype=T.float32, device="cuda")
+    if C0 is not None:
+        out[:, :K] = dev(T, C0)
+    plan = gcn.SpmmPlan(rp, m.nnz, max_k=K)
+    gcn.spmm(plan, rp, ci, v, Bd[:, :K], K=K, out=out[:, :K], alpha=alpha, beta=beta)
+    T.cuda.synchronize()
+    plan.close()
+    res = out.cpu().numpy()
+    if ld_pad:
+        assert np.all(res[:, K:] == 7.0), "wrote into the padding"
+    return res[:, :K]
+
+
+def test_spmm_known_answer_from_reference_sample(T):
+    k = json.load(open(os.path.join(GOLD, "spmm_kat_sparse_cu.json")))
+    m = sp.csr_matrix((np.array(k["val"], np.float32), np.array(k["ci"]), np.array(k["rp"])), shape=(4, 4))
+    B = np.array(k["B_colmajor"], np.float32).reshape(3, 4).T.copy()
+    Cexp = np.array(k["C_colmajor"], np.float32).reshape(3, 4).T
+    np.testing.assert_array_equal(run_spmm(T, m, B), Cexp)
+
+
+@pytest.mark.parametrize("K,ld_pad", [(1, 0), (3, 1), (16, 0), (41, 0), (41, 3), (64, 0), (128, 0), (130, 2), (256, 0), (300, 0)])
+def test_spmm_against_oracle(T, oracle, K, ld_pad):
+    m = random_csr(K, 300, 257, 0.05, hub=250)
+    B = np.random.default_rng(K).uniform(-1, 1, (257, K)).astype(np.float32)
+    got = run_spmm(T, m, B, ld_pad=ld_pad)
+    ref = oracle.spmm_f64acc(m.indptr, m.indices, m.data, B)
+    scale = oracle.spmm_f64acc(m.indptr, m.indices, np.abs(m.data), np.abs(B))
+    assert rel_err(got, ref, scale) <= 1e-4
+    assert np.all(got[np.diff(m.indptr) == 0] == 0.0)             # empty rows are written as zero (beta = 0)
+
+
+def test_spmm_long_rows_split_and_alpha_beta(T, oracle):
+    n = 9000
+    m = random_csr(5, 40, n, 0.002, hub=8500)                       # row 3 has > 4096 entries -> split path
+    assert np.diff(m.indptr).max() > 4096
+    B = np.random.default_rng(1).uniform(-1, 1, (n, 41)).astype(np.float32)
+    C0 = np.random.default_rng(2).uniform(-1, 1, (40, 41)).astype(np.float32)
+    got = run_spmm(T, m, B, alpha=0.5, beta=2.0, C0=C0)
+    ref = 0.5 * oracle.spmm_f64acc(m.indptr, m.indices, m.data, B) + 2.0 * C0
+    scale = 0.5 * oracle.spmm_f64acc(m.indptr, m.indices, np.abs(m.data), np.abs(B)) + 2.0 * np.abs(C0)
+    assert rel_err(got, ref, scale) <= 1e-4
+    a = run_spmm(T, m, B)
+    b = run_spmm(T, m, B)
+    np.testing.assert_array_equal(a, b)                             # fixed summation order: bitwise repeatable
+
+
+def test_spmm_empty_matrix_and_rows(T):
+    m = sp.csr_matrix((5, 7), dtype=np.float32)
+    got = run_spmm(T, m, np.ones((7, 16), np.float32))
+    np.testing.assert_array_equal(got, 0.0)
+
+
+@pytest.mark.parametrize("scale,ef,seed,K", [(12, 16, 3, 128), (13, 32, 5, 64)])
+def test_spmm_rmat_normalised_adjacency(T, oracle, scale, ef, seed, K):
+    """Third configuration's shape in miniature: undirected R-MAT + self-loops, sym-normalised, x U[-1,1]."""
+    from drone_amd import gcn, graphs
+    g = graphs.gcn_graph_np(scale, ef, seed)
+    H = np.random.default_rng(seed).uniform(-1, 1, (g["n"], K)).astype(np.float32)
+    m = sp.csr_matrix((g["val"], g["ci"], g["rp"]), shape=(g["n"], g["n"]))
+    got = run_spmm(T, m, H)
+    ref = oracle.spmm_f64acc(g["rp"], g["ci"], g["val"], H)
+    scale_ = oracle.spmm_f64acc(g["rp"], g["ci"], g["val"], np.abs(H))
+    assert rel_err(got, ref, scale_) <= 1e-4
+    # A_hat is symmetric: <A X, Y> == <X, A Y> (adjointness of forward and backward aggregation)
+    Y = np.random.default_rng(seed + 1).uniform(-1, 1, (g["n"], K)).astype(np.float32)
+    lhs = np.sum(got.astype(np.float64) * Y)
+    rhs = np.sum(H.astype(np.float64) * run_spmm(T, m, Y))
+    assert abs(lhs - rhs) <= 1e-4 * np.sum(np.abs(got.astype(np.float64) * Y))
+
+
+def test_edge_values_and_transpose(T, oracle):
+    from drone_amd import gcn
+    k = json.load(open(os.path.join(GOLD, "transpose_test_cu.json")))
+    rpT, ciT, vT = gcn.csr_transpose(3, 4, dev(T, np.array(k["rp"], np.int32)), dev(T, np.array(k["ci"], np.int32)),
+                                     dev(T, np.array(k["val"], np.float32)))
+    assert rpT.cpu().tolist() == k["rpT"] and ciT.cpu().tolist() == k["ciT"] and vT.cpu().tolist() == k["valT"]
+    for seed, (r, c) in enumerate([(50, 70), (400, 300), (1, 5)]):
+        m = random_csr(seed, r, c, 0.1)
+        rp, ci, v = m.indptr.astype(np.int32), m.indices.astype(np.int32), m.data
+        a = gcn.csr_transpose(r, c, dev(T, rp), dev(T, ci), dev(T, v))
+        b = oracle.csr_transpose(r, c, rp, ci, v)
+        for x, y in zip(a, b):
+            np.testing.assert_array_equal(x.cpu().numpy(), y)
+        pat = gcn.csr_transpose(r, c, dev(T, rp), dev(T, ci), None)
+        np.testing.assert_array_equal(pat[1].cpu().numpy(), b[1])
+        assert pat[2] is None
+    # edge values: exact float equality with the oracle's mixed double/float evaluation order
+    rng = np.random.default_rng(0)
+    m = random_csr(9, 500, 500, 0.05, hub=400)
+    ind = rng.integers(1, 3000, 500).astype(np.int32)
+    outd = rng.integers(1, 3000, 500).astype(np.int32)
+    got = gcn.edge_values(dev(T, m.indptr.astype(np.int32)), dev(T, m.indices.astype(np.int32)), dev(T, ind), dev(T, outd))
+    np.testing.assert_array_equal(got.cpu().numpy(), oracle.edge_values(m.indptr, m.indices, ind, outd))
+
+
+SHAPES = [(5, 7, 3), (33, 41, 70), (130, 128, 602), (257, 41, 128), (300, 130, 33), (128, 128, 16), (1, 1, 1)]
+
+
+@pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_sgemm_against_oracle(T, oracle, tA, tB, M, N, K):
+    from drone_amd import gcn
+    rng = np.random.default_rng(M * 7 + N * 3 + K + tA + 2 * tB)
+    A = rng.uniform(-1, 1, (K, M) if tA else (M, K)).astype(np.float32)
+    B = rng.uniform(-1, 1, (N, K) if tB else (K, N)).astype(np.float32)
+    got = gcn.sgemm(tA, tB, dev(T, A), dev(T, B)).cpu().numpy()
+    opA, opB = (A.T if tA else A).astype(np.float64), (B.T if tB else B).astype(np.float64)
+    assert rel_err(got, opA @ opB, np.abs(opA) @ np.abs(opB)) <= 1e-4
+    if not tA and not tB:
+        np.testing.assert_allclose(got, oracle.sgemm_f32(0, 0, A, B), rtol=1e-4, atol=1e-4)
+
+
+def test_sgemm_identity_alpha_beta_ld_and_split_reduction(T):
+    from drone_amd import gcn
+    rng = np.random.default_rng(3)
+    A = rng.uniform(-1, 1, (70, 70)).astype(np.float32)
+    P = np.eye(70, dtype=np.float32)[rng.permutation(70)]
+    np.testing.assert_array_equal(gcn.sgemm(0, 0, dev(T, P), dev(T, A)).cpu().numpy(), P @ A)
+    np.testing.assert_array_equal(gcn.sgemm(0, 1, dev(T, A), dev(T, P)).cpu().numpy(), A @ P.T)
+    # strided operands (ld > width) and alpha/beta
+    big = T.full((70, 100), 9.0, dtype=T.float32, device="cuda")
+    C0 = rng.uniform(-1, 1, (70, 70)).astype(np.float32)
+    big[:, :70] = dev(T, C0)
+    Ad = T.zeros((70, 90), dtype=T.float32, device="cuda")
+    Ad[:, :70] = dev(T, A)
+    gcn.sgemm(0, 0, Ad[:, :70], dev(T, A), out=big[:, :70], alpha=0.5, beta=2.0)
+    res = big.cpu().numpy()
+    np.testing.assert_allclose(res[:, :70], 0.5 * (A.astype(np.float64) @ A) + 2.0 * C0, rtol=1e-4, atol=1e-4)
+    assert np.all(res[:, 70:] == 9.0)
+    # weight-gradient shape: long reduction, small output -> split over the grid and summed in order
+    X = rng.normal(size=(20000, 60)).astype(np.float32)
+    G = rng.normal(size=(20000, 41)).astype(np.float32)
+    a = gcn.sgemm(1, 0, dev(T, X), dev(T, G)).cpu().numpy()
+    b = gcn.sgemm(1, 0, dev(T, X), dev(T, G)).cpu().numpy()
+    np.testing.assert_array_equal(a, b)
+    ref = X.T.astype(np.float64) @ G
+    assert rel_err(a, ref, np.abs(X.T).astype(np.float64) @ np.abs(G)) <= 1e-4
+
+
+def test_relu_dropout(T, oracle):
+    from drone_amd import gcn
+    rng = np.random.default_rng(0)
+    x = rng.normal(size=(1000, 37)).astype(np.float32)
+    x[rng.random(x.shape) < 0.1] = 0.0
+    xd = dev(T, x)
+    mask = T.zeros(x.shape, dtype=T.uint8, device="cuda")
+    gcn.relu_forward(xd, mask)
+    y, m = oracle.relu_forward(x)
+    np.testing.assert_array_equal(xd.cpu().numpy(), y)
+    np.testing.assert_array_equal(mask.cpu().numpy(), m)
+    g = rng.normal(size=x.shape).astype(np.float32)
+    gd = dev(T, g)
+    gcn.relu_backward(gd, mask)
+    np.testing.assert_array_equal(gd.cpu().numpy(), oracle.relu_backward(g, m))
+    keep = T.empty(x.shape, dtype=T.uint8, device="cuda")
+    gcn.dropout_mask(keep, seed=4, step=7, p=0.5)
+    k = keep.cpu().numpy()
+    assert abs(k.mean() - 0.5) < 0.01 and set(np.unique(k)) == {0, 1}
+    keep2 = T.empty_like(keep)
+    gcn.dropout_mask(keep2, seed=4, step=7, p=0.5)
+    assert T.equal(keep, keep2)
+    gcn.dropout_mask(keep2, seed=4, step=8, p=0.5)
+    assert not T.equal(keep, keep2)
+    xd = dev(T, x)
+    gcn.dropout_apply(xd, keep, 0.5)
+    np.testing.assert_array_equal(xd.cpu().numpy(), oracle.dropout_forward(x, k, 0.5))
+
+
+@pytest.mark.parametrize("classes,ld_pad", [(41, 0), (41, 3), (7, 0), (3, 1), (100, 0)])
+def test_cross_entropy_accuracy_argmax(T, oracle, classes, ld_pad):
+    from drone_amd import gcn
+    rng = np.random.default_rng(classes)
+    n = 3000
+    z = (rng.normal(size=(n, classes)) * 3).astype(np.float32)
+    z[5] = 1.0                                                      # a fully tied row
+    truth = rng.integers(0, classes, n).astype(np.int32)
+    truth[rng.random(n) < 0.34] = -1
+    zd = T.zeros((n, classes + ld_pad), dtype=T.float32, device="cuda")
+    zd[:, :classes] = dev(T, z)
+    gd = T.full((n, classes + ld_pad), 5.0, dtype=T.float32, device="cuda")
+    loss, cnt = gcn.cross_entropy(zd[:, :classes], dev(T, truth), grad=gd[:, :classes])
+    rl, rg, rc = oracle.cross_entropy(z, truth)
+    assert int(cnt.item()) == rc
+    np.testing.assert_allclose(loss.item(), rl, rtol=1e-5)
+    np.testing.assert_allclose(gd.cpu().numpy()[:, :classes], rg, rtol=1e-4, atol=1e-6)
+    if ld_pad:
+        assert np.all(gd.cpu().numpy()[:, classes:] == 5.0)
+    counts, pred = gcn.accuracy(zd[:, :classes], dev(T, truth), want_pred=True)
+    c = counts.cpu().numpy()
+    assert c[1] == rc and c[0] / c[1] == pytest.approx(oracle.accuracy(z, truth), abs=1e-7)
+    np.testing.assert_array_equal(pred.cpu().numpy(), oracle.argmax(z))    # identical predictions
+
+
+def test_sgd_adam(T, oracle):
+    from drone_amd import gcn
+    rng = np.random.default_rng(1)
+    w = rng.normal(size=77077).astype(np.float32)
+    g = rng.normal(size=77077).astype(np.float32)
+    wd = dev(T, w)
+    gcn.sgd_step(wd, dev(T, g), 0.01)
+    ws = w.copy()
+    oracle.sgd_step(ws, g, 0.01)
+    np.testing.assert_allclose(wd.cpu().numpy(), ws, rtol=1e-6, atol=1e-7)
+    wd, md, vd = dev(T, w), T.zeros(77077, device="cuda"), T.zeros(77077, device="cuda")
+    wa, m, v = w.copy(), np.zeros(77077, np.float32), np.zeros(77077, np.float32)
+    for t in (1, 2, 3):
+        gcn.adam_step(wd, dev(T, g), md, vd, True, 5e-4, 0.01, 0.9, 0.999, 1e-8, t)
+        oracle.adam_step(wa, g, m, v, True, 5e-4, 0.01, 0.9, 0.999, 1e-8, t)
+        np.testing.assert_allclose(wd.cpu().numpy(), wa, rtol=1e-5, atol=1e-6)
