@@ -55,6 +55,12 @@ class PRValues(C.Structure):
                 ("outDegree", C.c_void_p), ("ext", C.c_void_p)]
 
 
+class GcnConfig(C.Structure):
+    _fields_ = [("n", C.c_int), ("input_dim", C.c_int), ("hidden_dim", C.c_int), ("output_dim", C.c_int),
+                ("dropout", C.c_float), ("learning_rate", C.c_float), ("weight_decay", C.c_float),
+                ("use_dropout", C.c_int), ("use_adam", C.c_int), ("seed", C.c_uint64)]
+
+
 _lib = None
 
 _I, _I64, _U64, _D, _F, _P = C.c_int, C.c_int64, C.c_uint64, C.c_double, C.c_float, C.c_void_p
@@ -98,6 +104,17 @@ SIGNATURES = {
     "drone_sgd_step_f32": (_I, [_P, _P, _I64, _F, _P]),
     "drone_adam_step_f32": (_I, [_P, _P, _P, _P, _I64, _I, _F, _F, _F, _F, _F, _I, _P]),
     "drone_fill_f32": (_I, [_P, _I64, _F, _P]),
+    "drone_gcn_create": (_I, [C.POINTER(_P), C.POINTER(GcnConfig), _I64, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P]),
+    "drone_gcn_destroy": (_I, [_P]),
+    "drone_gcn_set_truth": (_I, [_P, _I]),
+    "drone_gcn_forward": (_I, [_P, _I]),
+    "drone_gcn_backward": (_I, [_P]),
+    "drone_gcn_optimizer_step": (_I, [_P]),
+    "drone_gcn_train_step_async": (_I, [_P]),
+    "drone_gcn_read_metrics": (_I, [_P, C.POINTER(_F), C.POINTER(_F)]),
+    "drone_gcn_train_epoch": (_I, [_P, C.POINTER(_F), C.POINTER(_F)]),
+    "drone_gcn_eval": (_I, [_P, _I, C.POINTER(_F), C.POINTER(_F)]),
+    "drone_gcn_tensor": (_I, [_P, C.c_char_p, C.POINTER(_P), C.POINTER(_I), C.POINTER(_I), C.POINTER(_I)]),
     "drone_rmat_edges": (_I, [_I, _I64, _D, _D, _D, _U64, _I64, _P, _P]),
     "drone_fill_uniform_f32": (_I, [_P, _I64, _U64, _F, _F]),
     "drone_fill_normal_f32": (_I, [_P, _I64, _U64]),

@@ -1,0 +1,178 @@
+// C handle API over the C++ module layer (include/drone_gcn_modules.hpp): what cuda_gcn exposes as
+// getHandle()/run() (cuda_gcn/src/gcn.h:10-12, gcn.cu:22-52) plus the per-epoch calls of its main loop
+// (gcn.cu:96-106 -> CUDAGCN::run_epoch, cuda_gcn.cu:356-379), so a host in any language can drive a training
+// run.  Data loading is out: the caller hands over device arrays.
+#include <cstring>
+
+#include "../../include/drone_gcn_modules.hpp"
+#include "common.h"
+
+using namespace drone;
+
+namespace {
+// cuda_kernel.cu:463-467
+__global__ void set_truth_kernel(int *__restrict__ truth, const int *__restrict__ split, const int *__restrict__ label,
+                                 int current_split, int n)
+{
+    const int id = blockIdx.x * blockDim.x + threadIdx.x;
+    if (id < n) truth[id] = split[id] == current_split ? label[id] : -1;
+}
+}  // namespace
+
+void drone_gcn_mod::GCN::set_truth(int current_split)
+{
+    const int n = params.localVertexSize;
+    set_truth_kernel<<<(n + 255) / 256, 256, 0, static_cast<hipStream_t>(s)>>>(truth, split, label, current_split, n);
+    DRONE_GCN_HIP(hipGetLastError());
+}
+
+struct drone_gcn {
+    drone_gcn_mod::GCN *model;
+};
+
+extern "C" int drone_gcn_create(struct drone_gcn **out, const drone_gcn_config *cfg, int64_t nnz, const int *rp,
+                                const int *ci, const int *in_degree, const int *out_degree, float *X, int ldx,
+                                const int *label, const int *split, const float *W1, const float *W2,
+                                drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(out && cfg, "null handle / config");
+    DRONE_REQUIRE(cfg->n > 0 && cfg->input_dim > 0 && cfg->hidden_dim > 0 && cfg->output_dim > 0, "dimensions");
+    DRONE_REQUIRE(nnz >= 0 && nnz < INT32_MAX && rp && (ci || nnz == 0) && in_degree && out_degree, "graph arrays");
+    DRONE_REQUIRE(X && ldx >= cfg->input_dim && label && split && W1 && W2, "feature / label / weight arrays");
+    DRONE_REQUIRE(cfg->dropout >= 0.0f && cfg->dropout < 1.0f, "dropout probability");
+    drone_gcn_mod::GCNParams p;
+    p.localVertexSize = cfg->n;
+    p.input_dim = cfg->input_dim;
+    p.hidden_dim = cfg->hidden_dim;
+    p.output_dim = cfg->output_dim;
+    p.dropout = cfg->dropout;
+    p.learning_rate = cfg->learning_rate;
+    p.weight_decay = cfg->weight_decay;
+    p.use_dropout = cfg->use_dropout != 0;
+    p.use_adam = cfg->use_adam != 0;
+    p.seed = cfg->seed;
+    struct drone_gcn *h = new drone_gcn();
+    h->model = new drone_gcn_mod::GCN(p, nnz, rp, ci, in_degree, out_degree, X, ldx, label, split, W1, W2, stream);
+    *out = h;
+    return DRONE_OK;
+}
+
+extern "C" int drone_gcn_destroy(struct drone_gcn *h)
+{
+    if (!h) return DRONE_OK;
+    delete h->model;
+    delete h;
+    return DRONE_OK;
+}
+
+extern "C" int drone_gcn_set_truth(struct drone_gcn *h, int split)
+{
+    clear_error();
+    DRONE_REQUIRE(h != nullptr, "handle");
+    h->model->set_truth(split);
+    return DRONE_OK;
+}
+
+extern "C" int drone_gcn_forward(struct drone_gcn *h, int training)
+{
+    clear_error();
+    DRONE_REQUIRE(h != nullptr, "handle");
+    h->model->forward(training != 0);
+    return DRONE_OK;
+}
+
+extern "C" int drone_gcn_backward(struct drone_gcn *h)
+{
+    clear_error();
+    DRONE_REQUIRE(h != nullptr, "handle");
+    h->model->backward();
+    return DRONE_OK;
+}
+
+extern "C" int drone_gcn_optimizer_step(struct drone_gcn *h)
+{
+    clear_error();
+    DRONE_REQUIRE(h != nullptr, "handle");
+    h->model->optimizer->step();
+    return DRONE_OK;
+}
+
+extern "C" int drone_gcn_train_step_async(struct drone_gcn *h)
+{
+    clear_error();
+    DRONE_REQUIRE(h != nullptr, "handle");
+    h->model->train_step_async();
+    return DRONE_OK;
+}
+
+extern "C" int drone_gcn_read_metrics(struct drone_gcn *h, float *loss, float *accuracy)
+{
+    clear_error();
+    DRONE_REQUIRE(h != nullptr, "handle");
+    const auto r = h->model->read_metrics();
+    if (loss) *loss = r.first;
+    if (accuracy) *accuracy = r.second;
+    return DRONE_OK;
+}
+
+extern "C" int drone_gcn_train_epoch(struct drone_gcn *h, float *loss, float *accuracy)
+{
+    clear_error();
+    DRONE_REQUIRE(h != nullptr, "handle");
+    const auto r = h->model->train_epoch();
+    if (loss) *loss = r.first;
+    if (accuracy) *accuracy = r.second;
+    return DRONE_OK;
+}
+
+extern "C" int drone_gcn_eval(struct drone_gcn *h, int split, float *loss, float *accuracy)
+{
+    clear_error();
+    DRONE_REQUIRE(h != nullptr, "handle");
+    const auto r = h->model->eval(split);
+    if (loss) *loss = r.first;
+    if (accuracy) *accuracy = r.second;
+    return DRONE_OK;
+}
+
+extern "C" int drone_gcn_tensor(struct drone_gcn *h, const char *name, void **ptr, int *rows, int *cols, int *ld)
+{
+    clear_error();
+    DRONE_REQUIRE(h && name && ptr, "null argument");
+    drone_gcn_mod::GCN *m = h->model;
+    struct Entry { const char *name; drone_gcn_mod::Variable *v; bool grad; };
+    const Entry table[] = {
+        {"X", m->input, false},           {"T1", m->layer1_var1, false},    {"dT1", m->layer1_var1, true},
+        {"W1", m->layer1_weight, false},  {"dW1", m->layer1_weight, true},  {"H1", m->layer1_var2, false},
+        {"dH1", m->layer1_var2, true},    {"T2", m->layer2_var1, false},    {"dT2", m->layer2_var1, true},
+        {"W2", m->layer2_weight, false},  {"dW2", m->layer2_weight, true},  {"Z", m->output, false},
+        {"dZ", m->output, true},
+    };
+    for (const Entry &e : table)
+        if (strcmp(e.name, name) == 0) {
+            *ptr = e.grad ? e.v->grad : e.v->data;
+            if (rows) *rows = e.v->rows;
+            if (cols) *cols = e.v->cols;
+            if (ld) *ld = e.v->ld;
+            return DRONE_OK;
+        }
+    const int N = m->params.localVertexSize;
+    const int64_t nnz = m->adj->nnz;
+    auto flat = [&](const void *p, int r, int c, int l) {
+        *ptr = const_cast<void *>(p);
+        if (rows) *rows = r;
+        if (cols) *cols = c;
+        if (ld) *ld = l;
+        return DRONE_OK;
+    };
+    if (!strcmp(name, "relu_mask")) return flat(m->relu->mask_ptr(), N, m->layer1_var2->cols, m->layer1_var2->ld);
+    if (!strcmp(name, "keep1") && m->drop) return flat(m->drop->keep_ptr(), N, m->layer1_var2->cols, m->layer1_var2->ld);
+    if (!strcmp(name, "truth")) return flat(m->truth, 1, N, N);
+    if (!strcmp(name, "val")) return flat(m->adj->val, 1, (int)nnz, (int)nnz);
+    if (!strcmp(name, "valT")) return flat(m->adj->valT, 1, (int)nnz, (int)nnz);
+    if (!strcmp(name, "rpT")) return flat(m->adj->rpT, 1, N + 1, N + 1);
+    if (!strcmp(name, "ciT")) return flat(m->adj->ciT, 1, (int)nnz, (int)nnz);
+    set_error(DRONE_ERR_INVALID, "drone_gcn_tensor: unknown tensor '%s'", name);
+    return DRONE_ERR_INVALID;
+}

@@ -119,3 +119,75 @@ def sgd_step(w, g, lr, stream=0):
 def adam_step(w, g, m, v, decay, weight_decay, lr, beta1, beta2, eps, step_count, stream=0):
     check(lib().drone_adam_step_f32(_ptr(w), _ptr(g), _ptr(m), _ptr(v), w.numel(), int(decay), float(weight_decay),
                                     float(lr), float(beta1), float(beta2), float(eps), int(step_count), stream))
+
+
+class GcnModel:
+    """Handle on the 2-layer GCN of cuda_gcn (CUDAGCN, cuda_gcn/src/cuda/cuda_gcn.cu:9-99,287-318) built from
+    device tensors.  rp/ci: out-edge CSR (int32), in_deg/out_deg: int32 degrees, X: float32 N x input_dim,
+    label/split: int32 (split 1 = train), W1/W2: float32 initial weights."""
+
+    def __init__(self, rp, ci, in_deg, out_deg, X, label, split, W1, W2, dropout=0.5, lr=0.01, weight_decay=5e-4,
+                 use_dropout=False, use_adam=True, seed=1234, stream=0):
+        from ._lib import GcnConfig
+        n, input_dim = X.shape
+        hidden, classes = W1.shape[1], W2.shape[1]
+        assert W1.shape[0] == input_dim and W2.shape[0] == hidden and W1.is_contiguous() and W2.is_contiguous()
+        assert X.stride(1) == 1
+        cfg = GcnConfig(n, input_dim, hidden, classes, dropout, lr, weight_decay, int(use_dropout), int(use_adam), seed)
+        self._keep = (rp, ci, in_deg, out_deg, X, label, split)
+        self.n, self.input_dim, self.hidden, self.classes = n, input_dim, hidden, classes
+        self.nnz = ci.numel()
+        h = C.c_void_p()
+        check(lib().drone_gcn_create(C.byref(h), C.byref(cfg), self.nnz, _ptr(rp), _ptr(ci), _ptr(in_deg), _ptr(out_deg),
+                                     _ptr(X), X.stride(0), _ptr(label), _ptr(split), _ptr(W1), _ptr(W2), stream))
+        self.h = h
+
+    def set_truth(self, split):
+        check(lib().drone_gcn_set_truth(self.h, int(split)))
+
+    def forward(self, training=True):
+        check(lib().drone_gcn_forward(self.h, int(training)))
+
+    def backward(self):
+        check(lib().drone_gcn_backward(self.h))
+
+    def optimizer_step(self):
+        check(lib().drone_gcn_optimizer_step(self.h))
+
+    def train_step_async(self):
+        check(lib().drone_gcn_train_step_async(self.h))
+
+    def read_metrics(self):
+        loss, acc = C.c_float(0), C.c_float(0)
+        check(lib().drone_gcn_read_metrics(self.h, C.byref(loss), C.byref(acc)))
+        return loss.value, acc.value
+
+    def train_epoch(self):
+        loss, acc = C.c_float(0), C.c_float(0)
+        check(lib().drone_gcn_train_epoch(self.h, C.byref(loss), C.byref(acc)))
+        return loss.value, acc.value
+
+    def eval(self, split):
+        loss, acc = C.c_float(0), C.c_float(0)
+        check(lib().drone_gcn_eval(self.h, int(split), C.byref(loss), C.byref(acc)))
+        return loss.value, acc.value
+
+    def tensor(self, name):
+        """Host copy (numpy) of a named tensor, logical columns only."""
+        import numpy as np
+        import torch
+        from .pagerank import lib_hip_memcpy_d2d
+        ptr, rows, cols, ld = C.c_void_p(), C.c_int(0), C.c_int(0), C.c_int(0)
+        check(lib().drone_gcn_tensor(self.h, name.encode(), C.byref(ptr), C.byref(rows), C.byref(cols), C.byref(ld)))
+        dtype = {"relu_mask": torch.uint8, "keep1": torch.uint8, "truth": torch.int32, "rpT": torch.int32,
+                 "ciT": torch.int32}.get(name, torch.float32)
+        buf = torch.empty((rows.value, ld.value), dtype=dtype, device="cuda")
+        torch.cuda.synchronize()
+        lib_hip_memcpy_d2d(buf.data_ptr(), ptr.value, buf.numel() * buf.element_size())
+        out = buf[:, :cols.value].cpu().numpy()
+        return out[0] if rows.value == 1 and name in ("truth", "rpT", "ciT", "val", "valT") else np.ascontiguousarray(out)
+
+    def close(self):
+        if self.h:
+            lib().drone_gcn_destroy(self.h)
+            self.h = None

@@ -1,0 +1,418 @@
+// C++ module layer of the 2-layer GCN, mirroring cuda_gcn's CUDAModule hierarchy
+// (cuda_gcn/src/cuda/cuda_module.cuh:31-148, cuda_variable.cuh:17-30) with every vendor call replaced by
+// the C ABI of drone_hip.h.  A maintainer of cuda_gcn can swap CUDAMatmul / CUDAGraphSum / CUDAReLU /
+// CUDADropout / CUDACrossEntropyLoss / CUDAAdam for these classes: constructor arguments keep the
+// reference's meaning (m, n, p; in/out variables; dim), forward(bool)/backward() keep its contract.
+// Differences, all forced by the single-subgraph scope: no mirror/master synchronisation after GraphSum,
+// no clearing of mirror rows before the weight gradient, no weight broadcast/reduce.
+//
+// Header-only on purpose: it holds host logic only and links against libdrone_hip.so + libamdhip64.
+#pragma once
+#include <hip/hip_runtime_api.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <memory>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "drone_hip.h"
+
+namespace drone_gcn_mod {
+
+// cuda_kernel.cuh:11-18: print and exit on failure (the reference's CUDA_CHECK contract).
+#define DRONE_GCN_CHECK(call)                                                              \
+    do {                                                                                   \
+        int rc_ = (call);                                                                  \
+        if (rc_ != 0) {                                                                    \
+            printf("drone_gcn failure %d at %s:%d: %s\n", rc_, __FILE__, __LINE__,         \
+                   drone_last_error_string());                                             \
+            exit(EXIT_FAILURE);                                                            \
+        }                                                                                  \
+    } while (0)
+#define DRONE_GCN_HIP(call)                                                                \
+    do {                                                                                   \
+        hipError_t e_ = (call);                                                            \
+        if (e_ != hipSuccess) {                                                            \
+            printf("HIP failure at %s:%d: %s\n", __FILE__, __LINE__, hipGetErrorString(e_)); \
+            exit(EXIT_FAILURE);                                                            \
+        }                                                                                  \
+    } while (0)
+
+// cuda_variable.cuh:17-30.  A row-major rows x cols matrix with leading dimension ld >= cols; ld is rounded
+// up to a multiple of 4 floats so that every row starts 16-byte aligned (the 41-class tensors get ld 44).
+// `size` keeps the reference's meaning (rows * cols logical elements).
+struct Variable {
+    float *data = nullptr, *grad = nullptr;
+    bool requires_grad, is_weight;
+    int rows, cols, ld, size;
+    bool owns_data = true;
+
+    Variable(int rows_, int cols_, bool requires_grad_ = true, bool is_weight_ = false, float *external = nullptr,
+             int external_ld = 0)
+        : requires_grad(requires_grad_), is_weight(is_weight_), rows(rows_), cols(cols_)
+    {
+        size = rows * cols;
+        if (external) {
+            data = external;
+            ld = external_ld;
+            owns_data = false;
+        } else {
+            ld = is_weight ? cols : (cols + 3) / 4 * 4;
+            DRONE_GCN_HIP(hipMalloc(&data, bytes()));
+            DRONE_GCN_HIP(hipMemset(data, 0, bytes()));
+        }
+        if (requires_grad) {
+            DRONE_GCN_HIP(hipMalloc(&grad, sizeof(float) * (size_t)rows * ld));
+            DRONE_GCN_HIP(hipMemset(grad, 0, sizeof(float) * (size_t)rows * ld));
+        }
+    }
+    Variable(const Variable &) = delete;
+    Variable &operator=(const Variable &) = delete;
+    ~Variable()
+    {
+        if (owns_data && data) (void)hipFree(data);
+        if (grad) (void)hipFree(grad);
+    }
+    size_t bytes() const { return sizeof(float) * (size_t)rows * ld; }
+};
+
+// cuda_module.cuh:31-37
+class Module {
+public:
+    virtual void forward(bool training) = 0;
+    virtual void backward() = 0;
+    virtual ~Module() {}
+    std::string ModuleName;
+};
+
+// cuda_module.cu:10-114: c(m x p) = a(m x n) * b(n x p); backward: a.grad = c.grad * b^T (if a requires grad),
+// b.grad = a^T * c.grad.
+class Matmul : public Module {
+    Variable *a, *b, *c;
+    int m, n, p;
+    drone_stream_t s;
+public:
+    Matmul(Variable *a_, Variable *b_, Variable *c_, int m_, int n_, int p_, std::string name, drone_stream_t stream)
+        : a(a_), b(b_), c(c_), m(m_), n(n_), p(p_), s(stream) { ModuleName = std::move(name); }
+    void forward(bool) override
+    {
+        DRONE_GCN_CHECK(drone_sgemm_rm_f32(0, 0, m, p, n, 1.0f, a->data, a->ld, b->data, b->ld, 0.0f, c->data, c->ld, s));
+    }
+    void backward() override
+    {
+        if (a->requires_grad)
+            DRONE_GCN_CHECK(drone_sgemm_rm_f32(0, 1, m, n, p, 1.0f, c->grad, c->ld, b->data, b->ld, 0.0f, a->grad, a->ld, s));
+        if (b->requires_grad)
+            DRONE_GCN_CHECK(drone_sgemm_rm_f32(1, 0, n, p, m, 1.0f, a->data, a->ld, c->grad, c->ld, 0.0f, b->grad, b->ld, s));
+    }
+};
+
+// The weighted adjacency shared by the GraphSum modules of one model: edge values, the transposed CSR and
+// one SpMM plan per orientation - what CUDAGraphSum's constructor builds per module (cuda_module.cu:149-202).
+struct Adjacency {
+    int n = 0;
+    int64_t nnz = 0;
+    const int *rp = nullptr, *ci = nullptr;  // out-edge CSR (borrowed, device)
+    float *val = nullptr;                    // owned
+    int *rpT = nullptr, *ciT = nullptr;      // in-edge CSR (owned)
+    float *valT = nullptr;
+    drone_spmm_plan *plan = nullptr, *planT = nullptr;
+
+    Adjacency(int n_, int64_t nnz_, const int *rp_, const int *ci_, const int *in_degree, const int *out_degree,
+              int max_dim, drone_stream_t s)
+        : n(n_), nnz(nnz_), rp(rp_), ci(ci_)
+    {
+        const size_t e = (size_t)(nnz ? nnz : 1);
+        DRONE_GCN_HIP(hipMalloc(&val, sizeof(float) * e));
+        DRONE_GCN_HIP(hipMalloc(&rpT, sizeof(int) * ((size_t)n + 1)));
+        DRONE_GCN_HIP(hipMalloc(&ciT, sizeof(int) * e));
+        DRONE_GCN_HIP(hipMalloc(&valT, sizeof(float) * e));
+        DRONE_GCN_CHECK(drone_gcn_edge_values(n, rp, ci, in_degree, out_degree, val, s));
+        DRONE_GCN_CHECK(drone_csr_transpose_f32(n, n, nnz, rp, ci, val, rpT, ciT, valT, s));
+        DRONE_GCN_CHECK(drone_spmm_plan_create(&plan, n, nnz, rp, max_dim, s));
+        DRONE_GCN_CHECK(drone_spmm_plan_create(&planT, n, nnz, rpT, max_dim, s));
+    }
+    Adjacency(const Adjacency &) = delete;
+    ~Adjacency()
+    {
+        drone_spmm_plan_destroy(plan);
+        drone_spmm_plan_destroy(planT);
+        (void)hipFree(val);
+        (void)hipFree(rpT);
+        (void)hipFree(ciT);
+        (void)hipFree(valT);
+    }
+};
+
+// cuda_module.cu:210-250 forward: out = A^T * in (pull over in-edges); :310-341 backward: in.grad = A * out.grad.
+class GraphSum : public Module {
+    Variable *in, *out;
+    Adjacency *adj;
+    int dim;
+    drone_stream_t s;
+public:
+    GraphSum(Variable *in_, Variable *out_, Adjacency *adj_, int dim_, std::string name, drone_stream_t stream)
+        : in(in_), out(out_), adj(adj_), dim(dim_), s(stream) { ModuleName = std::move(name); }
+    void forward(bool) override
+    {
+        DRONE_GCN_CHECK(drone_spmm_csr_f32(adj->planT, adj->rpT, adj->ciT, adj->valT, in->data, in->ld, out->data,
+                                           out->ld, dim, 1.0f, 0.0f, s));
+    }
+    void backward() override
+    {
+        DRONE_GCN_CHECK(drone_spmm_csr_f32(adj->plan, adj->rp, adj->ci, adj->val, out->grad, out->ld, in->grad,
+                                           in->ld, dim, 1.0f, 0.0f, s));
+    }
+};
+
+// cuda_module.cu:498-523.  The mask covers the padded rows x ld extent (padding stays zero).
+class ReLU : public Module {
+    Variable *in;
+    uint8_t *mask = nullptr;
+    drone_stream_t s;
+public:
+    ReLU(Variable *in_, std::string name, drone_stream_t stream) : in(in_), s(stream)
+    {
+        ModuleName = std::move(name);
+        DRONE_GCN_HIP(hipMalloc(&mask, (size_t)in->rows * in->ld));
+    }
+    ~ReLU() override { (void)hipFree(mask); }
+    void forward(bool training) override
+    {
+        DRONE_GCN_CHECK(drone_relu_forward_f32(in->data, mask, (int64_t)in->rows * in->ld, training, s));
+    }
+    void backward() override { DRONE_GCN_CHECK(drone_relu_backward_f32(in->grad, mask, (int64_t)in->rows * in->ld, s)); }
+    const uint8_t *mask_ptr() const { return mask; }
+};
+
+// cuda_module.cu:539-564.  The keep-mask is drawn per training step from (seed, step) by drone_dropout_mask
+// instead of the reference's shared cuRAND states; element i of the mask belongs to flat index i of the
+// rows x ld buffer.
+class Dropout : public Module {
+    Variable *in;
+    float p;
+    uint64_t seed, step = 0;
+    uint8_t *keep = nullptr;
+    drone_stream_t s;
+public:
+    Dropout(Variable *in_, float p_, uint64_t seed_, std::string name, drone_stream_t stream)
+        : in(in_), p(p_), seed(seed_), s(stream)
+    {
+        ModuleName = std::move(name);
+        DRONE_GCN_HIP(hipMalloc(&keep, (size_t)in->rows * in->ld));
+    }
+    ~Dropout() override { (void)hipFree(keep); }
+    void forward(bool training) override
+    {
+        if (!training) return;
+        const int64_t cnt = (int64_t)in->rows * in->ld;
+        DRONE_GCN_CHECK(drone_dropout_mask(keep, cnt, seed, step++, p, s));
+        DRONE_GCN_CHECK(drone_dropout_apply_f32(in->data, keep, cnt, p, s));
+    }
+    void backward() override
+    {
+        if (in->grad) DRONE_GCN_CHECK(drone_dropout_apply_f32(in->grad, keep, (int64_t)in->rows * in->ld, p, s));
+    }
+    const uint8_t *keep_ptr() const { return keep; }
+};
+
+// cuda_module.cu:406-483: writes logits->grad (sum-reduced) when training and the mean loss.
+class CrossEntropyLoss : public Module {
+    Variable *logits;
+    const int *truth;
+    int num_classes;
+    drone_stream_t s;
+public:
+    float *d_loss = nullptr;  // device scalars
+    int *d_count = nullptr;
+    CrossEntropyLoss(Variable *logits_, const int *truth_, int num_classes_, std::string name, drone_stream_t stream)
+        : logits(logits_), truth(truth_), num_classes(num_classes_), s(stream)
+    {
+        ModuleName = std::move(name);
+        DRONE_GCN_HIP(hipMalloc(&d_loss, sizeof(float)));
+        DRONE_GCN_HIP(hipMalloc(&d_count, sizeof(int)));
+    }
+    ~CrossEntropyLoss() override { (void)hipFree(d_loss); (void)hipFree(d_count); }
+    void forward(bool training) override
+    {
+        DRONE_GCN_CHECK(drone_cross_entropy_f32(logits->rows, num_classes, logits->data, logits->ld, truth,
+                                                training ? logits->grad : nullptr, logits->ld, d_loss, d_count, s));
+    }
+    void backward() override {}
+};
+
+// seq.cu:65-67 defaults; cuda_module.cu:566-600.
+struct AdamParams {
+    float lr = 0.001f, beta1 = 0.9f, beta2 = 0.999f, eps = 1e-8f, weight_decay = 0.0f;
+};
+
+class Optimizer {
+public:
+    virtual void step() = 0;
+    virtual ~Optimizer() {}
+};
+
+class Adam : public Optimizer {
+    struct Slot { Variable *var; bool decay; float *m, *v; };
+    std::vector<Slot> vars;
+    AdamParams params;
+    int step_count = 0;
+    drone_stream_t s;
+public:
+    Adam(std::vector<std::pair<Variable *, bool>> vs, AdamParams p, drone_stream_t stream) : params(p), s(stream)
+    {
+        for (auto &v : vs) {
+            Slot sl{v.first, v.second, nullptr, nullptr};
+            DRONE_GCN_HIP(hipMalloc(&sl.m, v.first->bytes()));
+            DRONE_GCN_HIP(hipMalloc(&sl.v, v.first->bytes()));
+            DRONE_GCN_HIP(hipMemset(sl.m, 0, v.first->bytes()));
+            DRONE_GCN_HIP(hipMemset(sl.v, 0, v.first->bytes()));
+            vars.push_back(sl);
+        }
+    }
+    ~Adam() override { for (auto &sl : vars) { (void)hipFree(sl.m); (void)hipFree(sl.v); } }
+    void step() override
+    {
+        step_count++;
+        for (auto &sl : vars)
+            DRONE_GCN_CHECK(drone_adam_step_f32(sl.var->data, sl.var->grad, sl.m, sl.v, (int64_t)sl.var->rows * sl.var->ld,
+                                                sl.decay, params.weight_decay, params.lr, params.beta1, params.beta2,
+                                                params.eps, step_count, s));
+    }
+};
+
+// Plain SGD (what the benchmark configuration names; the reference only ships Adam).
+class SGD : public Optimizer {
+    std::vector<Variable *> vars;
+    float lr;
+    drone_stream_t s;
+public:
+    SGD(std::vector<Variable *> vs, float lr_, drone_stream_t stream) : vars(std::move(vs)), lr(lr_), s(stream) {}
+    void step() override
+    {
+        for (auto *v : vars) DRONE_GCN_CHECK(drone_sgd_step_f32(v->data, v->grad, (int64_t)v->rows * v->ld, lr, s));
+    }
+};
+
+// seq.cu:98-100 defaults {2708, 1000, 1433, 64, 7, 0.5, 0.01, 5e-4, 5000, 0}; the fields used here.
+struct GCNParams {
+    int localVertexSize = 2708, input_dim = 1433, hidden_dim = 64, output_dim = 7;
+    float dropout = 0.5f, learning_rate = 0.01f, weight_decay = 5e-4f;
+    bool use_dropout = false;   // the reference leaves its dropout modules commented out (cuda_gcn.cu:35,64)
+    bool use_adam = true;       // reference optimiser; false = SGD
+    uint64_t seed = 1234;       // cuda_kernel.cu:426 seeds cuRAND with 1234
+};
+
+// cuda_gcn.cu:9-99 (module list) and :119-170, 287-306 (forward / backward / train_epoch).
+class GCN {
+public:
+    GCNParams params;
+    std::vector<std::unique_ptr<Variable>> variables;
+    std::vector<std::unique_ptr<Module>> modules;
+    std::unique_ptr<Adjacency> adj;
+    std::unique_ptr<Optimizer> optimizer;
+    Variable *input = nullptr, *layer1_var1 = nullptr, *layer1_weight = nullptr, *layer1_var2 = nullptr,
+             *layer2_var1 = nullptr, *layer2_weight = nullptr, *output = nullptr;
+    CrossEntropyLoss *ce = nullptr;
+    ReLU *relu = nullptr;
+    Dropout *drop = nullptr;
+    int *truth = nullptr;   // device [N]: label on rows of the current split, -1 elsewhere
+    int *counts = nullptr;  // device [2]: correct, labelled
+    const int *label = nullptr, *split = nullptr;  // device, borrowed
+    drone_stream_t s;
+
+    // X: device N x input_dim with leading dimension ldx (borrowed).  W1 / W2: device initial weights (copied).
+    GCN(const GCNParams &p, int64_t nnz, const int *rp, const int *ci, const int *in_degree, const int *out_degree,
+        float *X, int ldx, const int *label_, const int *split_, const float *W1, const float *W2, drone_stream_t stream)
+        : params(p), label(label_), split(split_), s(stream)
+    {
+        const int N = p.localVertexSize;
+        auto add = [&](Variable *v) { variables.emplace_back(v); return v; };
+        input = add(new Variable(N, p.input_dim, false, false, X, ldx));
+        layer1_var1 = add(new Variable(N, p.hidden_dim, true, false));
+        layer1_weight = add(new Variable(p.input_dim, p.hidden_dim, true, true));
+        layer1_var2 = add(new Variable(N, p.hidden_dim, true, false));
+        layer2_var1 = add(new Variable(N, p.output_dim, true, false));
+        layer2_weight = add(new Variable(p.hidden_dim, p.output_dim, true, true));
+        output = add(new Variable(N, p.output_dim, true, false));
+        DRONE_GCN_HIP(hipMemcpy(layer1_weight->data, W1, layer1_weight->bytes(), hipMemcpyDeviceToDevice));
+        DRONE_GCN_HIP(hipMemcpy(layer2_weight->data, W2, layer2_weight->bytes(), hipMemcpyDeviceToDevice));
+        const int max_dim = p.hidden_dim > p.output_dim ? p.hidden_dim : p.output_dim;
+        adj.reset(new Adjacency(N, nnz, rp, ci, in_degree, out_degree, max_dim, s));
+        DRONE_GCN_HIP(hipMalloc(&truth, sizeof(int) * (size_t)N));
+        DRONE_GCN_HIP(hipMalloc(&counts, sizeof(int) * 2));
+
+        modules.emplace_back(new Matmul(input, layer1_weight, layer1_var1, N, p.input_dim, p.hidden_dim, "matmul_layer1", s));
+        modules.emplace_back(new GraphSum(layer1_var1, layer1_var2, adj.get(), p.hidden_dim, "graphSum_layer1", s));
+        relu = new ReLU(layer1_var2, "Relu", s);
+        modules.emplace_back(relu);
+        if (p.use_dropout) {
+            drop = new Dropout(layer1_var2, p.dropout, p.seed, "dropout_layer1", s);
+            modules.emplace_back(drop);
+        }
+        modules.emplace_back(new Matmul(layer1_var2, layer2_weight, layer2_var1, N, p.hidden_dim, p.output_dim, "matmul_layer2", s));
+        modules.emplace_back(new GraphSum(layer2_var1, output, adj.get(), p.output_dim, "graphSum_layer2", s));
+        ce = new CrossEntropyLoss(output, truth, p.output_dim, "CrossEntropy", s);
+        modules.emplace_back(ce);
+        if (p.use_adam) {
+            AdamParams ap;
+            ap.lr = p.learning_rate;
+            ap.weight_decay = p.weight_decay;
+            optimizer.reset(new Adam({{layer1_weight, true}, {layer2_weight, false}}, ap, s));  // cuda_gcn.cu:89
+        } else {
+            optimizer.reset(new SGD({layer1_weight, layer2_weight}, p.learning_rate, s));
+        }
+        DRONE_GCN_HIP(hipDeviceSynchronize());
+    }
+    GCN(const GCN &) = delete;
+    ~GCN()
+    {
+        (void)hipFree(truth);
+        (void)hipFree(counts);
+    }
+
+    void set_truth(int current_split);  // cuda_gcn.cu:211-223; defined in gcn_model.hip (needs a kernel)
+    void forward(bool training) { for (auto &m : modules) m->forward(training); }
+    void backward() { for (int i = (int)modules.size() - 1; i >= 0; --i) modules[i]->backward(); }
+
+    // Enqueues one training step (cuda_gcn.cu:287-306 without the host read-backs): forward, accuracy counts,
+    // backward, optimiser.  Loss and counts stay on the device until read_metrics().
+    void train_step_async()
+    {
+        forward(true);
+        DRONE_GCN_HIP(hipMemsetAsync(counts, 0, sizeof(int) * 2, static_cast<hipStream_t>(s)));
+        DRONE_GCN_CHECK(drone_accuracy_f32(params.localVertexSize, params.output_dim, output->data, output->ld, truth,
+                                           nullptr, counts, s));
+        backward();
+        optimizer->step();
+    }
+    std::pair<float, float> read_metrics()
+    {
+        float loss = 0.0f;
+        int c[2] = {0, 0};
+        DRONE_GCN_HIP(hipStreamSynchronize(static_cast<hipStream_t>(s)));
+        DRONE_GCN_HIP(hipMemcpy(&loss, ce->d_loss, sizeof(float), hipMemcpyDeviceToHost));
+        DRONE_GCN_HIP(hipMemcpy(c, counts, sizeof(int) * 2, hipMemcpyDeviceToHost));
+        return {loss, c[1] ? (float)c[0] / (float)c[1] : 0.0f};
+    }
+    std::pair<float, float> train_epoch()
+    {
+        set_truth(1);
+        train_step_async();
+        return read_metrics();
+    }
+    std::pair<float, float> eval(int current_split)  // cuda_gcn.cu:308-318
+    {
+        set_truth(current_split);
+        forward(false);
+        DRONE_GCN_HIP(hipMemsetAsync(counts, 0, sizeof(int) * 2, static_cast<hipStream_t>(s)));
+        DRONE_GCN_CHECK(drone_accuracy_f32(params.localVertexSize, params.output_dim, output->data, output->ld, truth,
+                                           nullptr, counts, s));
+        return read_metrics();
+    }
+};
+
+}  // namespace drone_gcn_mod

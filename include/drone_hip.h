@@ -209,6 +209,40 @@ int drone_adam_step_f32(float *w, const float *g, float *m, float *v, int64_t n,
                         drone_stream_t stream);
 int drone_fill_f32(float *x, int64_t n, float value, drone_stream_t stream);
 
+/* ---- whole-model handle: the C surface of cuda_gcn (cuda_gcn/src/gcn.h:10-12 getHandle/run, and the
+ * epoch loop of gcn.cu:96-106 / cuda_gcn.cu:287-318,356-379) over the C++ module layer in
+ * drone_gcn_modules.hpp.  The caller hands over device arrays (the reference's file parser is not part
+ * of this path): out-edge CSR, global in/out degrees, features X (N x input_dim, leading dimension ldx,
+ * borrowed for the handle's lifetime), labels, split ids (1 = train as in cuda_gcn.cu:289), and initial
+ * weights W1 (input_dim x hidden) / W2 (hidden x output), which are copied.  Failures inside the module
+ * layer print and exit, as the reference does (cuda_kernel.cuh:11-18). */
+typedef struct drone_gcn drone_gcn;
+typedef struct drone_gcn_config {
+    int n, input_dim, hidden_dim, output_dim;
+    float dropout, learning_rate, weight_decay; /* seq.cu:98-100 defaults: 0.5, 0.01, 5e-4 */
+    int use_dropout; /* 0 = as the reference runs (its dropout modules are commented out, cuda_gcn.cu:35,64);
+                        1 = dropout(p) after the hidden ReLU */
+    int use_adam;    /* 1 = Adam as in the reference (cuda_gcn.cu:86-89); 0 = SGD */
+    uint64_t seed;   /* dropout mask stream */
+} drone_gcn_config;
+int drone_gcn_create(drone_gcn **handle, const drone_gcn_config *cfg, int64_t nnz, const int *rp, const int *ci,
+                     const int *in_degree, const int *out_degree, float *X, int ldx, const int *label,
+                     const int *split, const float *W1, const float *W2, drone_stream_t stream);
+int drone_gcn_destroy(drone_gcn *handle);
+int drone_gcn_set_truth(drone_gcn *handle, int split);   /* cuda_gcn.cu:211-223 */
+int drone_gcn_forward(drone_gcn *handle, int training);  /* cuda_gcn.cu:119-144 */
+int drone_gcn_backward(drone_gcn *handle);               /* cuda_gcn.cu:146-170 */
+int drone_gcn_optimizer_step(drone_gcn *handle);         /* cuda_gcn.cu:303 */
+/* forward(training) + accuracy counts + backward + optimiser step, enqueued without host synchronisation;
+ * drone_gcn_read_metrics waits and returns the mean training loss and accuracy of the last step. */
+int drone_gcn_train_step_async(drone_gcn *handle);
+int drone_gcn_read_metrics(drone_gcn *handle, float *loss, float *accuracy);
+int drone_gcn_train_epoch(drone_gcn *handle, float *loss, float *accuracy);     /* cuda_gcn.cu:287-306 */
+int drone_gcn_eval(drone_gcn *handle, int split, float *loss, float *accuracy); /* cuda_gcn.cu:308-318 */
+/* Device pointer and shape of a named tensor: X T1 dT1 W1 dW1 H1 dH1 T2 dT2 W2 dW2 Z dZ (float),
+ * relu_mask keep1 (uint8), truth rpT ciT (int), val valT (float). */
+int drone_gcn_tensor(drone_gcn *handle, const char *name, void **ptr, int *rows, int *cols, int *ld);
+
 /* ====================================================================================== */
 /* D. Utilities                                                                           */
 /* ====================================================================================== */

@@ -1,0 +1,159 @@
+"""GPU parity of the 2-layer GCN training step (module layer + C handle API) against the CPU oracle.
+Tolerance: outputs and gradients within 1e-4 of the oracle relative to the tensor's largest magnitude
+(fp32, summation order differs between the wavefront kernels and the oracle's serial loops); arg-max predictions
+identical; masks, counts and the CSR transpose exact."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+@pytest.fixture(scope="module")
+def T():
+    import torch
+    assert torch.cuda.is_available()
+    return torch
+
+
+def dev(T, a, dtype=None):
+    a = np.ascontiguousarray(a if dtype is None else np.asarray(a, dtype))
+    return T.from_numpy(a).cuda()
+
+
+def close(got, ref, tol=1e-4):
+    scale = max(np.abs(ref).max(), 1e-30)
+    err = np.abs(got.astype(np.float64) - ref.astype(np.float64)).max() / scale
+    assert err <= tol, f"max error {err:.3e} of scale {scale:.3e}"
+
+
+def make_model(T, g, X, W1, W2, label, split, **kw):
+    from drone_amd.gcn import GcnModel
+    deg = dev(T, g["deg"], np.int32)
+    return GcnModel(dev(T, g["rp"], np.int32), dev(T, g["ci"], np.int32), deg, deg, dev(T, X, np.float32),
+                    dev(T, label, np.int32), dev(T, split, np.int32), dev(T, W1, np.float32), dev(T, W2, np.float32), **kw)
+
+
+def oracle_step(oracle, g, X, W1, W2, truth, keep=None, p=0.5):
+    rpT, ciT, vT = oracle.csr_transpose(g["n"], g["n"], g["rp"], g["ci"], g["val"])
+    return oracle.gcn_forward_backward(g["rp"], g["ci"], g["val"], rpT, ciT, vT, X, W1, W2, truth, keep, p)
+
+
+@pytest.mark.parametrize("use_dropout", [False, True])
+def test_tiny_fixture_step(T, oracle, use_dropout):
+    d = {k: np.array(v) for k, v in json.load(open(os.path.join(GOLD, "gcn_tiny_step.json"))).items()}
+    n = 6
+    deg = np.diff(d["rp"]).astype(np.int32)
+    g = dict(n=n, rp=d["rp"], ci=d["ci"], val=d["val"].astype(np.float32), deg=deg)
+    truth = d["truth"].astype(np.int32)
+    split = np.where(truth >= 0, 1, 2).astype(np.int32)
+    label = np.maximum(truth, 0)
+    m = make_model(T, g, d["X"], d["W1"], d["W2"], label, split, use_dropout=use_dropout, use_adam=False, lr=0.01, seed=5)
+    np.testing.assert_array_equal(m.tensor("val"), oracle.edge_values(g["rp"], g["ci"], deg, deg))
+    m.set_truth(1)
+    np.testing.assert_array_equal(m.tensor("truth"), truth)
+    m.forward(True)
+    m.backward()
+    keep = m.tensor("keep1") if use_dropout else None
+    ref = oracle_step(oracle, g, d["X"], d["W1"], d["W2"], truth, keep, 0.5)
+    for name, key in (("Z", "Z"), ("H1", "H1"), ("dW1", "dW1"), ("dW2", "dW2"), ("dT1", "dT1")):
+        close(m.tensor(name), ref[key])
+    loss, acc = m.read_metrics()
+    assert loss == pytest.approx(ref["loss"], rel=1e-5)
+    m.optimizer_step()
+    W1n = d["W1"].astype(np.float32).copy()
+    oracle.sgd_step(W1n, ref["dW1"], 0.01)
+    close(m.tensor("W1"), W1n, 1e-6)
+    m.close()
+
+
+@pytest.mark.parametrize("scale,ef,fin,hid,cls,use_dropout", [(10, 8, 50, 16, 7, False), (11, 16, 602, 128, 41, True)])
+def test_rmat_step_against_oracle(T, oracle, scale, ef, fin, hid, cls, use_dropout):
+    """Second case keeps the fourth configuration's widths (602 -> 128 -> 41, dropout 0.5, SGD 0.01, 66 % train)."""
+    from drone_amd import graphs, rmat
+    g = graphs.gcn_graph_np(scale, ef, seed=4)
+    n = g["n"]
+    X = rmat.normal_f32((n, fin), seed=4)
+    lim1, lim2 = np.sqrt(6.0 / (fin + hid)), np.sqrt(6.0 / (hid + cls))
+    W1 = rmat.uniform_f32((fin, hid), seed=41, lo=-lim1, hi=lim1)
+    W2 = rmat.uniform_f32((hid, cls), seed=42, lo=-lim2, hi=lim2)
+    label = rmat.randint_i32(n, seed=43, bound=cls)
+    split = np.where(rmat.uniform_f32(n, seed=44, lo=0, hi=1) < 0.66, 1, 2).astype(np.int32)
+    truth = np.where(split == 1, label, -1).astype(np.int32)
+    m = make_model(T, g, X, W1, W2, label, split, use_dropout=use_dropout, use_adam=False, lr=0.01, seed=4)
+    # set-up products: edge values and the transposed CSR are exact
+    np.testing.assert_array_equal(m.tensor("val"), g["val"])
+    rpT, ciT, vT = oracle.csr_transpose(n, n, g["rp"], g["ci"], g["val"])
+    np.testing.assert_array_equal(m.tensor("rpT"), rpT)
+    np.testing.assert_array_equal(m.tensor("ciT"), ciT)
+    np.testing.assert_array_equal(m.tensor("valT"), vT)
+    m.set_truth(1)
+    m.train_step_async()
+    loss, acc = m.read_metrics()
+    keep = m.tensor("keep1") if use_dropout else None
+    if use_dropout:
+        assert abs(keep.mean() - 0.5) < 0.02
+    ref = oracle.gcn_forward_backward(g["rp"], g["ci"], g["val"], rpT, ciT, vT, X, W1, W2, truth, keep, 0.5)
+    close(m.tensor("Z"), ref["Z"])
+    close(m.tensor("H1"), ref["H1"])
+    close(m.tensor("dW1"), ref["dW1"])
+    close(m.tensor("dW2"), ref["dW2"])
+    close(m.tensor("dT1"), ref["dT1"])
+    assert loss == pytest.approx(ref["loss"], rel=1e-4)
+    assert acc == pytest.approx(oracle.accuracy(ref["Z"], truth), abs=2.0 / n)
+    # identical arg-max predictions
+    from drone_amd import gcn
+    Zd = dev(T, m.tensor("Z"))
+    _, pred = gcn.accuracy(Zd, dev(T, truth), want_pred=True)
+    pg, po = pred.cpu().numpy(), oracle.argmax(ref["Z"])
+    differ = np.nonzero(pg != po)[0]
+    for i in differ:            # a flip is only tolerable on a numerical tie of the two top logits
+        z = ref["Z"][i]
+        assert abs(z[pg[i]] - z[po[i]]) <= 1e-4 * np.abs(z).max()
+    assert len(differ) <= n // 1000
+    # SGD update
+    W1n, W2n = W1.copy(), W2.copy()
+    oracle.sgd_step(W1n, ref["dW1"], 0.01)
+    oracle.sgd_step(W2n, ref["dW2"], 0.01)
+    close(m.tensor("W1"), W1n, 1e-5)
+    close(m.tensor("W2"), W2n, 1e-5)
+    m.close()
+
+
+def test_training_reduces_loss_with_adam_and_eval_is_pure(T, oracle):
+    from drone_amd import graphs, rmat
+    g = graphs.gcn_graph_np(9, 8, seed=3)
+    n, fin, hid, cls = g["n"], 24, 16, 5
+    rng = np.random.default_rng(0)
+    label = rng.integers(0, cls, n).astype(np.int32)
+    X = (np.eye(cls, dtype=np.float32)[label] @ rng.normal(size=(cls, fin)).astype(np.float32)
+         + 0.5 * rng.normal(size=(n, fin)).astype(np.float32))
+    W1 = rmat.uniform_f32((fin, hid), seed=1, lo=-0.3, hi=0.3)
+    W2 = rmat.uniform_f32((hid, cls), seed=2, lo=-0.3, hi=0.3)
+    split = np.where(rng.random(n) < 0.66, 1, 2).astype(np.int32)
+    m = make_model(T, g, X, W1, W2, label, split, use_dropout=False, use_adam=True, lr=0.01, weight_decay=5e-4)
+    first = m.train_epoch()
+    # Adam step 1 against the oracle (weight decay on W1 only, cuda_gcn.cu:89)
+    truth = np.where(split == 1, label, -1).astype(np.int32)
+    ref = oracle_step(oracle, g, X, W1, W2, truth)
+    W1a, m1, v1 = W1.copy(), np.zeros_like(W1), np.zeros_like(W1)
+    oracle.adam_step(W1a, ref["dW1"], m1, v1, True, 5e-4, 0.01, 0.9, 0.999, 1e-8, 1)
+    W2a, m2, v2 = W2.copy(), np.zeros_like(W2), np.zeros_like(W2)
+    oracle.adam_step(W2a, ref["dW2"], m2, v2, False, 5e-4, 0.01, 0.9, 0.999, 1e-8, 1)
+    # Adam's first step is lr * sign(g) wherever |g| >> eps, so weights agree tightly except where the
+    # gradient is numerically zero
+    big1, big2 = np.abs(ref["dW1"]) > 1e-3 * np.abs(ref["dW1"]).max(), np.abs(ref["dW2"]) > 1e-3 * np.abs(ref["dW2"]).max()
+    np.testing.assert_allclose(m.tensor("W1")[big1], W1a[big1], rtol=1e-4, atol=1e-6)
+    np.testing.assert_allclose(m.tensor("W2")[big2], W2a[big2], rtol=1e-4, atol=1e-6)
+    for _ in range(60):
+        last = m.train_epoch()
+    assert last[0] < 0.6 * first[0] and last[1] > first[1]
+    w_before = m.tensor("W1")
+    e1 = m.eval(2)
+    e2 = m.eval(2)
+    assert e1 == e2 and e1[1] > 1.0 / cls + 0.1
+    np.testing.assert_array_equal(m.tensor("W1"), w_before)
+    m.close()
