@@ -19,6 +19,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# R-MAT candidates drawn for configs[3]: after rejecting ids >= 232,965, self-loops and duplicates this leaves
+# about 114.6 M undirected edges (the figure the configuration names); the exact count is printed and reported.
+C4_CANDIDATES = 221_000_000
 
 
 def log(*a):
@@ -32,17 +35,17 @@ def cpu_baselines(x_host, alpha, threads):
     from oracle import oracle as orc
     from drone_amd import rmat
     orc.build()
-    iters = 3
     t0 = time.time()
-    orc.pr_pull_f64(x_host["row_ptr"], x_host["col_idx"], x_host["inv_outdeg"], alpha, 1, threads)  # warm-up
+    orc.pr_pull_f64(x_host["row_ptr"], x_host["col_idx"], x_host["inv_outdeg"], alpha, 2, threads)  # warm-up
     warm = time.time() - t0
+    iters = max(3, min(200, int(12.0 / max(warm / 2, 1e-3))))   # about 12 s of CPU work
     t0 = time.time()
     orc.pr_pull_f64(x_host["row_ptr"], x_host["col_idx"], x_host["inv_outdeg"], alpha, iters, threads)
     dt = time.time() - t0
     nnz = len(x_host["col_idx"])
     pull = dict(value=nnz * iters / dt / 1e9, unit="GTEPS", cores=threads, kind="port",
                 sample=f"oracle fp64 pull PageRank (OpenMP) on the same scale-24 CSR, {iters} iterations "
-                       f"({dt:.1f} s, after a {warm:.1f} s one-iteration warm-up)")
+                       f"({dt:.1f} s, after a {warm:.1f} s two-iteration warm-up)")
     c1 = rmat.pagerank_inputs_np(16, 16, 1)
     g = orc.GoPR(c1["src"], c1["dst"], c1["outdeg"])
     t0 = time.time()
@@ -58,6 +61,167 @@ def cpu_baselines(x_host, alpha, threads):
     return pull, go
 
 
+class EventTimer:
+    """HIP-event stopwatch on a given stream (the library's drone_timer_* entry points)."""
+
+    def __init__(self, stream=0):
+        import ctypes as C
+        from drone_amd._lib import check, lib
+        self.C, self.check, self.lib, self.stream = C, check, lib(), stream
+        self.h = C.c_void_p()
+        check(self.lib.drone_timer_create(C.byref(self.h)))
+
+    def start(self):
+        self.check(self.lib.drone_timer_start(self.h, self.stream))
+
+    def stop_ms(self):
+        ms = self.C.c_float(0)
+        self.check(self.lib.drone_timer_stop(self.h, self.stream))
+        self.check(self.lib.drone_timer_elapsed_ms(self.h, self.C.byref(ms)))
+        return ms.value
+
+
+def time_call(fn, reps, warmup=1):
+    """Mean milliseconds of fn() over reps launches, HIP events on the null stream."""
+    t = EventTimer()
+    for _ in range(warmup):
+        fn()
+    t.start()
+    for _ in range(reps):
+        fn()
+    return t.stop_ms() / reps
+
+
+def spmm_report(name, n, nnz, K, ms):
+    from drone_amd._lib import lib
+    b = lib().drone_spmm_bytes(n, nnz, K)
+    gbs = b / (ms * 1e-3) / 1e9
+    gather = (8 * nnz + 4 * nnz * K + 4 * n * K) / (ms * 1e-3) / 1e9
+    return {"kernel": name, "K": K, "ms": ms, "algorithmic_bytes": b, "achieved_GBps": gbs,
+            "frac_of_hbm_peak": gbs / HBM_PEAK_GBS, "gather_inclusive_GBps": gather,
+            "gflops": 2.0 * nnz * K / (ms * 1e-3) / 1e9}
+
+
+def bench_gcn_step(steps, warmup):
+    """configs[3]: 2-layer GCN training step on the dense power-law graph (232,965 vertices)."""
+    import numpy as np
+    import torch
+    from drone_amd import gcn, graphs, rmat
+    N, FIN, HID, CLS = 232965, 602, 128, 41
+    t0 = time.time()
+    g = graphs.gcn_graph_torch(18, 0, seed=4, n=N, n_edges=C4_CANDIDATES)
+    nnz = g["nnz"]
+    X = torch.from_numpy(rmat.normal_f32((N, FIN), seed=4)).cuda()
+    l1, l2 = (6.0 / (FIN + HID)) ** 0.5, (6.0 / (HID + CLS)) ** 0.5
+    W1 = torch.from_numpy(rmat.uniform_f32((FIN, HID), seed=41, lo=-l1, hi=l1)).cuda()
+    W2 = torch.from_numpy(rmat.uniform_f32((HID, CLS), seed=42, lo=-l2, hi=l2)).cuda()
+    label = torch.from_numpy(rmat.randint_i32(N, seed=43, bound=CLS)).cuda()
+    split = torch.from_numpy(np.where(rmat.uniform_f32(N, seed=44, lo=0, hi=1) < 0.66, 1, 2).astype(np.int32)).cuda()
+    torch.cuda.synchronize()
+    log(f"GCN graph: N={N} nnz={nnz} (undirected R-MAT seed 4 + self-loops), max degree {int(g['deg'].max())}, "
+        f"inputs built in {time.time()-t0:.1f} s")
+    t0 = time.time()
+    model = gcn.GcnModel(g["rp"], g["ci"], g["deg"], g["deg"], X, label, split, W1, W2, dropout=0.5, lr=0.01,
+                         use_dropout=True, use_adam=False, mean_gradient=True, seed=4)
+    torch.cuda.synchronize()
+    setup_s = time.time() - t0
+    model.set_truth(1)
+    for _ in range(warmup):
+        model.train_step_async()
+    loss0, _ = model.read_metrics()
+    t = EventTimer()
+    t.start()
+    for _ in range(steps):
+        model.train_step_async()
+    step_ms = t.stop_ms() / steps
+    loss1, acc1 = model.read_metrics()
+    log(f"GCN step: {step_ms:.2f} ms (loss {loss0:.4f} -> {loss1:.4f}, train acc {acc1:.3f}); set-up (edge values, "
+        f"transpose, plans) {setup_s*1e3:.0f} ms one-off")
+    # the four SpMMs of the step, timed alone on operands of the same shape
+    rp, ci = g["rp"], g["ci"]
+    val = gcn.edge_values(rp, ci, g["deg"], g["deg"])
+    plan = gcn.SpmmPlan(rp, nnz, max_k=HID)
+    kernels = []
+    for K, ld in ((HID, HID), (CLS, 44)):
+        B = torch.rand((N, ld), device="cuda") * 2 - 1
+        out = torch.empty((N, ld), device="cuda")
+        ms = time_call(lambda: gcn.spmm(plan, rp, ci, val, B[:, :K], K=K, out=out[:, :K]), reps=5)
+        kernels.append(spmm_report(f"spmm_rows_kernel K={K}", N, nnz, K, ms))
+    spmm_ms = 2 * sum(k["ms"] for k in kernels)
+    spmm_bytes = 2 * sum(k["algorithmic_bytes"] for k in kernels)
+    gemms = []
+    for (tA, tB, M, Nn, Kk, what) in ((0, 0, N, HID, FIN, "X*W1"), (0, 0, N, CLS, HID, "H1*W2"), (0, 1, N, HID, CLS, "dT2*W2^T"),
+                                      (1, 0, HID, CLS, N, "H1^T*dT2"), (1, 0, FIN, HID, N, "X^T*dT1")):
+        A = torch.rand((Kk, M) if tA else (M, Kk), device="cuda")
+        Bm = torch.rand((Nn, Kk) if tB else (Kk, Nn), device="cuda")
+        out = torch.empty((M, Nn), device="cuda")
+        ms = time_call(lambda: gcn.sgemm(tA, tB, A, Bm, out=out), reps=5)
+        fl = 2.0 * M * Nn * Kk
+        gemms.append({"gemm": what, "M": M, "N": Nn, "K": Kk, "ms": ms, "tflops": fl / (ms * 1e-3) / 1e12,
+                      "frac_of_fp32_mfma_peak": fl / (ms * 1e-3) / 1e12 / 157.3})
+    plan.close()
+    model.close()
+    return {"workload": f"2-layer GCN training step (configs[3]): N={N}, nnz={nnz}, 602->128->41, ReLU, dropout 0.5, "
+                        "softmax cross-entropy, SGD lr 0.01, fp32",
+            "step_ms": step_ms, "steps": steps, "setup_ms_one_off": setup_s * 1e3, "spmm_kernels": kernels,
+            "spmm_ms_per_step": spmm_ms,
+            "spmm_frac_of_hbm_peak": spmm_bytes / (spmm_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "gemms": gemms}
+
+
+def bench_gcn_layer():
+    """configs[2]: one GCN layer forward ReLU(A_hat * (H * W)), R-MAT scale 20."""
+    import torch
+    from drone_amd import gcn, graphs, rmat
+    g = graphs.gcn_graph_torch(20, 16, seed=3)
+    N, nnz, K = g["n"], g["nnz"], 128
+    val = gcn.edge_values(g["rp"], g["ci"], g["deg"], g["deg"])
+    H = torch.from_numpy(rmat.uniform_f32((N, K), seed=3)).cuda()
+    lim = (6.0 / 256) ** 0.5
+    W = torch.from_numpy(rmat.uniform_f32((K, K), seed=33, lo=-lim, hi=lim)).cuda()
+    T1 = torch.empty((N, K), device="cuda")
+    out = torch.empty((N, K), device="cuda")
+    mask = torch.empty((N, K), dtype=torch.uint8, device="cuda")
+    plan = gcn.SpmmPlan(g["rp"], nnz, max_k=K)
+
+    def layer():
+        gcn.sgemm(0, 0, H, W, out=T1)
+        gcn.spmm(plan, g["rp"], g["ci"], val, T1, out=out)
+        gcn.relu_forward(out, mask, training=False)
+
+    ms = time_call(layer, reps=10)
+    ms_spmm = time_call(lambda: gcn.spmm(plan, g["rp"], g["ci"], val, T1, out=out), reps=10)
+    ms_gemm = time_call(lambda: gcn.sgemm(0, 0, H, W, out=T1), reps=10)
+    plan.close()
+    return {"workload": f"GCN layer forward (configs[2]): R-MAT scale 20 undirected + self-loops, N={N}, nnz={nnz}, K=128",
+            "layer_ms": ms, "spmm": spmm_report("spmm_rows_kernel K=128", N, nnz, K, ms_spmm),
+            "gemm_ms": ms_gemm, "gemm_tflops": 2.0 * N * K * K / (ms_gemm * 1e-3) / 1e12}
+
+
+def bench_spmm_sweep():
+    """configs[4]: skew-stress SpMM sweep, R-MAT scale 22 ef 32 a/b/c = .70/.12/.12, row-normalised, K in 16/64/256,
+    forward (A*H) and transpose (A^T*G)."""
+    import torch
+    from drone_amd import gcn, rmat
+    x = rmat.pagerank_inputs_torch(22, 32, 5, a=0.70, b=0.12, c=0.12)     # in-edge CSR of the directed graph
+    N, nnz = x["n"], x["nnz"]
+    rp = x["row_ptr"].to(torch.int32)
+    ci = x["col_idx"]
+    deg = (rp[1:] - rp[:-1]).clamp(min=1)
+    val = (1.0 / torch.repeat_interleave(deg.float(), (rp[1:] - rp[:-1]).long())).contiguous()
+    rpT, ciT, vT = gcn.csr_transpose(N, N, rp, ci, val)
+    out = {"workload": f"SpMM sweep (configs[4]): R-MAT scale 22 ef 32 skewed, N={N}, nnz={nnz}, max row "
+                       f"{int((rp[1:]-rp[:-1]).max())}, max transposed row {int((rpT[1:]-rpT[:-1]).max())}", "kernels": []}
+    for K in (16, 64, 256):
+        H = torch.rand((N, K), device="cuda") * 2 - 1
+        C_ = torch.empty((N, K), device="cuda")
+        for name, (a, b, c) in (("forward A*H", (rp, ci, val)), ("transpose A^T*G", (rpT, ciT, vT))):
+            plan = gcn.SpmmPlan(a, nnz, max_k=K)
+            ms = time_call(lambda: gcn.spmm(plan, a, b, c, H, out=C_), reps=5)
+            plan.close()
+            out["kernels"].append(spmm_report(f"{name} K={K}", N, nnz, K, ms))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -66,6 +230,11 @@ def main():
     ap.add_argument("--scale", type=int, default=24, help="R-MAT scale (24 = the benchmark configuration)")
     ap.add_argument("--iters", type=int, default=50)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="launch the 1 GiB stream-copy kernel exactly once (a dispatch of known traffic to scale "
+                         "rocprofv3 byte counters by)")
+    ap.add_argument("--suite", default="default", choices=["pr", "default", "full"],
+                    help="pr: PageRank only; default: + GCN training step (configs[3]); full: + configs[2] and [4]")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs one subgraph on ONE GPU; there is no multi-GPU path to time "
@@ -78,6 +247,15 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
     torch.cuda.set_device(0)
     alpha = 0.85
+    from drone_amd._lib import check, lib
+    a = torch.ones(1 << 27, dtype=torch.float64, device="cuda")      # 1 GiB
+    b = torch.empty_like(a)
+    copy_ms = time_call(lambda: check(lib().drone_stream_copy_f64(b.data_ptr(), a.data_ptr(), a.numel(), 0)),
+                        reps=1 if args.calibrate_copy else 5, warmup=0 if args.calibrate_copy else 1)
+    copy_gbs = 2 * a.numel() * 8 / (copy_ms * 1e-3) / 1e9
+    log(f"stream copy 1 GiB -> 1 GiB: {copy_ms:.3f} ms = {copy_gbs:.0f} GB/s (measured HBM stream rate, for reference)")
+    del a, b
+    torch.cuda.empty_cache()
 
     t0 = time.time()
     x = rmat.pagerank_inputs_torch(args.scale, 16, 2)
@@ -125,6 +303,7 @@ def main():
                      "algorithmic_bytes_per_launch": bytes_iter, "mean_launch_ms": prof["mean_ms"],
                      "launches_timed": prof["launches"]},
         "plan_ms_one_off": plan_s * 1e3,
+        "stream_copy_GBps_measured": copy_gbs,
     }
     if not args.no_cpu_baseline:
         x_host = {k: x[k].cpu().numpy() for k in ("row_ptr", "col_idx", "inv_outdeg")}
@@ -135,6 +314,15 @@ def main():
         result["cpu_baseline"] = pull
         result["cpu_baseline_drone_go_path"] = go
     plan.close()
+    del x, out, plan
+    torch.cuda.empty_cache()
+    if args.suite in ("default", "full"):
+        result["gcn_step"] = bench_gcn_step(steps=max(3, args.steps), warmup=max(1, args.warmup))
+        torch.cuda.empty_cache()
+    if args.suite == "full":
+        result["gcn_layer"] = bench_gcn_layer()
+        torch.cuda.empty_cache()
+        result["spmm_sweep"] = bench_spmm_sweep()
     print(json.dumps(result), flush=True)
 
 

@@ -58,7 +58,7 @@ class PRValues(C.Structure):
 class GcnConfig(C.Structure):
     _fields_ = [("n", C.c_int), ("input_dim", C.c_int), ("hidden_dim", C.c_int), ("output_dim", C.c_int),
                 ("dropout", C.c_float), ("learning_rate", C.c_float), ("weight_decay", C.c_float),
-                ("use_dropout", C.c_int), ("use_adam", C.c_int), ("seed", C.c_uint64)]
+                ("use_dropout", C.c_int), ("use_adam", C.c_int), ("mean_gradient", C.c_int), ("seed", C.c_uint64)]
 
 
 _lib = None
@@ -99,7 +99,7 @@ SIGNATURES = {
     "drone_relu_backward_f32": (_I, [_P, _P, _I64, _P]),
     "drone_dropout_mask": (_I, [_P, _I64, _U64, _U64, _F, _P]),
     "drone_dropout_apply_f32": (_I, [_P, _P, _I64, _F, _P]),
-    "drone_cross_entropy_f32": (_I, [_I, _I, _P, _I, _P, _P, _I, _P, _P, _P]),
+    "drone_cross_entropy_f32": (_I, [_I, _I, _P, _I, _P, _P, _I, _F, _P, _P, _P]),
     "drone_accuracy_f32": (_I, [_I, _I, _P, _I, _P, _P, _P, _P]),
     "drone_sgd_step_f32": (_I, [_P, _P, _I64, _F, _P]),
     "drone_adam_step_f32": (_I, [_P, _P, _P, _P, _I64, _I, _F, _F, _F, _F, _F, _I, _P]),
@@ -119,6 +119,7 @@ SIGNATURES = {
     "drone_fill_uniform_f32": (_I, [_P, _I64, _U64, _F, _F]),
     "drone_fill_normal_f32": (_I, [_P, _I64, _U64]),
     "drone_fill_randint_i32": (_I, [_P, _I64, _U64, C.c_int32]),
+    "drone_stream_copy_f64": (_I, [_P, _P, _I64, _P]),
     "drone_timer_create": (_I, [C.POINTER(_P)]),
     "drone_timer_start": (_I, [_P, _P]),
     "drone_timer_stop": (_I, [_P, _P]),

@@ -3,6 +3,7 @@
 // (gcn.cu:96-106 -> CUDAGCN::run_epoch, cuda_gcn.cu:356-379), so a host in any language can drive a training
 // run.  Data loading is out: the caller hands over device arrays.
 #include <cstring>
+#include <vector>
 
 #include "../../include/drone_gcn_modules.hpp"
 #include "common.h"
@@ -24,6 +25,18 @@ void drone_gcn_mod::GCN::set_truth(int current_split)
     const int n = params.localVertexSize;
     set_truth_kernel<<<(n + 255) / 256, 256, 0, static_cast<hipStream_t>(s)>>>(truth, split, label, current_split, n);
     DRONE_GCN_HIP(hipGetLastError());
+    if (params.mean_gradient && current_split != truth_split) {
+        // number of labelled rows, needed on the host to scale the loss gradient; recounted only when the
+        // split changes (labels and split ids are fixed for the handle's lifetime)
+        std::vector<int> h((size_t)n);
+        DRONE_GCN_HIP(hipMemcpyAsync(h.data(), truth, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost,
+                                     static_cast<hipStream_t>(s)));
+        DRONE_GCN_HIP(hipStreamSynchronize(static_cast<hipStream_t>(s)));
+        truth_count = 0;
+        for (int v : h) truth_count += v >= 0;
+        ce->grad_scale = truth_count > 0 ? 1.0f / (float)truth_count : 1.0f;
+    }
+    truth_split = current_split;
 }
 
 struct drone_gcn {
@@ -51,6 +64,7 @@ extern "C" int drone_gcn_create(struct drone_gcn **out, const drone_gcn_config *
     p.weight_decay = cfg->weight_decay;
     p.use_dropout = cfg->use_dropout != 0;
     p.use_adam = cfg->use_adam != 0;
+    p.mean_gradient = cfg->mean_gradient != 0;
     p.seed = cfg->seed;
     struct drone_gcn *h = new drone_gcn();
     h->model = new drone_gcn_mod::GCN(p, nnz, rp, ci, in_degree, out_degree, X, ldx, label, split, W1, W2, stream);

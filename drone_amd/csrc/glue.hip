@@ -61,7 +61,7 @@ __global__ void dropout_apply_kernel(float *__restrict__ x, const uint8_t *__res
 // labelled-row count go to block_loss / block_count.
 __global__ __launch_bounds__(kThreads) void cross_entropy_kernel(int n, int classes, const float *__restrict__ logits,
                                                                  int ld, const int *__restrict__ truth,
-                                                                 float *__restrict__ grad, int ldg,
+                                                                 float *__restrict__ grad, int ldg, float grad_scale,
                                                                  double *__restrict__ block_loss,
                                                                  int *__restrict__ block_count)
 {
@@ -89,7 +89,7 @@ __global__ __launch_bounds__(kThreads) void cross_entropy_kernel(int n, int clas
             for (int j = lane; j < classes; j += kWave) {
                 float g = expf(z[j] - mx) / sum;
                 if (j == t) g -= 1.0f;
-                grad[(size_t)row * ldg + j] = g;
+                grad[(size_t)row * ldg + j] = g * grad_scale;
             }
         if (lane == 0) {
             loss += (double)(logf(sum) - (z[t] - mx));
@@ -248,7 +248,8 @@ extern "C" int drone_dropout_apply_f32(float *x, const uint8_t *keep, int64_t n,
 }
 
 extern "C" int drone_cross_entropy_f32(int n, int classes, const float *logits, int ld, const int *truth, float *grad,
-                                       int ldg, float *loss_out, int *count_out, drone_stream_t stream)
+                                       int ldg, float grad_scale, float *loss_out, int *count_out,
+                                       drone_stream_t stream)
 {
     clear_error();
     DRONE_REQUIRE(n > 0 && classes > 0 && logits && truth && ld >= classes, "operands");
@@ -270,7 +271,7 @@ extern "C" int drone_cross_entropy_f32(int n, int classes, const float *logits, 
     double *bl = static_cast<double *>(ws);
     int *bc = reinterpret_cast<int *>(bl + 2048);
     hipStream_t s = as_stream(stream);
-    cross_entropy_kernel<<<blocks, kThreads, 0, s>>>(n, classes, logits, ld, truth, grad, ldg, bl, bc);
+    cross_entropy_kernel<<<blocks, kThreads, 0, s>>>(n, classes, logits, ld, truth, grad, ldg, grad_scale, bl, bc);
     cross_entropy_finish_kernel<<<1, kThreads, 0, s>>>(blocks, bl, bc, loss_out, count_out);
     DRONE_HIP_TRY(hipGetLastError());
     return DRONE_OK;

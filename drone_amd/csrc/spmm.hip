@@ -60,27 +60,35 @@ __device__ __forceinline__ void row_segment(int e0, int e1, const int *__restric
     const int sub = lane / G;
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
+    // U non-zeros per lane group are fetched per step so that U independent feature-row loads are in flight
+    // per lane; slots past the end of the segment carry (col 0, val 0) and add nothing.
+    constexpr int U = (kWave / P) < 8 ? (kWave / P) : 8;
     for (int base = e0; base < e1; base += kWave) {
         const int e = base + lane;
         const int c = e < e1 ? ci[e] : 0;
         const float a = e < e1 ? val[e] : 0.0f;
         const int cnt = (e1 - base) < kWave ? (e1 - base) : kWave;
-
-        for (int q = 0; q < cnt; q += P) {
-            int cc;
-            float aa;
-            if constexpr (P == 1) {
-                cc = __builtin_amdgcn_readlane(c, q);
-                aa = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, a), q));
-            } else {
-                cc = __shfl(c, q + sub, kWave);
-                aa = __shfl(a, q + sub, kWave);
+        for (int q = 0; q < cnt; q += P * U) {
+            int cc[U];
+            float aa[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if constexpr (P == 1) {
+                    cc[u] = __builtin_amdgcn_readlane(c, q + u);
+                    aa[u] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, a), q + u));
+                } else {
+                    cc[u] = __shfl(c, q + u * P + sub, kWave);
+                    aa[u] = __shfl(a, q + u * P + sub, kWave);
+                }
             }
             if (active) {
-                float b[VEC];
-                load_vec<VEC>(B + (size_t)cc * ldb + kbase, b);
+                float b[U][VEC];
 #pragma unroll
-                for (int v = 0; v < VEC; ++v) acc[v] = fmaf(aa, b[v], acc[v]);
+                for (int u = 0; u < U; ++u) load_vec<VEC>(B + (size_t)cc[u] * ldb + kbase, b[u]);
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) acc[v] = fmaf(aa[u], b[u][v], acc[v]);
             }
         }
     }

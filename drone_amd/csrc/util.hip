@@ -110,6 +110,24 @@ extern "C" int drone_fill_randint_i32(int32_t *out, int64_t n, uint64_t seed, in
     return DRONE_OK;
 }
 
+namespace {
+__global__ void stream_copy_f64_kernel(const double *__restrict__ src, double *__restrict__ dst, int64_t n)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        dst[i] = src[i];
+}
+}  // namespace
+
+extern "C" int drone_stream_copy_f64(double *dst, const double *src, int64_t n, drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(n >= 0 && (n == 0 || (dst && src)), "null operand");
+    if (n == 0) return DRONE_OK;
+    stream_copy_f64_kernel<<<8192, 256, 0, as_stream(stream)>>>(src, dst, n);
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
 struct drone_timer {
     hipEvent_t a, b;
 };

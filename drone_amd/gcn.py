@@ -89,7 +89,7 @@ def dropout_apply(x, keep, p, stream=0):
     check(lib().drone_dropout_apply_f32(_ptr(x), _ptr(keep), x.numel(), float(p), stream))
 
 
-def cross_entropy(logits, truth, classes=None, grad=None, stream=0):
+def cross_entropy(logits, truth, classes=None, grad=None, grad_scale=1.0, stream=0):
     """Returns (loss tensor [1], count tensor [1]); fills grad when given."""
     import torch
     n = logits.shape[0]
@@ -97,7 +97,7 @@ def cross_entropy(logits, truth, classes=None, grad=None, stream=0):
     loss = torch.empty(1, dtype=torch.float32, device=logits.device)
     count = torch.empty(1, dtype=torch.int32, device=logits.device)
     check(lib().drone_cross_entropy_f32(n, classes, _ptr(logits), logits.stride(0), _ptr(truth), _ptr(grad),
-                                        0 if grad is None else grad.stride(0), _ptr(loss), _ptr(count), stream))
+                                        0 if grad is None else grad.stride(0), float(grad_scale), _ptr(loss), _ptr(count), stream))
     return loss, count
 
 
@@ -127,13 +127,13 @@ class GcnModel:
     label/split: int32 (split 1 = train), W1/W2: float32 initial weights."""
 
     def __init__(self, rp, ci, in_deg, out_deg, X, label, split, W1, W2, dropout=0.5, lr=0.01, weight_decay=5e-4,
-                 use_dropout=False, use_adam=True, seed=1234, stream=0):
+                 use_dropout=False, use_adam=True, mean_gradient=False, seed=1234, stream=0):
         from ._lib import GcnConfig
         n, input_dim = X.shape
         hidden, classes = W1.shape[1], W2.shape[1]
         assert W1.shape[0] == input_dim and W2.shape[0] == hidden and W1.is_contiguous() and W2.is_contiguous()
         assert X.stride(1) == 1
-        cfg = GcnConfig(n, input_dim, hidden, classes, dropout, lr, weight_decay, int(use_dropout), int(use_adam), seed)
+        cfg = GcnConfig(n, input_dim, hidden, classes, dropout, lr, weight_decay, int(use_dropout), int(use_adam), int(mean_gradient), seed)
         self._keep = (rp, ci, in_deg, out_deg, X, label, split)
         self.n, self.input_dim, self.hidden, self.classes = n, input_dim, hidden, classes
         self.nnz = ci.numel()

@@ -228,6 +228,7 @@ class CrossEntropyLoss : public Module {
 public:
     float *d_loss = nullptr;  // device scalars
     int *d_count = nullptr;
+    float grad_scale = 1.0f;  // 1 = the reference's sum-reduced gradient
     CrossEntropyLoss(Variable *logits_, const int *truth_, int num_classes_, std::string name, drone_stream_t stream)
         : logits(logits_), truth(truth_), num_classes(num_classes_), s(stream)
     {
@@ -239,7 +240,7 @@ public:
     void forward(bool training) override
     {
         DRONE_GCN_CHECK(drone_cross_entropy_f32(logits->rows, num_classes, logits->data, logits->ld, truth,
-                                                training ? logits->grad : nullptr, logits->ld, d_loss, d_count, s));
+                                                training ? logits->grad : nullptr, logits->ld, grad_scale, d_loss, d_count, s));
     }
     void backward() override {}
 };
@@ -303,6 +304,7 @@ struct GCNParams {
     float dropout = 0.5f, learning_rate = 0.01f, weight_decay = 5e-4f;
     bool use_dropout = false;   // the reference leaves its dropout modules commented out (cuda_gcn.cu:35,64)
     bool use_adam = true;       // reference optimiser; false = SGD
+    bool mean_gradient = false; // false = sum-reduced loss gradient as in the reference (cuda_module.cu:452)
     uint64_t seed = 1234;       // cuda_kernel.cu:426 seeds cuRAND with 1234
 };
 
@@ -320,6 +322,7 @@ public:
     ReLU *relu = nullptr;
     Dropout *drop = nullptr;
     int *truth = nullptr;   // device [N]: label on rows of the current split, -1 elsewhere
+    int truth_split = -1, truth_count = 0;
     int *counts = nullptr;  // device [2]: correct, labelled
     const int *label = nullptr, *split = nullptr;  // device, borrowed
     drone_stream_t s;

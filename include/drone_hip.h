@@ -192,10 +192,11 @@ int drone_relu_backward_f32(float *grad, const uint8_t *mask, int64_t n, drone_s
 int drone_dropout_mask(uint8_t *keep, int64_t n, uint64_t seed, uint64_t step, float p, drone_stream_t stream);
 int drone_dropout_apply_f32(float *x, const uint8_t *keep, int64_t n, float p, drone_stream_t stream);
 /* cuda_kernel.cu:295-379 + cuda_module.cu:406-483.  truth[i] < 0 = unlabelled.  grad (optional) receives
- * softmax - onehot on labelled rows and 0 elsewhere - a SUM-reduced gradient (count_grad = 1 in the
- * reference); *loss_out (device) = mean loss over labelled rows, *count_out (device) = their number. */
+ * grad_scale * (softmax - onehot) on labelled rows and 0 elsewhere.  grad_scale = 1 is the reference's
+ * SUM-reduced gradient (count_grad = 1, cuda_module.cu:452); 1/labelled-count gives the mean-reduced one.
+ * *loss_out (device) = mean loss over labelled rows, *count_out (device) = their number. */
 int drone_cross_entropy_f32(int n, int classes, const float *logits, int ld, const int *truth, float *grad,
-                            int ldg, float *loss_out, int *count_out, drone_stream_t stream);
+                            int ldg, float grad_scale, float *loss_out, int *count_out, drone_stream_t stream);
 /* cuda_gcn.cu:226-246: a labelled row is correct unless some logit is strictly greater than the true-class
  * logit.  counts[0] += correct, counts[1] += labelled (device ints, zeroed by the caller); pred (optional)
  * receives the arg-max with ties to the lowest index. */
@@ -223,6 +224,8 @@ typedef struct drone_gcn_config {
     int use_dropout; /* 0 = as the reference runs (its dropout modules are commented out, cuda_gcn.cu:35,64);
                         1 = dropout(p) after the hidden ReLU */
     int use_adam;    /* 1 = Adam as in the reference (cuda_gcn.cu:86-89); 0 = SGD */
+    int mean_gradient; /* 0 = sum-reduced loss gradient as in the reference (cuda_module.cu:452); 1 = divided by
+                          the number of labelled rows, which a plain SGD step needs to stay stable */
     uint64_t seed;   /* dropout mask stream */
 } drone_gcn_config;
 int drone_gcn_create(drone_gcn **handle, const drone_gcn_config *cfg, int64_t nnz, const int *rp, const int *ci,
@@ -257,6 +260,10 @@ int drone_rmat_edges(int scale, int64_t n_edges, double a, double b, double c, u
 int drone_fill_uniform_f32(float *out, int64_t n, uint64_t seed, float lo, float hi);
 int drone_fill_normal_f32(float *out, int64_t n, uint64_t seed);
 int drone_fill_randint_i32(int32_t *out, int64_t n, uint64_t seed, int32_t bound);
+
+/* Plain device-to-device copy kernel of n doubles: reads 8n bytes, writes 8n bytes.  A dispatch of known
+ * traffic that profiler byte counters can be scaled by, and a measured stream-bandwidth reference. */
+int drone_stream_copy_f64(double *dst, const double *src, int64_t n, drone_stream_t stream);
 
 /* HIP-event stopwatch on a stream (bench harness plumbing). */
 typedef struct drone_timer drone_timer;
