@@ -89,7 +89,8 @@ SIGNATURES = {
     "drone_pr_run_graph_f64": (_I, [C.POINTER(Graph), C.POINTER(PRValues), _D, _I, _P]),
     "drone_gcn_edge_values": (_I, [_I, _P, _P, _P, _P, _P, _P]),
     "drone_csr_transpose_f32": (_I, [_I, _I, _I64, _P, _P, _P, _P, _P, _P, _P]),
-    "drone_spmm_plan_create": (_I, [C.POINTER(_P), _I, _I64, _P, _I, _P]),
+    "drone_spmm_plan_create": (_I, [C.POINTER(_P), _I, _I, _I64, _P, _P, _P, _I, _P]),
+    "drone_spmm_plan_update_values": (_I, [_P, _P, _P]),
     "drone_spmm_plan_destroy": (_I, [_P]),
     "drone_spmm_csr_f32": (_I, [_P, _P, _P, _P, _P, _I, _P, _I, _I, _F, _F, _P]),
     "drone_spmm_bytes": (_I64, [_I, _I64, _I]),

@@ -27,7 +27,7 @@ struct PrF64Epi {
     {
         const double base = (1.0 - alpha) * inv_n + alpha * dang[0] * inv_n;
         const double rn = base + alpha * s;
-        const double iv = inv[r];
+        const double iv = __builtin_nontemporal_load(inv + r);
         c_out[r] = rn * iv;
         if (r_out) r_out[order[r]] = rn;
         if (iv == 0.0) stat += rn;

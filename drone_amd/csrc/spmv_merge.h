@@ -140,7 +140,9 @@ __global__ __launch_bounds__(kSpmvBlock) void spmv_merge_kernel(
     const int ne = (int)(e1 - e0);
     const int items = nr + ne;
 
-    for (int i = tid; i < nr; i += kSpmvBlock) s_rowend[i] = (int)((int64_t)row_ptr[r0 + 1 + i] - e0);
+    // row_ptr and col_idx are streamed once: non-temporal loads keep them from evicting the gather source from L2
+    for (int i = tid; i < nr; i += kSpmvBlock)
+        s_rowend[i] = (int)((int64_t)__builtin_nontemporal_load(row_ptr + r0 + 1 + i) - e0);
     if (tid == 0) s_rowend[nr] = INT_MAX;
 
     {
@@ -148,7 +150,7 @@ __global__ __launch_bounds__(kSpmvBlock) void spmv_merge_kernel(
 #pragma unroll
         for (int k = 0; k < IPT; ++k) {
             const int i = tid + k * kSpmvBlock;
-            c[k] = i < ne ? col[e0 + i] : -1;
+            c[k] = i < ne ? __builtin_nontemporal_load(col + e0 + i) : -1;
         }
         V x[IPT];
 #pragma unroll

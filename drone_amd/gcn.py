@@ -33,13 +33,21 @@ def csr_transpose(n_rows, n_cols, rp, ci, val=None, stream=0):
 
 
 class SpmmPlan:
-    def __init__(self, rp, nnz, max_k, stream=0):
+    """Schedule (and band-sorted copy of the long rows) for the SpMM of one CSR; see drone_spmm_plan_create."""
+
+    def __init__(self, rp, ci, val, n_cols, max_k, stream=0):
         self.n_rows = rp.numel() - 1
-        self.nnz = int(nnz)
+        self.n_cols = int(n_cols)
+        self.nnz = int(ci.numel())
         self.max_k = int(max_k)
+        self._keep = (rp, ci, val)
         h = C.c_void_p()
-        check(lib().drone_spmm_plan_create(C.byref(h), self.n_rows, self.nnz, _ptr(rp), self.max_k, stream))
+        check(lib().drone_spmm_plan_create(C.byref(h), self.n_rows, self.n_cols, self.nnz, _ptr(rp), _ptr(ci), _ptr(val),
+                                           self.max_k, stream))
         self.h = h
+
+    def update_values(self, val, stream=0):
+        check(lib().drone_spmm_plan_update_values(self.h, _ptr(val), stream))
 
     def close(self):
         if self.h:

@@ -132,8 +132,8 @@ struct Adjacency {
         DRONE_GCN_HIP(hipMalloc(&valT, sizeof(float) * e));
         DRONE_GCN_CHECK(drone_gcn_edge_values(n, rp, ci, in_degree, out_degree, val, s));
         DRONE_GCN_CHECK(drone_csr_transpose_f32(n, n, nnz, rp, ci, val, rpT, ciT, valT, s));
-        DRONE_GCN_CHECK(drone_spmm_plan_create(&plan, n, nnz, rp, max_dim, s));
-        DRONE_GCN_CHECK(drone_spmm_plan_create(&planT, n, nnz, rpT, max_dim, s));
+        DRONE_GCN_CHECK(drone_spmm_plan_create(&plan, n, n, nnz, rp, ci, val, max_dim, s));
+        DRONE_GCN_CHECK(drone_spmm_plan_create(&planT, n, n, nnz, rpT, ciT, valT, max_dim, s));
     }
     Adjacency(const Adjacency &) = delete;
     ~Adjacency()

@@ -163,11 +163,17 @@ int drone_gcn_edge_values(int n, const int *rp, const int *ci, const int *in_deg
  * ascend within each output row.  v / vT may both be NULL (pattern only).  Synchronises `stream`. */
 int drone_csr_transpose_f32(int n_rows, int n_cols, int64_t nnz, const int *rp, const int *ci,
                             const float *v, int *rpT, int *ciT, float *vT, drone_stream_t stream);
-/* Row classification for the SpMM of one CSR (rows with more than 4096 entries are split); holds the
- * scratch for their partial rows, sized for feature widths up to max_k.  rp is read during the call. */
+/* Schedule for the SpMM of one CSR with feature widths up to max_k.  Rows of at most 512 entries run one
+ * wavefront each.  Longer rows are cut by column band (columns ranked by frequency; a band's feature rows fill
+ * about 2 MB of L2) and the plan keeps a (band,row)-sorted copy of their entries - columns AND values as
+ * passed here - plus the scratch for their partial rows.  The rp / ci / v later passed to
+ * drone_spmm_csr_f32 must be the arrays the plan was built from; after changing values in place call
+ * drone_spmm_plan_update_values.  Set-up step (the counterpart of cusparseSpMM_bufferSize + the
+ * preprocessing cuSPARSE hides, cuda_module.cu:232-243); synchronises `stream`. */
 typedef struct drone_spmm_plan drone_spmm_plan;
-int drone_spmm_plan_create(drone_spmm_plan **plan, int n_rows, int64_t nnz, const int *rp, int max_k,
-                           drone_stream_t stream);
+int drone_spmm_plan_create(drone_spmm_plan **plan, int n_rows, int n_cols, int64_t nnz, const int *rp,
+                           const int *ci, const float *v, int max_k, drone_stream_t stream);
+int drone_spmm_plan_update_values(drone_spmm_plan *plan, const float *v, drone_stream_t stream);
 int drone_spmm_plan_destroy(drone_spmm_plan *plan);
 /* cusparseSpMM(NON_TRANSPOSE, NON_TRANSPOSE, alpha, A, B, beta, C, ALG_DEFAULT) at cuda_module.cu:245
  * (forward: A = transposed CSR) and :335 (backward: A = original CSR):

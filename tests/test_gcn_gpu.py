@@ -33,9 +33,10 @@ def random_csr(seed, n_rows, n_cols, density, hub=None):
     rng = np.random.default_rng(seed)
     m = sp.random(n_rows, n_cols, density=density, random_state=np.random.RandomState(seed), format="lil",
                   dtype=np.float32)
-    if hub is not None:                       # one very long row to force the split path
-        cols = rng.choice(n_cols, size=hub, replace=False)
-        m[3, cols] = rng.uniform(-1, 1, hub).astype(np.float32)
+    if hub is not None:                       # very long rows to force the band-split path
+        for r, h in enumerate(hub if isinstance(hub, (list, tuple)) else [hub]):
+            cols = rng.choice(n_cols, size=h, replace=False)
+            m[(3 + 5 * r) % n_rows, cols] = rng.uniform(-1, 1, h).astype(np.float32)
     m = m.tocsr()
     m.sort_indices()
     m.data = rng.uniform(-1, 1, m.nnz).astype(np.float32)
@@ -51,7 +52,7 @@ def run_spmm(T, m, B, K=None, ld_pad=0, alpha=1.0, beta=0.0, C0=None):
     out = T.full((m.shape[0], K + ld_pad), 7.0, dtype=T.float32, device="cuda")
     if C0 is not None:
         out[:, :K] = dev(T, C0)
-    plan = gcn.SpmmPlan(rp, m.nnz, max_k=K)
+    plan = gcn.SpmmPlan(rp, ci, v, m.shape[1], max_k=K)
     gcn.spmm(plan, rp, ci, v, Bd[:, :K], K=K, out=out[:, :K], alpha=alpha, beta=beta)
     T.cuda.synchronize()
     plan.close()
@@ -80,12 +81,15 @@ def test_spmm_against_oracle(T, oracle, K, ld_pad):
     assert np.all(got[np.diff(m.indptr) == 0] == 0.0)             # empty rows are written as zero (beta = 0)
 
 
-def test_spmm_long_rows_split_and_alpha_beta(T, oracle):
+@pytest.mark.parametrize("K", [41, 128, 256])
+def test_spmm_long_rows_split_and_alpha_beta(T, oracle, K):
+    """Rows above 512 entries take the band-piece path: several of them, several column bands (a band holds
+    2 MB / (4 K) columns), pieces longer than 2048 entries, mixed with short and empty rows."""
     n = 9000
-    m = random_csr(5, 40, n, 0.002, hub=8500)                       # row 3 has > 4096 entries -> split path
+    m = random_csr(5, 40, n, 0.002, hub=[8500, 600, 3000, 513, 512])
     assert np.diff(m.indptr).max() > 4096
-    B = np.random.default_rng(1).uniform(-1, 1, (n, 41)).astype(np.float32)
-    C0 = np.random.default_rng(2).uniform(-1, 1, (40, 41)).astype(np.float32)
+    B = np.random.default_rng(1).uniform(-1, 1, (n, K)).astype(np.float32)
+    C0 = np.random.default_rng(2).uniform(-1, 1, (40, K)).astype(np.float32)
     got = run_spmm(T, m, B, alpha=0.5, beta=2.0, C0=C0)
     ref = 0.5 * oracle.spmm_f64acc(m.indptr, m.indices, m.data, B) + 2.0 * C0
     scale = 0.5 * oracle.spmm_f64acc(m.indptr, m.indices, np.abs(m.data), np.abs(B)) + 2.0 * np.abs(C0)
@@ -93,6 +97,21 @@ def test_spmm_long_rows_split_and_alpha_beta(T, oracle):
     a = run_spmm(T, m, B)
     b = run_spmm(T, m, B)
     np.testing.assert_array_equal(a, b)                             # fixed summation order: bitwise repeatable
+
+
+def test_spmm_plan_update_values(T, oracle):
+    from drone_amd import gcn
+    m = random_csr(8, 30, 5000, 0.01, hub=[2000, 700])
+    rp, ci = dev(T, m.indptr.astype(np.int32)), dev(T, m.indices.astype(np.int32))
+    v = dev(T, m.data)
+    B = np.random.default_rng(3).uniform(-1, 1, (5000, 64)).astype(np.float32)
+    plan = gcn.SpmmPlan(rp, ci, v, 5000, max_k=64)
+    v.mul_(-2.0)                                                    # values changed in place after planning
+    plan.update_values(v)
+    got = gcn.spmm(plan, rp, ci, v, dev(T, B)).cpu().numpy()
+    plan.close()
+    ref = oracle.spmm_f64acc(m.indptr, m.indices, -2.0 * m.data, B)
+    assert rel_err(got, ref, oracle.spmm_f64acc(m.indptr, m.indices, 2.0 * np.abs(m.data), np.abs(B))) <= 1e-4
 
 
 def test_spmm_empty_matrix_and_rows(T):
