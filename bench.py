@@ -271,7 +271,7 @@ def main():
     plan = PullPlanF64(x["row_ptr"], x["col_idx"], x["inv_outdeg"])
     torch.cuda.synchronize()
     plan_s = time.time() - t0
-    log(f"plan (hot-first relabel + merge-path tiling): {plan_s*1e3:.1f} ms (one-off, not timed)")
+    log(f"plan (hot-first relabel + source-sorted row blocks): {plan_s*1e3:.1f} ms (one-off, not timed)")
     out = torch.empty(n, dtype=torch.float64, device="cuda")
 
     for _ in range(args.warmup):
@@ -304,7 +304,7 @@ def main():
                    "iterations_per_step": args.iters, "vertices": n, "edges": nnz},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "spmv_merge_kernel<double,long,8,PrF64Epi>",
+                     "kernel": "pr_rowblock_kernel<PrF64Epi>",
                      "algorithmic_bytes_per_launch": bytes_iter, "mean_launch_ms": prof["mean_ms"],
                      "launches_timed": prof["launches"]},
         "plan_ms_one_off": plan_s * 1e3,

@@ -81,6 +81,7 @@ SIGNATURES = {
     "drone_graph_destroy": (None, [C.POINTER(Graph)]),
     "drone_pr_values_destroy": (None, [C.POINTER(Graph), C.POINTER(PRValues)]),
     "drone_pr_plan_create": (_I, [C.POINTER(_P), _I64, _I64, _P, _P, _P, _P]),
+    "drone_pr_plan_create_ex": (_I, [C.POINTER(_P), _I64, _I64, _P, _P, _P, _I, _P]),
     "drone_pr_plan_destroy": (_I, [_P]),
     "drone_pr_run_f64": (_I, [_P, _D, _I, _P, _P]),
     "drone_pr_profile_enable": (_I, [_P, _I]),

@@ -6,6 +6,7 @@
 // The aggregation kernel gathers c_{k-1}, and its row epilogue writes c_k (and r_k on the last
 // iteration) and accumulates d_k, so one iteration touches: row_ptr 8N, col_idx 4E, gather source 8N,
 // inv_outdeg 8N, c_k 8N  =  4E + 32N bytes.
+#include "pr_rowblock.h"
 #include "relabel.h"
 #include "spmv_merge.h"
 
@@ -74,6 +75,9 @@ struct drone_pr_plan {
     const double *inv_user = nullptr;  // caller's inverse out-degree, caller's vertex order
     Relabel rl;                        // hot-first copy of the CSR; all work vectors use its id space
     double *inv = nullptr;             // inverse out-degree in internal order
+    int deterministic = 0;             // 1: merge-path tiles (bit-reproducible); 0: source-sorted row blocks
+    RowBlocks rb;
+    int units = 0;                     // tiles or blocks of the active mode
     MergeTiling mt;
     MergeScratch ms;
     double *c[2] = {nullptr, nullptr};
@@ -89,12 +93,21 @@ extern "C" int64_t drone_pr_bytes_per_iteration(int64_t n, int64_t nnz) { return
 extern "C" int drone_pr_plan_create(drone_pr_plan **out, int64_t n, int64_t nnz, const int64_t *row_ptr,
                                     const int32_t *col_idx, const double *inv_outdeg, drone_stream_t stream)
 {
+    return drone_pr_plan_create_ex(out, n, nnz, row_ptr, col_idx, inv_outdeg, 0, stream);
+}
+
+extern "C" int drone_pr_plan_create_ex(drone_pr_plan **out, int64_t n, int64_t nnz, const int64_t *row_ptr,
+                                       const int32_t *col_idx, const double *inv_outdeg, int flags,
+                                       drone_stream_t stream)
+{
     clear_error();
     DRONE_REQUIRE(out != nullptr, "plan pointer");
     DRONE_REQUIRE(n > 0 && n < INT32_MAX, "vertex count must be in [1, 2^31-2]");
     DRONE_REQUIRE(nnz >= 0, "nnz");
     DRONE_REQUIRE(row_ptr && inv_outdeg && (col_idx || nnz == 0), "null CSR array");
+    DRONE_REQUIRE((flags & ~DRONE_PR_DETERMINISTIC) == 0, "unknown flag");
     drone_pr_plan *p = new drone_pr_plan();
+    p->deterministic = (flags & DRONE_PR_DETERMINISTIC) != 0 || nnz >= (int64_t)UINT32_MAX;
     DRONE_HIP_TRY(hipGetDevice(&p->device));
     p->n = n;
     p->nnz = nnz;
@@ -102,17 +115,35 @@ extern "C" int drone_pr_plan_create(drone_pr_plan **out, int64_t n, int64_t nnz,
     hipStream_t s = as_stream(stream);
     int rc = relabel_create(&p->rl, n, nnz, row_ptr, col_idx, s);
     if (rc != DRONE_OK) { delete p; return rc; }
-    rc = merge_tiling_create<int64_t>(&p->mt, n, nnz, p->rl.row_ptr, kSpmvBlock * kPrIpt, s);
-    if (rc != DRONE_OK) { drone_pr_plan_destroy(p); return rc; }
-    rc = merge_scratch_create(&p->ms, p->mt, sizeof(double));
-    if (rc != DRONE_OK) { drone_pr_plan_destroy(p); return rc; }
+    if (p->deterministic) {
+        rc = merge_tiling_create<int64_t>(&p->mt, n, nnz, p->rl.row_ptr, kSpmvBlock * kPrIpt, s);
+        if (rc != DRONE_OK) { drone_pr_plan_destroy(p); return rc; }
+        p->units = p->mt.num_tiles;
+    } else {
+        rc = row_blocks_create(&p->rb, n, nnz, p->rl.row_ptr, p->rl.col, s);
+        if (rc != DRONE_OK) { drone_pr_plan_destroy(p); return rc; }
+        p->units = p->rb.num_blocks;
+        // the row-ordered copy is only needed to build the blocks
+        (void)hipFree(p->rl.row_ptr);
+        (void)hipFree(p->rl.col);
+        p->rl.row_ptr = nullptr;
+        p->rl.col = nullptr;
+        DRONE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&pr_rowblock_kernel<PrF64Epi>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, kRbLdsBytes));
+    }
+    {
+        MergeTiling shape;  // scratch is sized by the number of work units of the active mode
+        shape.num_tiles = p->units;
+        rc = merge_scratch_create(&p->ms, shape, sizeof(double));
+        if (rc != DRONE_OK) { drone_pr_plan_destroy(p); return rc; }
+    }
     DRONE_HIP_TRY(hipMalloc(&p->c[0], sizeof(double) * (size_t)n));
     DRONE_HIP_TRY(hipMalloc(&p->c[1], sizeof(double) * (size_t)n));
     DRONE_HIP_TRY(hipMalloc(&p->dang, sizeof(double)));
     DRONE_HIP_TRY(hipMalloc(&p->inv, sizeof(double) * (size_t)n));
     // the init kernel parks its block partials in block_stat: never more blocks than it holds
     int ib = (int)ceil_div(n, kSpmvBlock * 8);
-    const int fb = fixup_blocks(p->mt.num_tiles);
+    const int fb = fixup_blocks(p->units);
     p->init_blocks = ib < fb ? ib : fb;
     if (p->init_blocks < 1) p->init_blocks = 1;
     DRONE_HIP_TRY(hipStreamSynchronize(s));
@@ -125,6 +156,7 @@ extern "C" int drone_pr_plan_destroy(drone_pr_plan *p)
     if (!p) return DRONE_OK;
     merge_tiling_destroy(&p->mt);
     merge_scratch_destroy(&p->ms);
+    row_blocks_destroy(&p->rb);
     relabel_destroy(&p->rl);
     if (p->inv) (void)hipFree(p->inv);
     if (p->c[0]) (void)hipFree(p->c[0]);
@@ -215,13 +247,19 @@ extern "C" int drone_pr_run_f64(drone_pr_plan *p, double alpha, int iters, doubl
         epi.inv_n = inv_n;
         const bool prof = p->prof_n < p->prof_cap;
         double *carry = static_cast<double *>(p->ms.tile_carry);
+        const int fb = fixup_blocks(p->units);
         if (prof) DRONE_HIP_TRY(hipEventRecord(p->ev0[p->prof_n], s));
-        spmv_merge_kernel<double, int64_t, kPrIpt, PrF64Epi><<<p->mt.num_tiles, kSpmvBlock, 0, s>>>(
-            p->n, p->nnz, p->mt.tile_row, p->rl.row_ptr, p->rl.col, epi, carry, p->ms.tile_stat);
+        if (p->deterministic) {
+            spmv_merge_kernel<double, int64_t, kPrIpt, PrF64Epi><<<p->mt.num_tiles, kSpmvBlock, 0, s>>>(
+                p->n, p->nnz, p->mt.tile_row, p->rl.row_ptr, p->rl.col, epi, carry, p->ms.tile_stat);
+        } else {
+            pr_rowblock_kernel<PrF64Epi><<<p->rb.num_blocks, kRbThreads, kRbLdsBytes, s>>>(
+                p->rb.block_row, p->rb.block_nnz, p->rb.col, p->rb.lrow, epi, carry, p->ms.tile_stat);
+        }
         if (prof) DRONE_HIP_TRY(hipEventRecord(p->ev1[p->prof_n++], s));
-        const int fb = fixup_blocks(p->mt.num_tiles);
         spmv_fixup_kernel<double, PrF64Epi><<<fb, kSpmvBlock, 0, s>>>(
-            p->mt.num_tiles, p->mt.tile_row, p->mt.walk_len, carry, p->ms.tile_stat, epi, p->ms.block_stat);
+            p->units, p->deterministic ? p->mt.tile_row : p->rb.block_row,
+            p->deterministic ? p->mt.walk_len : p->rb.walk_len, carry, p->ms.tile_stat, epi, p->ms.block_stat);
         // dang is read by the kernels above and overwritten here, in stream order
         reduce_stat_kernel<0><<<1, kSpmvBlock, 0, s>>>(p->ms.block_stat, fb, p->dang);
     }

@@ -1,0 +1,104 @@
+// Row-block pull aggregation with source-sorted entries and LDS accumulators (fp64 PageRank fast path).
+//
+// Why: an 8-byte gather costs a whole 128-byte line on its way from L2 (or beyond) to the CU, so the gather
+// stream is priced by distinct lines per unit time, not by bytes.  In row order, consecutive gathers hit
+// unrelated lines.  Here the rows are cut into blocks of at most kRbRows rows / kRbItems entries, and inside a
+// block the entries are sorted by source id once, at plan time.  A block then sweeps the source vector in
+// ascending order: the popular sources (which hot-first relabelling packs into few lines) are hit by adjacent
+// lanes and back-to-back instructions, so they are served by lane coalescing and L1 instead of L2, and the cold
+// tail is read in address order.  Sorting destroys row order, so every entry carries its block-local row (16 bit)
+// and is added into a per-block accumulator array in LDS with ds_add_f64; the row epilogue then runs over the
+// block's rows with coalesced loads and stores.
+//
+// Blocks are equal shares of the weighted merge of {row ends (weight W)} and {entries (weight 1)}, W =
+// kRbItems / kRbRows, so a block never exceeds its row or entry capacity and empty-row runs and hub rows cost about
+// the same.  A row may straddle blocks: the block in which it ends applies the epilogue to its local part, the
+// parts in earlier blocks are written as carries and folded in by spmv_fixup_kernel (spmv_merge.h), exactly as
+// for the merge-path tiles.  The LDS additions are unordered, so the last bits of a sum can differ between runs
+// (the reference's float atomics have the same property); the merge-path kernel stays available for
+// bit-reproducible results.
+#pragma once
+#include "spmv_merge.h"
+
+namespace drone {
+
+constexpr int kRbThreads = 1024;
+constexpr int kRbRows = 16384;       // most rows ending in one block (LDS accumulators: 128 KB)
+constexpr int kRbItems = 1 << 19;    // most entries in one block
+constexpr int kRbWeight = kRbItems / kRbRows;
+constexpr int kRbUnroll = 8;
+constexpr int kRbLdsBytes = (kRbRows + 8) * (int)sizeof(double);  // rows ending in a block <= kRbRows + 1, + the open row
+
+struct RowBlocks {
+    int64_t n = 0, nnz = 0;
+    int num_blocks = 0;
+    int32_t *block_row = nullptr;   // device [num_blocks + 1]: first row of the block
+    int64_t *block_nnz = nullptr;   // device [num_blocks + 1]: first entry of the block
+    int32_t *walk_len = nullptr;    // device [num_blocks]
+    int32_t *col = nullptr;         // device [nnz]: sources, ascending inside each block
+    uint16_t *lrow = nullptr;       // device [nnz]: row of the entry relative to the block's first row
+};
+
+// Builds the blocks for a CSR with device row_ptr / col (already in the plan's internal id space).
+int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_ptr, const int32_t *col,
+                      hipStream_t stream);
+void row_blocks_destroy(RowBlocks *rb);
+
+// Sum of `v` over the 1024 threads of the block, valid in thread 0.  s_red: 16 doubles of LDS.
+__device__ __forceinline__ double block_sum_1024(double v, double *s_red)
+{
+#pragma unroll
+    for (int m = kWave / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, kWave);
+    const int wave = threadIdx.x / kWave;
+    if ((threadIdx.x & (kWave - 1)) == 0) s_red[wave] = v;
+    __syncthreads();
+    double t = 0.0;
+    if (threadIdx.x == 0)
+        for (int w = 0; w < kRbThreads / kWave; ++w) t += s_red[w];
+    return t;
+}
+
+template <typename Epi>
+__global__ __launch_bounds__(kRbThreads) void pr_rowblock_kernel(const int32_t *__restrict__ block_row,
+                                                                 const int64_t *__restrict__ block_nnz,
+                                                                 const int32_t *__restrict__ col,
+                                                                 const uint16_t *__restrict__ lrow, Epi epi,
+                                                                 double *__restrict__ block_carry,
+                                                                 double *__restrict__ block_stat)
+{
+    extern __shared__ double s_acc[];  // [rows ending in the block + 1 (the row left open)]
+    __shared__ double s_red[kRbThreads / kWave];
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const int r0 = block_row[b], nr = block_row[b + 1] - r0;
+    const int64_t e0 = block_nnz[b], e1 = block_nnz[b + 1];
+    for (int i = tid; i <= nr; i += kRbThreads) s_acc[i] = 0.0;
+    __syncthreads();
+
+    for (int64_t base = e0; base < e1; base += (int64_t)kRbThreads * kRbUnroll) {
+        int c[kRbUnroll], l[kRbUnroll];
+#pragma unroll
+        for (int k = 0; k < kRbUnroll; ++k) {
+            const int64_t e = base + tid + (int64_t)k * kRbThreads;
+            const bool ok = e < e1;
+            c[k] = ok ? __builtin_nontemporal_load(col + e) : -1;
+            l[k] = ok ? (int)__builtin_nontemporal_load(lrow + e) : 0;
+        }
+        double v[kRbUnroll];
+#pragma unroll
+        for (int k = 0; k < kRbUnroll; ++k) v[k] = c[k] >= 0 ? epi.load(c[k]) : 0.0;
+#pragma unroll
+        for (int k = 0; k < kRbUnroll; ++k)
+            if (c[k] >= 0) atomicAdd(&s_acc[l[k]], v[k]);
+    }
+    __syncthreads();
+
+    double stat = 0.0;
+    for (int i = tid; i < nr; i += kRbThreads) epi.row(r0 + i, s_acc[i], stat);
+    const double total = block_sum_1024(stat, s_red);
+    if (tid == 0) {
+        block_stat[b] = total;
+        block_carry[b] = s_acc[nr];
+    }
+}
+
+}  // namespace drone

@@ -1,0 +1,143 @@
+#include "pr_rowblock.h"
+
+#include <cstring>
+#include <rocprim/device/device_radix_sort.hpp>
+
+namespace drone {
+namespace {
+
+// Block b starts where the weighted merge path reaches b * kRbItems.  F(i) = W*i + row_ptr[i] is the path
+// position at which row i begins; inside row i the path first consumes its entries, then the row end (W).
+__global__ void rb_search_kernel(const int64_t *__restrict__ row_ptr, int64_t n, int64_t nnz, int num_blocks,
+                                 int32_t *__restrict__ block_row, int64_t *__restrict__ block_nnz)
+{
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b > num_blocks) return;
+    const int64_t total = (int64_t)kRbWeight * n + nnz;
+    int64_t d = (int64_t)b * kRbItems;
+    if (d > total) d = total;
+    int64_t lo = 0, hi = n;  // largest i in [0, n] with F(i) <= d
+    while (lo < hi) {
+        const int64_t mid = (lo + hi + 1) >> 1;
+        if ((int64_t)kRbWeight * mid + row_ptr[mid] <= d) lo = mid; else hi = mid - 1;
+    }
+    int64_t i = lo, e;
+    if (i >= n) {
+        i = n;
+        e = nnz;
+    } else {
+        const int64_t rem = d - ((int64_t)kRbWeight * i + row_ptr[i]);
+        const int64_t len = row_ptr[i + 1] - row_ptr[i];
+        if (rem <= len) {
+            e = row_ptr[i] + rem;  // boundary inside (or right after) the row's entries; its end comes later
+        } else {
+            e = row_ptr[i + 1];    // boundary inside the row-end cost: the whole row stays in the earlier block
+            i += 1;
+        }
+    }
+    block_row[b] = (int32_t)i;
+    block_nnz[b] = e;
+}
+
+__global__ void rb_walk_len_kernel(const int64_t *__restrict__ row_ptr, int num_blocks,
+                                   const int32_t *__restrict__ block_row, const int64_t *__restrict__ block_nnz,
+                                   int32_t *__restrict__ walk_len)
+{
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= num_blocks) return;
+    int wl = 0;
+    const int r0 = block_row[b], r1 = block_row[b + 1];
+    if (b > 0 && r1 > r0 && row_ptr[r0] < block_nnz[b]) {
+        int s = b - 1;
+        while (s > 0 && block_row[s + 1] == block_row[s]) --s;
+        wl = b - s;
+    }
+    walk_len[b] = wl;
+}
+
+// One work-group per block: key = (block << 32) | source, value = row relative to the block's first row.
+__global__ __launch_bounds__(256) void rb_keys_kernel(const int64_t *__restrict__ row_ptr, const int32_t *__restrict__ col,
+                                                      const int32_t *__restrict__ block_row,
+                                                      const int64_t *__restrict__ block_nnz,
+                                                      uint64_t *__restrict__ keys, uint16_t *__restrict__ lrow)
+{
+    const int b = blockIdx.x;
+    const int r0 = block_row[b], r1 = block_row[b + 1];
+    const int64_t e0 = block_nnz[b], e1 = block_nnz[b + 1];
+    for (int64_t e = e0 + threadIdx.x; e < e1; e += blockDim.x) {
+        int lo = r0, hi = r1;  // largest r in [r0, r1] with row_ptr[r] <= e
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (row_ptr[mid] <= e) lo = mid; else hi = mid - 1;
+        }
+        keys[e] = ((uint64_t)b << 32) | (uint32_t)col[e];
+        lrow[e] = (uint16_t)(lo - r0);
+    }
+}
+
+__global__ void rb_unpack_kernel(const uint64_t *__restrict__ keys, int64_t nnz, int32_t *__restrict__ col)
+{
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < nnz; e += (int64_t)gridDim.x * blockDim.x)
+        col[e] = (int32_t)(keys[e] & 0xFFFFFFFFull);
+}
+
+}  // namespace
+
+int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_ptr, const int32_t *col,
+                      hipStream_t stream)
+{
+    DRONE_REQUIRE(n > 0 && n < INT32_MAX && nnz >= 0 && nnz < (int64_t)UINT32_MAX, "sizes");
+    rb->n = n;
+    rb->nnz = nnz;
+    const int64_t total = (int64_t)kRbWeight * n + nnz;
+    rb->num_blocks = (int)ceil_div(total, kRbItems);
+    const int nb = rb->num_blocks;
+    uint64_t *keys = nullptr, *keys_sorted = nullptr;
+    uint16_t *lrow_in = nullptr;
+    void *temp = nullptr;
+    size_t temp_bytes = 0;
+    auto body = [&]() -> int {
+        const size_t e = (size_t)(nnz ? nnz : 1);
+        DRONE_HIP_TRY(hipMalloc(&rb->block_row, sizeof(int32_t) * ((size_t)nb + 1)));
+        DRONE_HIP_TRY(hipMalloc(&rb->block_nnz, sizeof(int64_t) * ((size_t)nb + 1)));
+        DRONE_HIP_TRY(hipMalloc(&rb->walk_len, sizeof(int32_t) * (size_t)nb));
+        DRONE_HIP_TRY(hipMalloc(&rb->col, sizeof(int32_t) * e));
+        DRONE_HIP_TRY(hipMalloc(&rb->lrow, sizeof(uint16_t) * e));
+        rb_search_kernel<<<(int)ceil_div(nb + 1, 256), 256, 0, stream>>>(row_ptr, n, nnz, nb, rb->block_row, rb->block_nnz);
+        rb_walk_len_kernel<<<(int)ceil_div(nb, 256), 256, 0, stream>>>(row_ptr, nb, rb->block_row, rb->block_nnz, rb->walk_len);
+        if (nnz > 0) {
+            DRONE_HIP_TRY(hipMalloc(&keys, sizeof(uint64_t) * e));
+            DRONE_HIP_TRY(hipMalloc(&keys_sorted, sizeof(uint64_t) * e));
+            DRONE_HIP_TRY(hipMalloc(&lrow_in, sizeof(uint16_t) * e));
+            rb_keys_kernel<<<nb, 256, 0, stream>>>(row_ptr, col, rb->block_row, rb->block_nnz, keys, lrow_in);
+            int bits = 32;
+            while (bits < 64 && (1ull << (bits - 32)) < (unsigned long long)nb) ++bits;
+            DRONE_HIP_TRY(rocprim::radix_sort_pairs(nullptr, temp_bytes, keys, keys_sorted, lrow_in, rb->lrow, (size_t)nnz, 0, bits, stream));
+            DRONE_HIP_TRY(hipMalloc(&temp, temp_bytes ? temp_bytes : 1));
+            DRONE_HIP_TRY(rocprim::radix_sort_pairs(temp, temp_bytes, keys, keys_sorted, lrow_in, rb->lrow, (size_t)nnz, 0, bits, stream));
+            rb_unpack_kernel<<<4096, 256, 0, stream>>>(keys_sorted, nnz, rb->col);
+        }
+        DRONE_HIP_TRY(hipGetLastError());
+        DRONE_HIP_TRY(hipStreamSynchronize(stream));
+        return DRONE_OK;
+    };
+    const int rc = body();
+    (void)hipFree(keys);
+    (void)hipFree(keys_sorted);
+    (void)hipFree(lrow_in);
+    (void)hipFree(temp);
+    if (rc != DRONE_OK) row_blocks_destroy(rb);
+    return rc;
+}
+
+void row_blocks_destroy(RowBlocks *rb)
+{
+    (void)hipFree(rb->block_row);
+    (void)hipFree(rb->block_nnz);
+    (void)hipFree(rb->walk_len);
+    (void)hipFree(rb->col);
+    (void)hipFree(rb->lrow);
+    *rb = RowBlocks{};
+}
+
+}  // namespace drone

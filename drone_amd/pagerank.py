@@ -123,7 +123,7 @@ class PRWorkerCUDA:
 class PullPlanF64:
     """fp64 pull PageRank over device tensors: row_ptr int64 [n+1], col_idx int32 [nnz], inv_outdeg f64 [n]."""
 
-    def __init__(self, row_ptr, col_idx, inv_outdeg, stream=0):
+    def __init__(self, row_ptr, col_idx, inv_outdeg, stream=0, deterministic=False):
         import torch
         assert row_ptr.is_cuda and row_ptr.dtype == torch.int64 and row_ptr.is_contiguous()
         assert col_idx.is_cuda and col_idx.dtype == torch.int32 and col_idx.is_contiguous()
@@ -135,8 +135,9 @@ class PullPlanF64:
         self.stream = stream
         torch.cuda.synchronize()
         h = C.c_void_p()
-        check(lib().drone_pr_plan_create(C.byref(h), self.n, self.nnz, row_ptr.data_ptr(), col_idx.data_ptr(),
-                                         inv_outdeg.data_ptr(), stream))
+        check(lib().drone_pr_plan_create_ex(C.byref(h), self.n, self.nnz, row_ptr.data_ptr(), col_idx.data_ptr(),
+                                            inv_outdeg.data_ptr(), 1 if deterministic else 0, stream))
+        self.deterministic = bool(deterministic)
         self.h = h
 
     def run(self, alpha, iters, out=None):

@@ -128,6 +128,13 @@ typedef struct drone_pr_plan drone_pr_plan;
  * Results are returned in the caller's vertex order. */
 int drone_pr_plan_create(drone_pr_plan **plan, int64_t n, int64_t nnz, const int64_t *row_ptr,
                          const int32_t *col_idx, const double *inv_outdeg, drone_stream_t stream);
+/* Same with flags.  By default the aggregation runs over row blocks whose entries are sorted by source
+ * (fastest; row sums are added in LDS in no fixed order, so the last bits may differ between runs, as
+ * with the reference's float atomics).  DRONE_PR_DETERMINISTIC selects the merge-path kernel, whose
+ * results are bitwise reproducible. */
+#define DRONE_PR_DETERMINISTIC 1
+int drone_pr_plan_create_ex(drone_pr_plan **plan, int64_t n, int64_t nnz, const int64_t *row_ptr,
+                            const int32_t *col_idx, const double *inv_outdeg, int flags, drone_stream_t stream);
 int drone_pr_plan_destroy(drone_pr_plan *plan);
 /* Runs `iters` iterations from r_0 = 1/N and writes r_iters to rank_out [n] (device).
  * Asynchronous on `stream`; allocates nothing. */
