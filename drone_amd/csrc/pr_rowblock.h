@@ -23,10 +23,13 @@
 namespace drone {
 
 constexpr int kRbThreads = 1024;
+// Shape chosen by measurement on R-MAT scale 24 (ms per iteration): 512 K entries / unroll 8: 1.07; 1 M / 8: 0.96;
+// 1 M / 4: 0.92; 1 M / 2: 0.88; 1 M / 1: 1.00; 2 M / 4: 1.02 (too few heavy blocks for 256 CUs).  Larger blocks reuse
+// popular lines more often; a small unroll keeps a wavefront's gathers close together in the sorted order.
 constexpr int kRbRows = 16384;       // most rows ending in one block (LDS accumulators: 128 KB)
-constexpr int kRbItems = 1 << 19;    // most entries in one block
+constexpr int kRbItems = 1 << 20;    // most entries in one block
 constexpr int kRbWeight = kRbItems / kRbRows;
-constexpr int kRbUnroll = 8;
+constexpr int kRbUnroll = 2;
 constexpr int kRbLdsBytes = (kRbRows + 8) * (int)sizeof(double);  // rows ending in a block <= kRbRows + 1, + the open row
 
 struct RowBlocks {
