@@ -146,9 +146,9 @@ def bench_gcn_step(steps, warmup):
         B = torch.rand((N, ld), device="cuda") * 2 - 1
         out = torch.empty((N, ld), device="cuda")
         ms = time_call(lambda: gcn.spmm(plan, rp, ci, val, B[:, :K], K=K, out=out[:, :K]), reps=5)
-        kernels.append(spmm_report(f"spmm (rows + band pieces) K={K}", N, nnz, K, ms))
-    spmm_ms = 2 * sum(k["ms"] for k in kernels)
-    spmm_bytes = 2 * sum(k["algorithmic_bytes"] for k in kernels)
+        kernels.append(spmm_report(f"spmm (rows + band pieces) K={K} ld={ld}", N, nnz, K, ms))
+    spmm_ms = 2 * sum(k["ms"] for k in kernels[:2])
+    spmm_bytes = 2 * sum(k["algorithmic_bytes"] for k in kernels[:2])
     gemms = []
     for (tA, tB, M, Nn, Kk, what) in ((0, 0, N, HID, FIN, "X*W1"), (0, 0, N, CLS, HID, "H1*W2"), (0, 1, N, HID, CLS, "dT2*W2^T"),
                                       (1, 0, HID, CLS, N, "H1^T*dT2"), (1, 0, FIN, HID, N, "X^T*dT1")):
@@ -303,7 +303,10 @@ def main():
                                f"damping 0.85, {args.iters} iterations per step",
                    "iterations_per_step": args.iters, "vertices": n, "edges": nnz},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS,
+                     # fabric bytes per launch: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by the 1 GiB copy
+                     # kernel; measured for this workload only (profiles/pr_rowblock_pagerank_c2.hbm_traffic.txt)
+                     "traffic": 5.08e9 if (args.scale == 24 and n == 16777216) else None,
                      "kernel": "pr_rowblock_kernel<PrF64Epi>",
                      "algorithmic_bytes_per_launch": bytes_iter, "mean_launch_ms": prof["mean_ms"],
                      "launches_timed": prof["launches"]},

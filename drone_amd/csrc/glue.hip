@@ -162,9 +162,17 @@ __global__ __launch_bounds__(kThreads) void accuracy_kernel(int n, int classes, 
             }
         }
     }
-    if (counts && lane == 0 && total) {
-        atomicAdd(&counts[0], correct);
-        atomicAdd(&counts[1], total);
+    // one pair of atomics per work-group, not per wavefront: they all hit the same two addresses
+    __shared__ int s_correct[kThreads / kWave], s_total[kThreads / kWave];
+    if (lane == 0) { s_correct[wave] = correct; s_total[wave] = total; }
+    __syncthreads();
+    if (counts && threadIdx.x == 0) {
+        int c = 0, t = 0;
+        for (int w = 0; w < kThreads / kWave; ++w) { c += s_correct[w]; t += s_total[w]; }
+        if (t) {
+            atomicAdd(&counts[0], c);
+            atomicAdd(&counts[1], t);
+        }
     }
 }
 
@@ -284,7 +292,7 @@ extern "C" int drone_accuracy_f32(int n, int classes, const float *logits, int l
     DRONE_REQUIRE(n > 0 && classes > 0 && logits && ld >= classes, "operands");
     hipStream_t s = as_stream(stream);
     int blocks = (int)ceil_div(n, kThreads / kWave);
-    if (blocks > 4096) blocks = 4096;
+    if (blocks > 1024) blocks = 1024;
     accuracy_kernel<<<blocks, kThreads, 0, s>>>(n, classes, logits, ld, truth, pred, counts);
     DRONE_HIP_TRY(hipGetLastError());
     return DRONE_OK;
