@@ -122,6 +122,19 @@ SIGNATURES = {
     "drone_fill_normal_f32": (_I, [_P, _I64, _U64]),
     "drone_fill_randint_i32": (_I, [_P, _I64, _U64, C.c_int32]),
     "drone_stream_copy_f64": (_I, [_P, _P, _I64, _P]),
+    "drone_load_edge_file": (_I, [C.c_char_p, C.POINTER(C.POINTER(_I)), C.POINTER(C.POINTER(_I)), C.POINTER(_I)]),
+    "drone_load_master_file": (_I, [C.c_char_p, C.POINTER(C.POINTER(_I)), C.POINTER(C.POINTER(_I)), C.POINTER(C.POINTER(_I)),
+                                    C.POINTER(_I), C.POINTER(_I)]),
+    "drone_load_mirror_file": (_I, [C.c_char_p, C.POINTER(C.POINTER(_I)), C.POINTER(C.POINTER(_I)), C.POINTER(_I)]),
+    "drone_load_degree_file": (_I, [C.c_char_p, C.POINTER(C.POINTER(_I)), C.POINTER(_I)]),
+    "drone_free_host": (None, [_P]),
+    "drone_pr_worker_create": (_I, [C.POINTER(_P), C.c_char_p, _I, _I, _I]),
+    "drone_pr_worker_peval": (Response, [_P]),
+    "drone_pr_worker_inceval": (Response, [_P]),
+    "drone_pr_worker_local_size": (_I, [_P]),
+    "drone_pr_worker_read": (_I, [_P, _P, _P]),
+    "drone_pr_worker_run_f64": (_I, [_P, _D, _I, _P]),
+    "drone_pr_worker_destroy": (_I, [_P]),
     "drone_timer_create": (_I, [C.POINTER(_P)]),
     "drone_timer_start": (_I, [_P, _P]),
     "drone_timer_stop": (_I, [_P, _P]),
@@ -139,6 +152,13 @@ def lib():
             raise DroneError(
                 f"{_SO} is missing: build it with `make -C drone_amd/csrc` (or __graft_entry__.build()). "
                 "There is no CPU fallback.")
+        # PyTorch-ROCm ships its own copy of the HIP runtime.  A process must not end up with two of them (the second
+        # one finds no device), so when torch is installed it is imported first and this library binds to the
+        # runtime torch has already loaded; without torch the system runtime is used.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         handle = C.CDLL(_SO)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(handle, name)

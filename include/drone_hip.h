@@ -287,6 +287,34 @@ int drone_timer_elapsed_ms(drone_timer *t, float *ms); /* synchronises on the st
 int drone_timer_destroy(drone_timer *t);
 int drone_device_synchronize(void);
 
+/* ====================================================================================== */
+/* E. Partition files and the pr_cuda worker's compute side (host code)                   */
+/* ====================================================================================== */
+/* Text formats written by the EBV partitioner and read by DRONE/src/graph/cuda_graph.go:15-164.  As in the
+ * Go loader only lines terminated by '\n' are read, a '\r' ends the line early, tokens are separated by single
+ * spaces.  Output arrays are malloc'd; release them with drone_free_host.  A malformed line makes the Go loader
+ * log.Fatal; here it returns DRONE_ERR_INVALID with file:line in drone_last_error_string(). */
+int drone_load_edge_file(const char *path, int **u, int **v, int *edge_count);          /* G.<i>: "src dst[ w]"      */
+int drone_load_master_file(const char *path, int **master_vertex, int **mirror_number,  /* Master.<i>: "v w1 w2 .."  */
+                           int **mirror_workers, int *master_size, int *mirror_worker_size);
+int drone_load_mirror_file(const char *path, int **mirror_vertex, int **master_worker,  /* Mirror.<i>: "v w[ backup]" */
+                           int *mirror_size);
+int drone_load_degree_file(const char *path, int **degree, int *count);                 /* out_degree.txt           */
+void drone_free_host(void *p);
+/* DRONE/src/worker/PRWorkerCUDA.go:115-175 (newPRWorkerCUDA) without the gRPC peers: reads
+ * <data_path>/G.<self_id-1>, Master.<self_id-1>, Mirror.<self_id-1>, out_degree.txt, builds the graph, loads the
+ * out-degrees.  self_id counts from 1 (0 is the master); worker_num must be 1 and the Master/Mirror files empty.
+ * peval / inceval are PRWorkerCUDA.go:52-65 / :76-88 minus the SuperStepFinish RPC. */
+typedef struct drone_pr_worker drone_pr_worker;
+int drone_pr_worker_create(drone_pr_worker **w, const char *data_path, int self_id, int worker_num,
+                           int global_vertex_size);
+Response drone_pr_worker_peval(drone_pr_worker *w);
+Response drone_pr_worker_inceval(drone_pr_worker *w);
+int drone_pr_worker_local_size(drone_pr_worker *w);
+int drone_pr_worker_read(drone_pr_worker *w, int *global_ids, float *pr); /* host [local size] each, may be NULL */
+int drone_pr_worker_run_f64(drone_pr_worker *w, double alpha, int iters, double *rank_out); /* host [local size] */
+int drone_pr_worker_destroy(drone_pr_worker *w);
+
 #ifdef __cplusplus
 }
 #endif

@@ -81,10 +81,11 @@ def test_spmm_against_oracle(T, oracle, K, ld_pad):
     assert np.all(got[np.diff(m.indptr) == 0] == 0.0)             # empty rows are written as zero (beta = 0)
 
 
-@pytest.mark.parametrize("K", [41, 128, 256])
+@pytest.mark.parametrize("K", [8, 16, 41, 64, 128, 256])
 def test_spmm_long_rows_split_and_alpha_beta(T, oracle, K):
-    """Rows above 512 entries take the band-piece path: several of them, several column bands (a band holds
-    2 MB / (4 K) columns), pieces longer than 2048 entries, mixed with short and empty rows."""
+    """Rows above 512 entries take the band path: several of them, several column bands (a band holds
+    2 MB / (4 K) columns), mixed with short and empty rows.  The long rows are dense enough in every band for the
+    LDS-staged kernel, one lane-group width per K."""
     n = 9000
     m = random_csr(5, 40, n, 0.002, hub=[8500, 600, 3000, 513, 512])
     assert np.diff(m.indptr).max() > 4096
@@ -97,6 +98,16 @@ def test_spmm_long_rows_split_and_alpha_beta(T, oracle, K):
     a = run_spmm(T, m, B)
     b = run_spmm(T, m, B)
     np.testing.assert_array_equal(a, b)                             # fixed summation order: bitwise repeatable
+
+
+def test_spmm_sparse_long_rows_use_unstaged_pieces(T, oracle):
+    """Long rows that are too sparse in their bands for staging: pieces of up to 2048 entries straight from L2."""
+    n = 300000
+    m = random_csr(11, 30, n, 0.00002, hub=[5000, 2500, 700])
+    B = np.random.default_rng(4).uniform(-1, 1, (n, 128)).astype(np.float32)
+    got = run_spmm(T, m, B)
+    ref = oracle.spmm_f64acc(m.indptr, m.indices, m.data, B)
+    assert rel_err(got, ref, oracle.spmm_f64acc(m.indptr, m.indices, np.abs(m.data), np.abs(B))) <= 1e-4
 
 
 def test_spmm_plan_update_values(T, oracle):
