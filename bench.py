@@ -102,7 +102,7 @@ def spmm_report(name, n, nnz, K, ms):
             "gflops": 2.0 * nnz * K / (ms * 1e-3) / 1e9}
 
 
-def bench_gcn_step(steps, warmup):
+def bench_gcn_step(steps, warmup, cpu_baseline=False):
     """configs[3]: 2-layer GCN training step on the dense power-law graph (232,965 vertices)."""
     import numpy as np
     import torch
@@ -159,9 +159,25 @@ def bench_gcn_step(steps, warmup):
         fl = 2.0 * M * Nn * Kk
         gemms.append({"gemm": what, "M": M, "N": Nn, "K": Kk, "ms": ms, "tflops": fl / (ms * 1e-3) / 1e12,
                       "frac_of_fp32_mfma_peak": fl / (ms * 1e-3) / 1e12 / 157.3})
+    # CPU baseline: the oracle's CSR SpMM of identical semantics (OpenMP, all host cores) on the same matrix, K=128
+    cpu = None
+    if cpu_baseline:
+        from oracle import oracle as orc
+        orc.build()
+        h_rp, h_ci, h_val = rp.cpu().numpy(), ci.cpu().numpy(), val.cpu().numpy()
+        Bh = rmat.uniform_f32((N, HID), seed=7)
+        t0 = time.time()
+        orc.spmm_f32(h_rp, h_ci, h_val, Bh)
+        dt = time.time() - t0
+        threads = min(16, os.cpu_count() or 1)
+        cpu = {"value": dt * 1e3, "unit": "ms per SpMM (K=128)", "cores": threads, "kind": "port",
+               "sample": f"oracle fp32 CSR SpMM (OpenMP) on the same {nnz}-entry matrix, one product, {dt:.1f} s",
+               "gpu_ms": kernels[0]["ms"]}
+        log(f"cpu baseline SpMM K=128: {dt*1e3:.0f} ms on {threads} threads (GPU {kernels[0]['ms']:.2f} ms)")
     plan.close()
     model.close()
-    return {"workload": f"2-layer GCN training step (configs[3]): N={N}, nnz={nnz}, 602->128->41, ReLU, dropout 0.5, "
+    return {"cpu_baseline_spmm": cpu,
+            "workload": f"2-layer GCN training step (configs[3]): N={N}, nnz={nnz}, 602->128->41, ReLU, dropout 0.5, "
                         "softmax cross-entropy, SGD lr 0.01, fp32",
             "step_ms": step_ms, "steps": steps, "setup_ms_one_off": setup_s * 1e3, "spmm_kernels": kernels,
             "spmm_ms_per_step": spmm_ms,
@@ -325,7 +341,8 @@ def main():
     del x, out, plan
     torch.cuda.empty_cache()
     if args.suite in ("default", "full"):
-        result["gcn_step"] = bench_gcn_step(steps=max(3, args.steps), warmup=max(1, args.warmup))
+        result["gcn_step"] = bench_gcn_step(steps=max(3, args.steps), warmup=max(1, args.warmup),
+                                            cpu_baseline=not args.no_cpu_baseline)
         torch.cuda.empty_cache()
     if args.suite == "full":
         result["gcn_layer"] = bench_gcn_layer()

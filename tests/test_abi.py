@@ -105,3 +105,23 @@ def test_fill_generators():
     z = rmat.randint_i32(100000, seed=5, bound=41)
     assert z.min() == 0 and z.max() == 40
     np.testing.assert_array_equal(rmat.uniform_f32(50, seed=3), x.ravel()[:50])
+
+
+def test_gcn_entry_points_validate_arguments_on_the_host():
+    """Bad arguments are rejected before any device work (runs without a GPU)."""
+    L = _lib.lib()
+    h = C.c_void_p()
+    assert L.drone_spmm_plan_create(C.byref(h), -1, 4, 0, None, None, None, 16, None) == -1
+    assert L.drone_spmm_plan_create(C.byref(h), 4, 4, 0, None, None, None, 16, None) == -1      # null row_ptr
+    assert L.drone_spmm_csr_f32(None, None, None, None, None, 1, None, 1, 1, 1.0, 0.0, None) == -1
+    assert b"plan" in L.drone_last_error_string()
+    assert L.drone_sgemm_rm_f32(0, 0, 4, 4, 4, 1.0, None, 2, None, 4, 0.0, None, 4, None) == -1  # lda < K
+    assert L.drone_sgemm_rm_f32(0, 0, 0, 4, 4, 1.0, None, 4, None, 4, 0.0, None, 4, None) == 0   # empty product
+    assert L.drone_cross_entropy_f32(0, 3, None, 3, None, None, 3, 1.0, None, None, None) == -1
+    assert L.drone_dropout_mask(None, 0, 1, 0, 1.5, None) == -1                                   # p out of range
+    assert L.drone_adam_step_f32(None, None, None, None, 0, 0, 0.0, 0.01, 0.9, 0.999, 1e-8, 0, None) == -1
+    assert L.drone_spmm_bytes(10, 100, 8) == 4 * 11 + 8 * 100 + 8 * 10 * 8
+    assert L.drone_sgemm_flops(3, 4, 5) == 120
+    cfg = _lib.GcnConfig(0, 1, 1, 1, 0.5, 0.01, 0.0, 0, 1, 0, 1)
+    assert L.drone_gcn_create(C.byref(h), C.byref(cfg), 0, None, None, None, None, None, 1, None, None, None, None, None) == -1
+    assert L.drone_pr_plan_create_ex(C.byref(h), 10, 0, None, None, None, 4, None) == -1
