@@ -157,3 +157,68 @@ def test_training_reduces_loss_with_adam_and_eval_is_pure(T, oracle):
     assert e1 == e2 and e1[1] > 1.0 / cls + 0.1
     np.testing.assert_array_equal(m.tensor("W1"), w_before)
     m.close()
+
+
+def test_full_size_properties_config4(T):
+    """Fourth configuration at full size (232,965 vertices, ~229 M entries, 602 -> 128 -> 41): properties that
+    need no CPU oracle - A_hat * 1 against fp64 row sums, forward/backward adjointness <A^T X, Y> = <X, A Y>,
+    the big GEMMs against torch.matmul in fp32/fp64, and a bitwise repeatable, finite training step."""
+    torch = T
+    from drone_amd import gcn, graphs, rmat
+    N, FIN, HID, CLS = 232965, 602, 128, 41
+    g = graphs.gcn_graph_torch(18, 0, seed=4, n=N, n_edges=221_000_000)
+    rp, ci, deg, nnz = g["rp"], g["ci"], g["deg"], g["nnz"]
+    assert 110e6 < (nnz - N) / 2 < 120e6                      # ~114.6 M undirected edges, as the configuration says
+    val = gcn.edge_values(rp, ci, deg, deg)
+    rpT, ciT, vT = gcn.csr_transpose(N, N, rp, ci, val)
+    assert torch.equal(rpT, rp) and torch.equal(ciT, ci) and torch.equal(vT, val)      # symmetric graph
+    plan = gcn.SpmmPlan(rp, ci, val, N, max_k=HID)
+    # A * ones == row sums (fp64 prefix sums as the reference value)
+    ones = torch.ones((N, 4), device="cuda")
+    got = gcn.spmm(plan, rp, ci, val, ones)
+    cs = torch.cumsum(val.double(), 0)
+    cs = torch.cat([torch.zeros(1, dtype=torch.float64, device="cuda"), cs])
+    rows = cs[rp[1:].long()] - cs[rp[:-1].long()]
+    assert float(((got[:, 0].double() - rows).abs() / rows.abs().clamp(min=1e-30)).max()) <= 1e-4
+    # adjointness at K = 41 and 128
+    for K, ld in ((CLS, 44), (HID, HID)):
+        X = (torch.rand((N, ld), device="cuda") * 2 - 1)[:, :K]
+        Y = (torch.rand((N, ld), device="cuda") * 2 - 1)[:, :K]
+        AX = torch.empty((N, ld), device="cuda")[:, :K]
+        AY = torch.empty((N, ld), device="cuda")[:, :K]
+        gcn.spmm(plan, rp, ci, val, X, K=K, out=AX)
+        gcn.spmm(plan, rp, ci, val, Y, K=K, out=AY)
+        lhs = float((AX.double() * Y.double()).sum())
+        rhs = float((X.double() * AY.double()).sum())
+        scale = float((AX.double().abs() * Y.double().abs()).sum())
+        assert abs(lhs - rhs) <= 1e-4 * scale
+        again = torch.empty((N, ld), device="cuda")[:, :K]       # same leading dimension -> same lane layout
+        gcn.spmm(plan, rp, ci, val, X, K=K, out=again)
+        assert torch.equal(again, AX)                          # fixed summation order
+    plan.close()
+    # the step's GEMM shapes against torch (fp64 reference on a row sample, fp32 on the whole)
+    Xf = torch.from_numpy(rmat.normal_f32((N, FIN), seed=4)).cuda()
+    W1 = torch.from_numpy(rmat.uniform_f32((FIN, HID), seed=41, lo=-0.09, hi=0.09)).cuda()
+    T1 = gcn.sgemm(0, 0, Xf, W1)
+    ref = Xf[:4096].double() @ W1.double()
+    assert float((T1[:4096].double() - ref).abs().max() / ref.abs().max()) <= 1e-4
+    assert float((T1 - Xf @ W1).abs().max() / T1.abs().max()) <= 1e-4
+    G = torch.rand((N, HID), device="cuda") - 0.5
+    dW = gcn.sgemm(1, 0, Xf, G)                                # weight gradient: reduction over 232,965 rows
+    refw = Xf.double().T @ G.double()
+    assert float((dW.double() - refw).abs().max() / refw.abs().max()) <= 1e-4
+    # one full training step, twice from the same state: finite and bitwise repeatable
+    label = torch.from_numpy(rmat.randint_i32(N, seed=43, bound=CLS)).cuda()
+    split = torch.from_numpy(np.where(rmat.uniform_f32(N, seed=44, lo=0, hi=1) < 0.66, 1, 2).astype(np.int32)).cuda()
+    W2 = torch.from_numpy(rmat.uniform_f32((HID, CLS), seed=42, lo=-0.18, hi=0.18)).cuda()
+    losses = []
+    for _ in range(2):
+        m = gcn.GcnModel(rp, ci, deg, deg, Xf, label, split, W1, W2, dropout=0.5, lr=0.01, use_dropout=True,
+                         use_adam=False, mean_gradient=True, seed=4)
+        m.set_truth(1)
+        m.train_step_async()
+        loss, acc = m.read_metrics()
+        losses.append((loss, float(np.abs(m.tensor("dW1")).sum())))
+        m.close()
+    assert np.isfinite(losses[0][0]) and abs(losses[0][0] - np.log(CLS)) < 0.5
+    assert losses[0] == losses[1]
