@@ -135,6 +135,7 @@ SIGNATURES = {
     "drone_pr_worker_read": (_I, [_P, _P, _P]),
     "drone_pr_worker_run_f64": (_I, [_P, _D, _I, _P]),
     "drone_pr_worker_destroy": (_I, [_P]),
+    "drone_copy_to_host": (_I, [_P, _P, C.c_size_t]),
     "drone_timer_create": (_I, [C.POINTER(_P)]),
     "drone_timer_start": (_I, [_P, _P]),
     "drone_timer_stop": (_I, [_P, _P]),

@@ -108,45 +108,51 @@ extern "C" int drone_pr_plan_create_ex(drone_pr_plan **out, int64_t n, int64_t n
     DRONE_REQUIRE((flags & ~DRONE_PR_DETERMINISTIC) == 0, "unknown flag");
     drone_pr_plan *p = new drone_pr_plan();
     p->deterministic = (flags & DRONE_PR_DETERMINISTIC) != 0 || nnz >= (int64_t)UINT32_MAX;
-    DRONE_HIP_TRY(hipGetDevice(&p->device));
     p->n = n;
     p->nnz = nnz;
     p->inv_user = inv_outdeg;
     hipStream_t s = as_stream(stream);
-    int rc = relabel_create(&p->rl, n, nnz, row_ptr, col_idx, s);
-    if (rc != DRONE_OK) { delete p; return rc; }
-    if (p->deterministic) {
-        rc = merge_tiling_create<int64_t>(&p->mt, n, nnz, p->rl.row_ptr, kSpmvBlock * kPrIpt, s);
-        if (rc != DRONE_OK) { drone_pr_plan_destroy(p); return rc; }
-        p->units = p->mt.num_tiles;
-    } else {
-        rc = row_blocks_create(&p->rb, n, nnz, p->rl.row_ptr, p->rl.col, s);
-        if (rc != DRONE_OK) { drone_pr_plan_destroy(p); return rc; }
-        p->units = p->rb.num_blocks;
-        // the row-ordered copy is only needed to build the blocks
-        (void)hipFree(p->rl.row_ptr);
-        (void)hipFree(p->rl.col);
-        p->rl.row_ptr = nullptr;
-        p->rl.col = nullptr;
-        DRONE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&pr_rowblock_kernel<PrF64Epi>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, kRbLdsBytes));
-    }
-    {
+    const auto build = [&]() -> int {
+        DRONE_HIP_TRY(hipGetDevice(&p->device));
+        int rc = relabel_create(&p->rl, n, nnz, row_ptr, col_idx, s);
+        if (rc != DRONE_OK) return rc;
+        if (p->deterministic) {
+            rc = merge_tiling_create<int64_t>(&p->mt, n, nnz, p->rl.row_ptr, kSpmvBlock * kPrIpt, s);
+            if (rc != DRONE_OK) return rc;
+            p->units = p->mt.num_tiles;
+        } else {
+            rc = row_blocks_create(&p->rb, n, nnz, p->rl.row_ptr, p->rl.col, s);
+            if (rc != DRONE_OK) return rc;
+            p->units = p->rb.num_blocks;
+            // the row-ordered copy is only needed to build the blocks
+            (void)hipFree(p->rl.row_ptr);
+            (void)hipFree(p->rl.col);
+            p->rl.row_ptr = nullptr;
+            p->rl.col = nullptr;
+            DRONE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&pr_rowblock_kernel<PrF64Epi>),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, kRbLdsBytes));
+        }
         MergeTiling shape;  // scratch is sized by the number of work units of the active mode
         shape.num_tiles = p->units;
         rc = merge_scratch_create(&p->ms, shape, sizeof(double));
-        if (rc != DRONE_OK) { drone_pr_plan_destroy(p); return rc; }
+        if (rc != DRONE_OK) return rc;
+        DRONE_HIP_TRY(hipMalloc(&p->c[0], sizeof(double) * (size_t)n));
+        DRONE_HIP_TRY(hipMalloc(&p->c[1], sizeof(double) * (size_t)n));
+        DRONE_HIP_TRY(hipMalloc(&p->dang, sizeof(double)));
+        DRONE_HIP_TRY(hipMalloc(&p->inv, sizeof(double) * (size_t)n));
+        DRONE_HIP_TRY(hipStreamSynchronize(s));
+        return DRONE_OK;
+    };
+    const int rc = build();
+    if (rc != DRONE_OK) {  // the error text is already recorded; release whatever was built
+        drone_pr_plan_destroy(p);
+        return rc;
     }
-    DRONE_HIP_TRY(hipMalloc(&p->c[0], sizeof(double) * (size_t)n));
-    DRONE_HIP_TRY(hipMalloc(&p->c[1], sizeof(double) * (size_t)n));
-    DRONE_HIP_TRY(hipMalloc(&p->dang, sizeof(double)));
-    DRONE_HIP_TRY(hipMalloc(&p->inv, sizeof(double) * (size_t)n));
     // the init kernel parks its block partials in block_stat: never more blocks than it holds
     int ib = (int)ceil_div(n, kSpmvBlock * 8);
     const int fb = fixup_blocks(p->units);
     p->init_blocks = ib < fb ? ib : fb;
     if (p->init_blocks < 1) p->init_blocks = 1;
-    DRONE_HIP_TRY(hipStreamSynchronize(s));
     *out = p;
     return DRONE_OK;
 }

@@ -128,6 +128,14 @@ extern "C" int drone_stream_copy_f64(double *dst, const double *src, int64_t n, 
     return DRONE_OK;
 }
 
+extern "C" int drone_copy_to_host(void *dst_host, const void *src_device, size_t bytes)
+{
+    clear_error();
+    DRONE_REQUIRE(bytes == 0 || (dst_host && src_device), "null operand");
+    if (bytes) DRONE_HIP_TRY(hipMemcpy(dst_host, src_device, bytes, hipMemcpyDeviceToHost));
+    return DRONE_OK;
+}
+
 struct drone_timer {
     hipEvent_t a, b;
 };

@@ -183,17 +183,15 @@ class GcnModel:
     def tensor(self, name):
         """Host copy (numpy) of a named tensor, logical columns only."""
         import numpy as np
-        import torch
-        from .pagerank import lib_hip_memcpy_d2d
+        from .pagerank import copy_to_host
         ptr, rows, cols, ld = C.c_void_p(), C.c_int(0), C.c_int(0), C.c_int(0)
         check(lib().drone_gcn_tensor(self.h, name.encode(), C.byref(ptr), C.byref(rows), C.byref(cols), C.byref(ld)))
-        dtype = {"relu_mask": torch.uint8, "keep1": torch.uint8, "truth": torch.int32, "rpT": torch.int32,
-                 "ciT": torch.int32}.get(name, torch.float32)
-        buf = torch.empty((rows.value, ld.value), dtype=dtype, device="cuda")
-        torch.cuda.synchronize()
-        lib_hip_memcpy_d2d(buf.data_ptr(), ptr.value, buf.numel() * buf.element_size())
-        out = buf[:, :cols.value].cpu().numpy()
-        return out[0] if rows.value == 1 and name in ("truth", "rpT", "ciT", "val", "valT") else np.ascontiguousarray(out)
+        dtype = {"relu_mask": np.uint8, "keep1": np.uint8, "truth": np.int32, "rpT": np.int32,
+                 "ciT": np.int32}.get(name, np.float32)
+        check(lib().drone_device_synchronize())
+        buf = copy_to_host(ptr.value, rows.value * ld.value, dtype).reshape(rows.value, ld.value)
+        out = buf[:, :cols.value]
+        return out[0].copy() if rows.value == 1 and name in ("truth", "rpT", "ciT", "val", "valT") else np.ascontiguousarray(out)
 
     def close(self):
         if self.h:

@@ -44,26 +44,11 @@ def CUDA_PR_IncEVal(g, values, workerId, workerNum, comm):
     return lib().PR_IncEVal(g, C.byref(values), int(workerId), int(workerNum), C.byref(comm))
 
 
-def _copy_out(ptr, n, dtype):
-    """Device -> host copy of n elements (torch is only the memcpy here)."""
-    import torch
-    out = torch.empty(n, dtype=dtype, device="cuda")
-    lib_hip_memcpy_d2d(out.data_ptr(), ptr, out.element_size() * n)
-    return out.cpu().numpy()
-
-
-_hip = None
-
-
-def lib_hip_memcpy_d2d(dst, src, nbytes):
-    global _hip
-    if _hip is None:
-        _hip = C.CDLL("libamdhip64.so")
-        _hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
-        _hip.hipMemcpy.restype = C.c_int
-    rc = _hip.hipMemcpy(C.c_void_p(dst), C.c_void_p(src), C.c_size_t(nbytes), 3)  # hipMemcpyDeviceToDevice
-    if rc != 0:
-        raise _lib.DroneError(f"hipMemcpy failed with {rc}")
+def copy_to_host(ptr, n, dtype):
+    """Host numpy copy of n elements at device address ptr."""
+    out = np.empty(n, dtype)
+    check(lib().drone_copy_to_host(out.ctypes.data_as(C.c_void_p), C.c_void_p(ptr), out.nbytes))
+    return out
 
 
 class PRWorkerCUDA:
@@ -88,12 +73,10 @@ class PRWorkerCUDA:
 
     # --- state read-back for tests
     def _f32(self, ptr, n=None):
-        import torch
-        return _copy_out(ptr, self.n if n is None else n, torch.float32)
+        return copy_to_host(ptr, self.n if n is None else n, np.float32)
 
     def _i32(self, ptr, n=None):
-        import torch
-        return _copy_out(ptr, self.n if n is None else n, torch.int32)
+        return copy_to_host(ptr, self.n if n is None else n, np.int32)
 
     def state(self):
         v, g = self.values, self.g.contents

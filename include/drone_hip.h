@@ -278,6 +278,9 @@ int drone_fill_randint_i32(int32_t *out, int64_t n, uint64_t seed, int32_t bound
  * traffic that profiler byte counters can be scaled by, and a measured stream-bandwidth reference. */
 int drone_stream_copy_f64(double *dst, const double *src, int64_t n, drone_stream_t stream);
 
+/* Synchronous device-to-host copy (for hosts that have no HIP binding of their own, e.g. to read PRValues). */
+int drone_copy_to_host(void *dst_host, const void *src_device, size_t bytes);
+
 /* HIP-event stopwatch on a stream (bench harness plumbing). */
 typedef struct drone_timer drone_timer;
 int drone_timer_create(drone_timer **t);
