@@ -260,7 +260,8 @@ extern "C" int drone_pr_run_f64(drone_pr_plan *p, double alpha, int iters, doubl
                 p->n, p->nnz, p->mt.tile_row, p->rl.row_ptr, p->rl.col, epi, carry, p->ms.tile_stat);
         } else {
             pr_rowblock_kernel<PrF64Epi><<<p->rb.num_blocks, kRbThreads, kRbLdsBytes, s>>>(
-                p->rb.block_row, p->rb.block_nnz, p->rb.col, p->rb.lrow, epi, carry, p->ms.tile_stat);
+                p->rb.block_row, p->rb.block_nnz, p->rb.col, p->rb.lrow, p->rb.packed, p->rb.batch_base, p->rb.block_batch,
+                p->rb.block_wide, epi, carry, p->ms.tile_stat);
         }
         if (prof) DRONE_HIP_TRY(hipEventRecord(p->ev1[p->prof_n++], s));
         spmv_fixup_kernel<double, PrF64Epi><<<fb, kSpmvBlock, 0, s>>>(

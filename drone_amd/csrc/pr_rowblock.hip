@@ -1,6 +1,7 @@
 #include "pr_rowblock.h"
 
 #include <cstring>
+#include <vector>
 #include <rocprim/device/device_radix_sort.hpp>
 
 namespace drone {
@@ -75,6 +76,31 @@ __global__ __launch_bounds__(256) void rb_keys_kernel(const int64_t *__restrict_
     }
 }
 
+// One thread per 64-entry batch: base = first source of the batch, packed = lrow << 16 | (source - base);
+// a batch that spans more than 65,535 ids flags its block as wide.
+__global__ void rb_pack_kernel(int num_blocks, const int64_t *__restrict__ block_nnz, const int32_t *__restrict__ block_batch,
+                               const int32_t *__restrict__ col, const uint16_t *__restrict__ lrow,
+                               uint32_t *__restrict__ packed, int32_t *__restrict__ batch_base,
+                               int32_t *__restrict__ block_wide)
+{
+    const int b = blockIdx.x;
+    const int64_t e0 = block_nnz[b], e1 = block_nnz[b + 1];
+    const int batches = block_batch[b + 1] - block_batch[b];
+    for (int j = threadIdx.x; j < batches; j += blockDim.x) {
+        const int64_t s = e0 + (int64_t)j * 64;
+        const int64_t t = s + 64 < e1 ? s + 64 : e1;
+        const int32_t base = col[s];
+        batch_base[block_batch[b] + j] = base;
+        bool overflow = false;
+        for (int64_t e = s; e < t; ++e) {
+            const int32_t off = col[e] - base;  // sources ascend inside a block
+            if (off > 0xFFFF) overflow = true;
+            packed[e] = ((uint32_t)lrow[e] << 16) | (uint32_t)(off & 0xFFFF);
+        }
+        if (overflow) block_wide[b] = 1;
+    }
+}
+
 __global__ void rb_unpack_kernel(const uint64_t *__restrict__ keys, int64_t nnz, int32_t *__restrict__ col)
 {
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < nnz; e += (int64_t)gridDim.x * blockDim.x)
@@ -117,6 +143,21 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
             DRONE_HIP_TRY(rocprim::radix_sort_pairs(temp, temp_bytes, keys, keys_sorted, lrow_in, rb->lrow, (size_t)nnz, 0, bits, stream));
             rb_unpack_kernel<<<4096, 256, 0, stream>>>(keys_sorted, nnz, rb->col);
         }
+        // packed 4-byte entries
+        DRONE_HIP_TRY(hipMalloc(&rb->block_batch, sizeof(int32_t) * ((size_t)nb + 1)));
+        DRONE_HIP_TRY(hipMalloc(&rb->block_wide, sizeof(int32_t) * (size_t)nb));
+        DRONE_HIP_TRY(hipMalloc(&rb->packed, sizeof(uint32_t) * e));
+        DRONE_HIP_TRY(hipMemsetAsync(rb->block_wide, 0, sizeof(int32_t) * (size_t)nb, stream));
+        std::vector<int64_t> h_nnz((size_t)nb + 1);
+        DRONE_HIP_TRY(hipMemcpyAsync(h_nnz.data(), rb->block_nnz, sizeof(int64_t) * h_nnz.size(), hipMemcpyDeviceToHost, stream));
+        DRONE_HIP_TRY(hipStreamSynchronize(stream));
+        std::vector<int32_t> h_batch((size_t)nb + 1, 0);
+        for (int b = 0; b < nb; ++b) h_batch[b + 1] = h_batch[b] + (int32_t)ceil_div(h_nnz[b + 1] - h_nnz[b], 64);
+        DRONE_HIP_TRY(hipMalloc(&rb->batch_base, sizeof(int32_t) * (size_t)(h_batch[nb] ? h_batch[nb] : 1)));
+        DRONE_HIP_TRY(hipMemcpyAsync(rb->block_batch, h_batch.data(), sizeof(int32_t) * h_batch.size(), hipMemcpyHostToDevice, stream));
+        if (nnz > 0)
+            rb_pack_kernel<<<nb, 256, 0, stream>>>(nb, rb->block_nnz, rb->block_batch, rb->col, rb->lrow, rb->packed,
+                                                  rb->batch_base, rb->block_wide);
         DRONE_HIP_TRY(hipGetLastError());
         DRONE_HIP_TRY(hipStreamSynchronize(stream));
         return DRONE_OK;
@@ -137,6 +178,10 @@ void row_blocks_destroy(RowBlocks *rb)
     (void)hipFree(rb->walk_len);
     (void)hipFree(rb->col);
     (void)hipFree(rb->lrow);
+    (void)hipFree(rb->packed);
+    (void)hipFree(rb->batch_base);
+    (void)hipFree(rb->block_batch);
+    (void)hipFree(rb->block_wide);
     *rb = RowBlocks{};
 }
 
