@@ -55,6 +55,18 @@ class PRValues(C.Structure):
                 ("outDegree", C.c_void_p), ("ext", C.c_void_p)]
 
 
+class CCValues(C.Structure):
+    """DRONE/src/cuda/algorithm/cc.h:17-25 (+ ext)"""
+    _fields_ = [("sendID", C.c_void_p), ("recvID", C.c_void_p), ("sendCCValue", C.c_void_p),
+                ("recvCCValue", C.c_void_p), ("ccValue", C.c_void_p), ("ext", C.c_void_p)]
+
+
+class SSSPValues(C.Structure):
+    """DRONE/src/cuda/algorithm/sssp.h:17-25 (+ ext)"""
+    _fields_ = [("sendID", C.c_void_p), ("recvID", C.c_void_p), ("sendDis", C.c_void_p),
+                ("recvDis", C.c_void_p), ("distance", C.c_void_p), ("ext", C.c_void_p)]
+
+
 class GcnConfig(C.Structure):
     _fields_ = [("n", C.c_int), ("input_dim", C.c_int), ("hidden_dim", C.c_int), ("output_dim", C.c_int),
                 ("dropout", C.c_float), ("learning_rate", C.c_float), ("weight_decay", C.c_float),
@@ -136,12 +148,23 @@ SIGNATURES = {
     "drone_pr_worker_run_f64": (_I, [_P, _D, _I, _P]),
     "drone_pr_worker_destroy": (_I, [_P]),
     "drone_copy_to_host": (_I, [_P, _P, C.c_size_t]),
+    "drone_copy_to_device": (_I, [_P, _P, C.c_size_t]),
     "drone_timer_create": (_I, [C.POINTER(_P)]),
     "drone_timer_start": (_I, [_P, _P]),
     "drone_timer_stop": (_I, [_P, _P]),
     "drone_timer_elapsed_ms": (_I, [_P, C.POINTER(_F)]),
     "drone_timer_destroy": (_I, [_P]),
     "drone_device_synchronize": (_I, []),
+    "drone_pr_worker_attach_loopback": (_I, [_P, _P]),
+    "drone_loopback_create": (_I, [C.POINTER(_P), _I, _I]),
+    "drone_loopback_attach": (_I, [_P, _I, C.POINTER(Comm)]),
+    "drone_loopback_destroy": (_I, [_P]),
+    "CC_PEVal": (Response, [C.POINTER(Graph), C.POINTER(CCValues), _I, _I, C.POINTER(Comm)]),
+    "CC_IncEVal": (Response, [C.POINTER(Graph), C.POINTER(CCValues), _I, _I, C.POINTER(Comm)]),
+    "drone_cc_values_destroy": (None, [C.POINTER(Graph), C.POINTER(CCValues)]),
+    "SSSP_PEVal": (Response, [C.POINTER(Graph), C.POINTER(SSSPValues), _I, _I, _I, C.POINTER(Comm)]),
+    "SSSP_IncEVal": (Response, [C.POINTER(Graph), C.POINTER(SSSPValues), _I, _I, C.POINTER(Comm)]),
+    "drone_sssp_values_destroy": (None, [C.POINTER(Graph), C.POINTER(SSSPValues)]),
 }
 
 

@@ -1,0 +1,426 @@
+// Replica exchange: static send lists, pack / apply kernels, the in-process loopback transport.
+#include "exchange.h"
+
+#include <chrono>
+#include <condition_variable>
+#include <mutex>
+#include <rocprim/device/device_scan.hpp>
+
+using namespace drone;
+
+namespace {
+
+template <typename T> T *to_device_vec(const std::vector<T> &h)
+{
+    T *d = nullptr;
+    if (hipMalloc(&d, sizeof(T) * (h.empty() ? 1 : h.size())) != hipSuccess) return nullptr;
+    if (!h.empty() && hipMemcpy(d, h.data(), sizeof(T) * h.size(), hipMemcpyHostToDevice) != hipSuccess) {
+        (void)hipFree(d);
+        return nullptr;
+    }
+    return d;
+}
+
+// flag[i] = 1 iff item i of the static list sends this step; flag[items] = 0 so that the exclusive scan over
+// items + 1 elements ends with the total.
+template <typename Policy>
+__global__ void exchange_flag_kernel(int phase, int items, const int *__restrict__ item_vertex,
+                                     const int *__restrict__ active, const int *__restrict__ ubm,
+                                     int *__restrict__ flag)
+{
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i <= items; i += gridDim.x * blockDim.x) {
+        int f = 0;
+        if (i < items) {
+            const int v = item_vertex[i];
+            f = phase == kMirrorToMaster ? Policy::send_mirror(active[v]) : Policy::send_master(active[v], ubm[v]);
+        }
+        flag[i] = f;
+    }
+}
+
+// send_index[w] = pos[group_off[w]]: where worker w's segment starts in the send buffers
+__global__ void exchange_index_kernel(int workers, const int *__restrict__ group_off, const int *__restrict__ pos,
+                                      int *__restrict__ send_index)
+{
+    const int w = blockIdx.x * blockDim.x + threadIdx.x;
+    if (w <= workers) send_index[w] = pos[group_off[w]];
+}
+
+template <typename T>
+__global__ void exchange_pack_kernel(int items, const int *__restrict__ item_vertex, const int *__restrict__ flag,
+                                     const int *__restrict__ pos, const int *__restrict__ l2g,
+                                     const T *__restrict__ vals, int *__restrict__ send_id, T *__restrict__ send_val)
+{
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < items; i += gridDim.x * blockDim.x) {
+        if (!flag[i]) continue;
+        const int v = item_vertex[i], p = pos[i];
+        send_id[p] = l2g[v];
+        send_val[p] = vals[v];
+    }
+}
+
+// One received segment (all from the same worker: no vertex appears twice).  Unknown ids are counted, as the
+// reference prints them (pr.cu:183-187) and carries on.
+template <typename Policy>
+__global__ void exchange_apply_kernel(int phase, int count, const int *__restrict__ recv_id,
+                                      const typename Policy::T *__restrict__ recv_val, const int *__restrict__ g2l,
+                                      int nglobal, typename Policy::T *__restrict__ vals, int *__restrict__ ubm,
+                                      int *__restrict__ unknown)
+{
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < count; i += gridDim.x * blockDim.x) {
+        const int gid = recv_id[i];
+        const int l = gid >= 0 && gid < nglobal ? g2l[gid] : -1;
+        if (l < 0) {
+            atomicAdd(unknown, 1);
+            continue;
+        }
+        Policy::combine(phase, vals + l, recv_val[i], ubm + l);
+    }
+}
+
+int grid_for(int count) { return count > 0 ? (int)(ceil_div(count, 256) < 2048 ? ceil_div(count, 256) : 2048) : 1; }
+
+drone_transport *transport_of(Comm *comm, int workerNum, const char *who)
+{
+    if (!comm || !comm->comm) {
+        set_error(DRONE_ERR_INVALID, "%s: workerNum = %d needs a transport in Comm::comm (see drone_loopback_attach)",
+                  who, workerNum);
+        return nullptr;
+    }
+    drone_transport *t = static_cast<drone_transport *>(comm->comm);
+    if (!t->exchange || !t->allreduce_sum_f32) {
+        set_error(DRONE_ERR_INVALID, "%s: the transport in Comm::comm has null entries", who);
+        return nullptr;
+    }
+    return t;
+}
+
+}  // namespace
+
+void drone::routes_release(RouteLists *r)
+{
+    if (r->mirror_vertex) (void)hipFree(r->mirror_vertex);
+    if (r->master_vertex) (void)hipFree(r->master_vertex);
+    if (r->group_off) (void)hipFree(r->group_off);
+    if (r->flag) (void)hipFree(r->flag);
+    if (r->pos) (void)hipFree(r->pos);
+    if (r->scan_tmp) (void)hipFree(r->scan_tmp);
+    if (r->send_index_d) (void)hipFree(r->send_index_d);
+    if (r->send_index_h) (void)hipHostFree(r->send_index_h);
+    if (r->unknown) (void)hipFree(r->unknown);
+    *r = RouteLists{};
+}
+
+int drone::routes_prepare(Graph *g, int workerNum)
+{
+    GraphExt *x = static_cast<GraphExt *>(g->ext);
+    RouteLists &r = x->routes;
+    if (r.ready && r.workers == workerNum) return DRONE_OK;
+    routes_release(&r);
+    const int n = x->n;
+    DRONE_REQUIRE(workerNum >= 1, "workerNum");
+    // the tables are tiny next to the edge arrays: group them on the host
+    std::vector<int> m2w((size_t)n), mwi((size_t)n + 1), m2ws((size_t)(g->MirrorWorkerSize > 0 ? g->MirrorWorkerSize : 0));
+    if (n > 0) {
+        DRONE_HIP_TRY(hipMemcpy(m2w.data(), g->Mirror2Worker, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost));
+        DRONE_HIP_TRY(hipMemcpy(mwi.data(), g->MasterWorkerIndex, sizeof(int) * ((size_t)n + 1), hipMemcpyDeviceToHost));
+    }
+    if (!m2ws.empty())
+        DRONE_HIP_TRY(hipMemcpy(m2ws.data(), g->Master2Workers, sizeof(int) * m2ws.size(), hipMemcpyDeviceToHost));
+    DRONE_REQUIRE(n == 0 || mwi[n] == (int)m2ws.size(), "MasterWorkerIndex does not end at MirrorWorkerSize");
+
+    r.mirror_off.assign((size_t)workerNum + 1, 0);
+    r.master_off.assign((size_t)workerNum + 1, 0);
+    for (int v = 0; v < n; ++v) {
+        const int w = m2w[v];
+        if (w == -1) continue;
+        DRONE_REQUIRE(w >= 0 && w < workerNum, "Mirror2Worker names a worker outside [0, workerNum)");
+        ++r.mirror_off[(size_t)w + 1];
+    }
+    for (int w : m2ws) {
+        DRONE_REQUIRE(w >= 0 && w < workerNum, "Master2Workers names a worker outside [0, workerNum)");
+        ++r.master_off[(size_t)w + 1];
+    }
+    for (int w = 0; w < workerNum; ++w) {
+        r.mirror_off[w + 1] += r.mirror_off[w];
+        r.master_off[w + 1] += r.master_off[w];
+    }
+    r.mirror_items = r.mirror_off[workerNum];
+    r.master_items = r.master_off[workerNum];
+    std::vector<int> mirror_vertex((size_t)r.mirror_items), master_vertex((size_t)r.master_items);
+    {
+        std::vector<int> cur(r.mirror_off.begin(), r.mirror_off.end() - 1);
+        for (int v = 0; v < n; ++v)
+            if (m2w[v] != -1) mirror_vertex[(size_t)cur[m2w[v]]++] = v;
+        cur.assign(r.master_off.begin(), r.master_off.end() - 1);
+        for (int v = 0; v < n; ++v)
+            for (int k = mwi[v]; k < mwi[v + 1]; ++k) master_vertex[(size_t)cur[m2ws[k]]++] = v;
+    }
+    r.mirror_vertex = to_device_vec(mirror_vertex);
+    r.master_vertex = to_device_vec(master_vertex);
+    std::vector<int> offs(r.mirror_off);
+    offs.insert(offs.end(), r.master_off.begin(), r.master_off.end());
+    r.group_off = to_device_vec(offs);
+    DRONE_REQUIRE(r.mirror_vertex && r.master_vertex && r.group_off, "device allocation of the send lists failed");
+    r.capacity = r.mirror_items > r.master_items ? r.mirror_items : r.master_items;
+    if (r.capacity < 1) r.capacity = 1;
+    DRONE_HIP_TRY(hipMalloc(&r.flag, sizeof(int) * ((size_t)r.capacity + 1)));
+    DRONE_HIP_TRY(hipMalloc(&r.pos, sizeof(int) * ((size_t)r.capacity + 1)));
+    DRONE_HIP_TRY(rocprim::exclusive_scan(nullptr, r.scan_tmp_bytes, r.flag, r.pos, 0, (size_t)r.capacity + 1,
+                                          rocprim::plus<int>(), nullptr));
+    DRONE_HIP_TRY(hipMalloc(&r.scan_tmp, r.scan_tmp_bytes ? r.scan_tmp_bytes : 1));
+    DRONE_HIP_TRY(hipMalloc(&r.send_index_d, sizeof(int) * ((size_t)workerNum + 1)));
+    DRONE_HIP_TRY(hipHostMalloc(&r.send_index_h, sizeof(int) * ((size_t)workerNum + 1)));
+    DRONE_HIP_TRY(hipMalloc(&r.unknown, sizeof(int)));
+    r.workers = workerNum;
+    r.ready = true;
+    return DRONE_OK;
+}
+
+int drone::exchange_buffers_create(Graph *g, int workerNum, int **send_id, int **recv_id, void **send_val,
+                                   void **recv_val)
+{
+    const int rc = routes_prepare(g, workerNum);
+    if (rc != DRONE_OK) return rc;
+    const size_t cap = (size_t) static_cast<GraphExt *>(g->ext)->routes.capacity;
+    DRONE_HIP_TRY(hipMalloc(send_id, sizeof(int) * cap));
+    DRONE_HIP_TRY(hipMalloc(recv_id, sizeof(int) * cap));
+    DRONE_HIP_TRY(hipMalloc(send_val, 4 * cap));
+    DRONE_HIP_TRY(hipMalloc(recv_val, 4 * cap));
+    return DRONE_OK;
+}
+
+template <typename Policy>
+int drone::exchange_phase(Graph *g, int phase, typename Policy::T *vals, int *send_id, int *recv_id,
+                          typename Policy::T *send_val, typename Policy::T *recv_val, int workerId, int workerNum,
+                          Comm *comm, int *sent, int *received)
+{
+    using T = typename Policy::T;
+    static_assert(sizeof(T) == 4, "exchange values are 4 bytes");
+    drone_transport *tr = transport_of(comm, workerNum, "exchange");
+    if (!tr) return DRONE_ERR_INVALID;
+    DRONE_REQUIRE(workerId >= 0 && workerId < workerNum, "workerId");
+    int rc = routes_prepare(g, workerNum);
+    if (rc != DRONE_OK) return rc;
+    GraphExt *x = static_cast<GraphExt *>(g->ext);
+    RouteLists &r = x->routes;
+    hipStream_t s = static_cast<hipStream_t>(comm->s);
+    const bool up = phase == kMirrorToMaster;
+    const int items = up ? r.mirror_items : r.master_items;
+    const int *item_vertex = up ? r.mirror_vertex : r.master_vertex;
+    const int *group_off = r.group_off + (up ? 0 : workerNum + 1);
+
+    exchange_flag_kernel<Policy><<<grid_for(items + 1), 256, 0, s>>>(phase, items, item_vertex, g->active,
+                                                                     g->updateByMessage, r.flag);
+    size_t tmp = r.scan_tmp_bytes;
+    DRONE_HIP_TRY(rocprim::exclusive_scan(r.scan_tmp, tmp, r.flag, r.pos, 0, (size_t)items + 1, rocprim::plus<int>(), s));
+    exchange_index_kernel<<<(int)ceil_div(workerNum + 1, 64), 64, 0, s>>>(workerNum, group_off, r.pos, r.send_index_d);
+    exchange_pack_kernel<T><<<grid_for(items), 256, 0, s>>>(items, item_vertex, r.flag, r.pos, g->Local2Global, vals,
+                                                            send_id, send_val);
+    DRONE_HIP_TRY(hipGetLastError());
+    DRONE_HIP_TRY(hipMemcpyAsync(r.send_index_h, r.send_index_d, sizeof(int) * ((size_t)workerNum + 1),
+                                 hipMemcpyDeviceToHost, s));
+    DRONE_HIP_TRY(hipStreamSynchronize(s));
+
+    std::vector<int> send_len((size_t)workerNum), recv_len((size_t)workerNum, 0);
+    for (int w = 0; w < workerNum; ++w) send_len[w] = r.send_index_h[w + 1] - r.send_index_h[w];
+    DRONE_REQUIRE(send_len[workerId] == 0, "the routing tables name this worker as its own peer");
+    rc = tr->exchange(tr->ctx, workerId, workerNum, send_len.data(), r.send_index_h, send_id, send_val,
+                      recv_len.data(), recv_id, recv_val, r.capacity, comm->s);
+    if (rc != DRONE_OK) return rc;
+
+    int *unknown = r.unknown;
+    DRONE_HIP_TRY(hipMemsetAsync(unknown, 0, sizeof(int), s));
+    int total = 0;
+    for (int w = 0; w < workerNum; ++w) {
+        const int len = recv_len[w];
+        if (len <= 0) continue;
+        exchange_apply_kernel<Policy><<<grid_for(len), 256, 0, s>>>(phase, len, recv_id + total, recv_val + total,
+                                                                    g->Global2Local, *g->globalVertexSize, vals,
+                                                                    g->updateByMessage, unknown);
+        total += len;
+    }
+    DRONE_HIP_TRY(hipGetLastError());
+    int bad = 0;
+    DRONE_HIP_TRY(hipMemcpyAsync(&bad, unknown, sizeof(int), hipMemcpyDeviceToHost, s));
+    DRONE_HIP_TRY(hipStreamSynchronize(s));
+    if (bad > 0) printf("error global id: %d received ids are not on worker %d\n", bad, workerId);
+    *sent = r.send_index_h[workerNum];
+    *received = total;
+    return DRONE_OK;
+}
+
+template int drone::exchange_phase<PrExchange>(Graph *, int, float *, int *, int *, float *, float *, int, int,
+                                               Comm *, int *, int *);
+template int drone::exchange_phase<CcExchange>(Graph *, int, int *, int *, int *, int *, int *, int, int, Comm *,
+                                               int *, int *);
+template int drone::exchange_phase<SsspExchange>(Graph *, int, float *, int *, int *, float *, float *, int, int,
+                                                 Comm *, int *, int *);
+
+int drone::exchange_allreduce_f32(float *device_scalar, int workerId, int workerNum, Comm *comm)
+{
+    drone_transport *tr = transport_of(comm, workerNum, "allreduce");
+    if (!tr) return DRONE_ERR_INVALID;
+    return tr->allreduce_sum_f32(tr->ctx, workerId, workerNum, device_scalar, comm->s);
+}
+
+// ---- loopback transport -------------------------------------------------------------------------------------
+struct drone_loopback {
+    int workers = 0;
+    int timeout_ms = 0;
+    std::mutex mu;
+    std::condition_variable cv;
+    int waiting = 0;
+    uint64_t generation = 0;
+    bool broken = false;
+    struct Slot {
+        const int *send_len = nullptr, *send_index = nullptr, *send_id = nullptr;
+        const void *send_val = nullptr;
+        float *scalar = nullptr;
+    };
+    std::vector<Slot> slot;
+    struct Endpoint {
+        drone_transport table;
+        drone_loopback *group;
+    };
+    std::vector<Endpoint> endpoint;
+
+    // Returns false when a peer did not arrive in time (the group is then unusable).
+    bool barrier()
+    {
+        std::unique_lock<std::mutex> lk(mu);
+        if (broken) return false;
+        const uint64_t gen = generation;
+        if (++waiting == workers) {
+            waiting = 0;
+            ++generation;
+            cv.notify_all();
+            return true;
+        }
+        auto arrived = [&] { return generation != gen || broken; };
+        if (timeout_ms > 0) {
+            if (!cv.wait_for(lk, std::chrono::milliseconds(timeout_ms), arrived)) {
+                broken = true;
+                cv.notify_all();
+                return false;
+            }
+        } else {
+            cv.wait(lk, arrived);
+        }
+        return !broken;
+    }
+};
+
+namespace {
+
+int loopback_fail(const char *what)
+{
+    set_error(DRONE_ERR_INVALID, "loopback transport: %s: a peer did not arrive (timeout) or the group is broken", what);
+    return DRONE_ERR_INVALID;
+}
+
+int loopback_exchange(void *ctx, int workerId, int workerNum, const int *send_len, const int *send_index,
+                      const int *send_id, const void *send_val, int *recv_len, int *recv_id, void *recv_val,
+                      int recv_capacity, drone_stream_t stream)
+{
+    drone_loopback *grp = static_cast<drone_loopback::Endpoint *>(ctx)->group;
+    DRONE_REQUIRE(workerNum == grp->workers && workerId >= 0 && workerId < workerNum, "worker id / count");
+    hipStream_t s = as_stream(stream);
+    grp->slot[workerId].send_len = send_len;
+    grp->slot[workerId].send_index = send_index;
+    grp->slot[workerId].send_id = send_id;
+    grp->slot[workerId].send_val = send_val;
+    if (!grp->barrier()) return loopback_fail("exchange");
+    int total = 0, rc = DRONE_OK;
+    for (int w = 0; w < workerNum && rc == DRONE_OK; ++w) {
+        recv_len[w] = 0;
+        if (w == workerId) continue;
+        const drone_loopback::Slot &src = grp->slot[w];
+        const int len = src.send_len[workerId];
+        if (len <= 0) continue;
+        if (total + len > recv_capacity) {
+            set_error(DRONE_ERR_INVALID, "loopback transport: worker %d receives more than its %d staging elements",
+                      workerId, recv_capacity);
+            rc = DRONE_ERR_INVALID;
+            break;
+        }
+        const size_t off = (size_t)src.send_index[workerId];
+        if (hipMemcpyAsync(recv_id + total, src.send_id + off, sizeof(int) * (size_t)len, hipMemcpyDeviceToDevice, s) != hipSuccess ||
+            hipMemcpyAsync(static_cast<char *>(recv_val) + 4 * (size_t)total, static_cast<const char *>(src.send_val) + 4 * off,
+                           4 * (size_t)len, hipMemcpyDeviceToDevice, s) != hipSuccess) {
+            set_error(DRONE_ERR_HIP, "loopback transport: device copy failed");
+            rc = DRONE_ERR_HIP;
+            break;
+        }
+        recv_len[w] = len;
+        total += len;
+    }
+    if (hipStreamSynchronize(s) != hipSuccess && rc == DRONE_OK) {
+        set_error(DRONE_ERR_HIP, "loopback transport: stream synchronise failed");
+        rc = DRONE_ERR_HIP;
+    }
+    if (!grp->barrier()) return loopback_fail("exchange");  // the senders' buffers are free again
+    return rc;
+}
+
+int loopback_allreduce(void *ctx, int workerId, int workerNum, float *device_scalar, drone_stream_t stream)
+{
+    drone_loopback *grp = static_cast<drone_loopback::Endpoint *>(ctx)->group;
+    DRONE_REQUIRE(workerNum == grp->workers && workerId >= 0 && workerId < workerNum, "worker id / count");
+    hipStream_t s = as_stream(stream);
+    DRONE_HIP_TRY(hipStreamSynchronize(s));  // the scalar is final before the peers read it
+    grp->slot[workerId].scalar = device_scalar;
+    if (!grp->barrier()) return loopback_fail("allreduce");
+    float sum = 0.0f;
+    int rc = DRONE_OK;
+    for (int w = 0; w < workerNum; ++w) {
+        float v = 0.0f;
+        if (hipMemcpy(&v, grp->slot[w].scalar, sizeof(float), hipMemcpyDeviceToHost) != hipSuccess) {
+            set_error(DRONE_ERR_HIP, "loopback transport: reading a peer's scalar failed");
+            rc = DRONE_ERR_HIP;
+        }
+        sum += v;
+    }
+    if (!grp->barrier()) return loopback_fail("allreduce");  // everyone has read before anyone writes
+    if (rc != DRONE_OK) return rc;
+    DRONE_HIP_TRY(hipMemcpy(device_scalar, &sum, sizeof(float), hipMemcpyHostToDevice));
+    return DRONE_OK;
+}
+
+}  // namespace
+
+extern "C" int drone_loopback_create(drone_loopback **group, int workerNum, int timeout_ms)
+{
+    clear_error();
+    DRONE_REQUIRE(group != nullptr, "group");
+    DRONE_REQUIRE(workerNum >= 1 && workerNum <= 4096, "workerNum");
+    DRONE_REQUIRE(timeout_ms >= 0, "timeout_ms");
+    drone_loopback *g = new drone_loopback();
+    g->workers = workerNum;
+    g->timeout_ms = timeout_ms;
+    g->slot.resize((size_t)workerNum);
+    g->endpoint.resize((size_t)workerNum);
+    for (int w = 0; w < workerNum; ++w) {
+        g->endpoint[w].group = g;
+        g->endpoint[w].table.ctx = &g->endpoint[w];
+        g->endpoint[w].table.exchange = loopback_exchange;
+        g->endpoint[w].table.allreduce_sum_f32 = loopback_allreduce;
+    }
+    *group = g;
+    return DRONE_OK;
+}
+
+extern "C" int drone_loopback_attach(drone_loopback *group, int workerId, Comm *comm)
+{
+    clear_error();
+    DRONE_REQUIRE(group != nullptr && comm != nullptr, "group / comm");
+    DRONE_REQUIRE(workerId >= 0 && workerId < group->workers, "workerId");
+    comm->comm = &group->endpoint[workerId].table;
+    return DRONE_OK;
+}
+
+extern "C" int drone_loopback_destroy(drone_loopback *group)
+{
+    delete group;
+    return DRONE_OK;
+}

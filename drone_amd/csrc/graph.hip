@@ -45,10 +45,9 @@ extern "C" Graph *build_graph(int globalVertexSize, int edgeSize, int *u, int *v
                               int workerNum, Comm *comm)
 {
     clear_error();
-    if (workerNum != 1 || workerId != 0) {
-        set_error(DRONE_ERR_UNSUPPORTED, "build_graph: this build holds one subgraph on one GPU (workerNum=%d)",
-                  workerNum);
-        printf("Failed: build_graph supports workerNum == 1 only (got worker %d of %d)\n", workerId, workerNum);
+    if (workerNum < 1 || workerId < 0 || workerId >= workerNum) {
+        set_error(DRONE_ERR_INVALID, "build_graph: worker %d of %d", workerId, workerNum);
+        printf("Failed: build_graph: worker %d of %d\n", workerId, workerNum);
         exit(EXIT_FAILURE);
     }
     if (globalVertexSize < 0 || edgeSize < 0 || (edgeSize > 0 && (!u || !v))) {
@@ -57,7 +56,7 @@ extern "C" Graph *build_graph(int globalVertexSize, int edgeSize, int *u, int *v
         exit(EXIT_FAILURE);
     }
     Graph *g = (Graph *)calloc(1, sizeof(Graph));
-    g->GID = 0;  // the reference picks workerId % 4 (graph.cu:39); one worker -> device 0
+    g->GID = 0;  // the reference picks workerId % 4 (graph.cu:39); here every subgraph of the process shares device 0
     DRONE_HIP_OR_DIE(hipSetDevice(g->GID));
 
     // graph.cu:52-60: local ids in first-seen order, scanning u[i] then v[i]
@@ -117,7 +116,9 @@ extern "C" Graph *build_graph(int globalVertexSize, int edgeSize, int *u, int *v
     g->ext = x;
 
     if (comm) {
-        comm->comm = nullptr;  // one worker: no communicator (the reference creates an NCCL one, graph.cu:128)
+        // The reference creates an NCCL communicator here (graph.cu:128).  The transport is attached by the caller
+        // (drone_loopback_attach, or a drone_transport of its own); one worker needs none.
+        comm->comm = nullptr;
         hipStream_t s;
         DRONE_HIP_OR_DIE(hipStreamCreate(&s));
         comm->s = s;
@@ -139,6 +140,7 @@ extern "C" void addMasterRoute(Graph *g, int *masterVertex, int *mirrorNumber, i
     const int n = getLocalVertexSize(g);
     g->MasterSize = masterSize;
     g->MirrorWorkerSize = mirrorWorkerSize;
+    static_cast<GraphExt *>(g->ext)->routes.ready = false;  // the exchange's send lists are rebuilt on next use
     std::vector<int> g2l((size_t)*g->globalVertexSize);
     if (!g2l.empty())
         DRONE_HIP_OR_DIE(hipMemcpy(g2l.data(), g->Global2Local, sizeof(int) * g2l.size(), hipMemcpyDeviceToHost));
@@ -163,6 +165,7 @@ extern "C" void addMirrorRoute(Graph *g, int *mirrorVertex, int *masterWorker, i
     clear_error();
     DRONE_HIP_OR_DIE(hipSetDevice(g->GID));
     g->MirrorSize = mirrorSize;
+    static_cast<GraphExt *>(g->ext)->routes.ready = false;
     const int n = getLocalVertexSize(g);
     fill_i32_kernel<<<256, 256>>>(g->Mirror2Worker, -1, n);
     if (mirrorSize > 0) {

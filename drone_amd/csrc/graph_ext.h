@@ -1,10 +1,32 @@
 // Library-private state hung off Graph::ext and PRValues::ext.
 #pragma once
+#include <vector>
+
 #include "spmv_merge.h"
 
 struct drone_pr_plan;
 
 namespace drone {
+
+// Static send lists of the replica exchange and the scratch of one pack step.
+struct RouteLists {
+    bool ready = false;
+    int workers = 0;
+    int mirror_items = 0;          // = MirrorSize
+    int master_items = 0;          // = MirrorWorkerSize: one item per (master, worker holding a mirror of it)
+    int *mirror_vertex = nullptr;  // device [mirror_items]: local ids grouped by master worker, ascending inside a group
+    int *master_vertex = nullptr;  // device [master_items]: local ids grouped by mirror worker, ascending inside a group
+    std::vector<int> mirror_off, master_off;  // host [workers + 1]: group boundaries in the two lists
+    int *group_off = nullptr;      // device [2][workers + 1]: the same boundaries
+    int capacity = 0;              // max(mirror_items, master_items), at least 1
+    int *flag = nullptr;           // device [capacity + 1]
+    int *pos = nullptr;            // device [capacity + 1]
+    void *scan_tmp = nullptr;
+    size_t scan_tmp_bytes = 0;
+    int *send_index_d = nullptr;   // device [workers + 1]
+    int *send_index_h = nullptr;   // pinned [workers + 1]
+    int *unknown = nullptr;        // device scalar: received ids that are not on this worker
+};
 
 struct GraphExt {
     int n = 0;
@@ -20,9 +42,17 @@ struct GraphExt {
     int64_t *row_ptr64 = nullptr;
     double *inv64 = nullptr;
     double *rank64 = nullptr;
+    RouteLists routes;
+    // SSSP: edge lengths in in-edge order
+    int *in_eid = nullptr;    // device [edges]: position in the out-edge CSR (g->dst / g->edgeLen) of each in-edge
+    float *in_len = nullptr;  // device [edges]: g->edgeLen gathered through in_eid at every SSSP_PEVal
 };
 
 void graph_ext_release(GraphExt *x);  // frees everything but the struct itself
+
+// Merge-path tiling and scratch over the in-edge CSR (x->mt, x->ms), shared by the float PageRank, CC and SSSP
+// aggregations (their value types are at most 8 bytes).  Built on first use; exits on failure.
+void ensure_aggregation_ready(Graph *g);
 
 struct PRExt {
     float *push = nullptr;        // device [n]: value each vertex pushes along its out-edges this step

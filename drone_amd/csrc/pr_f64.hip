@@ -23,7 +23,7 @@ struct PrF64Epi {
     const double *__restrict__ dang;   // device scalar: dangling mass of the previous ranks
     double alpha, inv_n;
 
-    __device__ __forceinline__ double load(int c) const { return c_in[c]; }
+    __device__ __forceinline__ double load(int c, int64_t = 0) const { return c_in[c]; }
     __device__ __forceinline__ void row(int r, double s, double &stat) const
     {
         const double base = (1.0 - alpha) * inv_n + alpha * dang[0] * inv_n;

@@ -5,7 +5,7 @@
 // in-edges of v together with the number of non-zero pushes, which gives g->active and VisitedSize.
 #include <chrono>
 
-#include "graph_ext.h"
+#include "exchange.h"
 
 using namespace drone;
 
@@ -20,7 +20,7 @@ struct PushEpi {
     float *__restrict__ diff;
     int *__restrict__ active;
 
-    __device__ __forceinline__ PushF2 load(int c) const
+    __device__ __forceinline__ PushF2 load(int c, int64_t) const
     {
         const float v = push[c];
         return PushF2{v, v != 0.0f ? 1.0f : 0.0f};
@@ -133,7 +133,9 @@ double seconds_since(std::chrono::steady_clock::time_point t0)
     return std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
 }
 
-void ensure_push_ready(Graph *g)
+}  // namespace
+
+void drone::ensure_aggregation_ready(Graph *g)
 {
     GraphExt *x = static_cast<GraphExt *>(g->ext);
     if (x->push_ready) return;
@@ -143,6 +145,32 @@ void ensure_push_ready(Graph *g)
         exit(EXIT_FAILURE);
     }
     x->push_ready = true;
+}
+
+namespace {
+
+// pr.cu:415-421 / :478-483: the two exchange phases and the sum of the dangling mass over the workers.
+void exchange_push(Graph *g, PRValues *values, int workerId, int workerNum, Comm *comm, Response *res)
+{
+    if (workerNum <= 1) return;  // one subgraph: the reference moves zero elements
+    int rc = DRONE_OK;
+    if (!values->sendID)
+        rc = exchange_buffers_create(g, workerNum, &values->sendID, &values->recvID,
+                                     reinterpret_cast<void **>(&values->sendDiff),
+                                     reinterpret_cast<void **>(&values->recvDiff));
+    if (rc == DRONE_OK)
+        rc = exchange_phase<PrExchange>(g, kMirrorToMaster, values->diffValue, values->sendID, values->recvID,
+                                        values->sendDiff, values->recvDiff, workerId, workerNum, comm,
+                                        &res->Mirror2MasterSendSize, &res->Mirror2MasterRecvSize);
+    if (rc == DRONE_OK)
+        rc = exchange_phase<PrExchange>(g, kMasterToMirror, values->diffValue, values->sendID, values->recvID,
+                                        values->sendDiff, values->recvDiff, workerId, workerNum, comm,
+                                        &res->Master2MirrorSendSize, &res->Master2MirrorRecvSize);
+    if (rc == DRONE_OK) rc = exchange_allreduce_f32(values->globalDiff, workerId, workerNum, comm);
+    if (rc != DRONE_OK) {
+        printf("Failed: exchange on worker %d: %s\n", workerId, drone_last_error_string());
+        exit(EXIT_FAILURE);
+    }
 }
 
 int aggregate_push(Graph *g, PRValues *values, hipStream_t s)
@@ -170,6 +198,9 @@ void drone::graph_ext_release(GraphExt *x)
     if (x->row_ptr64) (void)hipFree(x->row_ptr64);
     if (x->inv64) (void)hipFree(x->inv64);
     if (x->rank64) (void)hipFree(x->rank64);
+    routes_release(&x->routes);
+    if (x->in_eid) (void)hipFree(x->in_eid);
+    if (x->in_len) (void)hipFree(x->in_len);
     *x = GraphExt{};
 }
 
@@ -189,7 +220,6 @@ extern "C" void loadOutDegree(Graph *g, PRValues *values, int *globalOutDegree)
 
 extern "C" Response PR_PEVal(Graph *g, PRValues *values, int workerId, int workerNum, Comm *comm)
 {
-    (void)workerId; (void)workerNum;
     clear_error();
     const auto t0 = std::chrono::steady_clock::now();
     DRONE_HIP_OR_DIE(hipSetDevice(g->GID));
@@ -202,7 +232,7 @@ extern "C" Response PR_PEVal(Graph *g, PRValues *values, int workerId, int worke
         printf("Failed: PR_PEVal before loadOutDegree\n");
         exit(EXIT_FAILURE);
     }
-    ensure_push_ready(g);
+    ensure_aggregation_ready(g);
     // pr.cu:383-389: the state vectors are allocated by this call
     if (!g->active) DRONE_HIP_OR_DIE(hipMalloc(&g->active, sizeof(int) * cnt));
     if (!g->updateByMessage) DRONE_HIP_OR_DIE(hipMalloc(&g->updateByMessage, sizeof(int) * cnt));
@@ -219,7 +249,7 @@ extern "C" Response PR_PEVal(Graph *g, PRValues *values, int workerId, int worke
         if (px->vertex_blocks > 4096) px->vertex_blocks = 4096;
         DRONE_HIP_OR_DIE(hipMalloc(&px->block_part, sizeof(double) * (size_t)px->vertex_blocks));
         values->ext = px;
-        // exchange staging (pr.cu:402-405) has no use with one subgraph: left null
+        // exchange staging (pr.cu:402-405) is allocated by the first exchange; with one subgraph it stays null
     }
     PRExt *px = static_cast<PRExt *>(values->ext);
     DRONE_HIP_OR_DIE(hipMemsetAsync(values->globalDiff, 0, sizeof(float), s));
@@ -228,16 +258,17 @@ extern "C" Response PR_PEVal(Graph *g, PRValues *values, int workerId, int worke
                                                                   values->prValue, values->accValue, px->push,
                                                                   g->updateByMessage, px->block_part);
     pr_add_global_diff_kernel<<<1, kSpmvBlock, 0, s>>>(px->block_part, px->vertex_blocks, values->globalDiff);
-    res.VisitedSize = aggregate_push(g, values, s);
+    res.VisitedSize = aggregate_push(g, values, s);  // countActive reads g->active, which the exchange leaves alone
     res.LocalVertexSize = n;
     res.CalTime = (float)seconds_since(t0);
-    res.SendTime = 0.0f;  // one subgraph: nothing to exchange (pr.cu:415-421 moves zero elements)
+    const auto t1 = std::chrono::steady_clock::now();
+    exchange_push(g, values, workerId, workerNum, comm, &res);
+    res.SendTime = (float)seconds_since(t1);
     return res;
 }
 
 extern "C" Response PR_IncEVal(Graph *g, PRValues *values, int workerId, int workerNum, Comm *comm)
 {
-    (void)workerId; (void)workerNum;
     clear_error();
     const auto t0 = std::chrono::steady_clock::now();
     DRONE_HIP_OR_DIE(hipSetDevice(g->GID));
@@ -258,7 +289,9 @@ extern "C" Response PR_IncEVal(Graph *g, PRValues *values, int workerId, int wor
     res.VisitedSize = aggregate_push(g, values, s);
     res.LocalVertexSize = n;
     res.CalTime = (float)seconds_since(t0);
-    res.SendTime = 0.0f;
+    const auto t1 = std::chrono::steady_clock::now();
+    exchange_push(g, values, workerId, workerNum, comm, &res);
+    res.SendTime = (float)seconds_since(t1);
     return res;
 }
 
@@ -279,6 +312,10 @@ extern "C" void drone_pr_values_destroy(Graph *g, PRValues *values)
     if (values->globalAcc) (void)hipFree(values->globalAcc);
     if (values->globalDiff) (void)hipFree(values->globalDiff);
     if (values->outDegree) (void)hipFree(values->outDegree);
+    if (values->sendID) (void)hipFree(values->sendID);
+    if (values->recvID) (void)hipFree(values->recvID);
+    if (values->sendDiff) (void)hipFree(values->sendDiff);
+    if (values->recvDiff) (void)hipFree(values->recvDiff);
     *values = PRValues{};
 }
 
@@ -308,6 +345,8 @@ extern "C" int drone_pr_run_graph_f64(Graph *g, PRValues *values, double alpha, 
     DRONE_HIP_TRY(hipSetDevice(g->GID));
     GraphExt *x = static_cast<GraphExt *>(g->ext);
     DRONE_REQUIRE(x->n > 0, "empty graph");
+    DRONE_REQUIRE(g->MirrorSize == 0 && g->MirrorWorkerSize == 0,
+                  "the fp64 pull run covers one whole subgraph: this graph has replicated vertices");
     if (!x->plan64) {
         DRONE_HIP_TRY(hipMalloc(&x->row_ptr64, sizeof(int64_t) * ((size_t)x->n + 1)));
         DRONE_HIP_TRY(hipMalloc(&x->inv64, sizeof(double) * (size_t)x->n));

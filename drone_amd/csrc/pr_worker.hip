@@ -243,7 +243,7 @@ extern "C" int drone_pr_worker_create(drone_pr_worker **out, const char *data_pa
 {
     clear_error();
     DRONE_REQUIRE(out && data_path, "null argument");
-    DRONE_REQUIRE(self_id >= 1 && worker_num == 1 && self_id <= worker_num, "this build runs one worker (self_id 1 of 1)");
+    DRONE_REQUIRE(worker_num >= 1 && self_id >= 1 && self_id <= worker_num, "self_id must be in [1, worker_num]");
     DRONE_REQUIRE(global_vertex_size > 0, "global vertex count");
     std::string dir(data_path);
     if (!dir.empty() && dir.back() != '/') dir += '/';  // tools.SetDataPath (Settings.go:21-27)
@@ -267,11 +267,11 @@ extern "C" int drone_pr_worker_create(drone_pr_worker **out, const char *data_pa
             set_error(DRONE_ERR_INVALID, "G.%s: edge %d has an id outside [0, %d)", id.c_str(), i, global_vertex_size);
             return DRONE_ERR_INVALID;
         }
-    if (masters > 0 || mirrors > 0) {
+    if (worker_num == 1 && (masters > 0 || mirrors > 0)) {
         cleanup();
-        set_error(DRONE_ERR_UNSUPPORTED, "partition files list %d masters / %d mirrors: replicated vertices need the "
-                  "exchange step, which this one-subgraph build does not have", masters, mirrors);
-        return DRONE_ERR_UNSUPPORTED;
+        set_error(DRONE_ERR_INVALID, "partition files list %d masters / %d mirrors but worker_num is 1: replicated "
+                  "vertices need the other workers of the partition", masters, mirrors);
+        return DRONE_ERR_INVALID;
     }
     drone_pr_worker *w = new drone_pr_worker();
     w->self_id = self_id;
@@ -283,6 +283,13 @@ extern "C" int drone_pr_worker_create(drone_pr_worker **out, const char *data_pa
     cleanup();
     *out = w;
     return DRONE_OK;
+}
+
+extern "C" int drone_pr_worker_attach_loopback(drone_pr_worker *w, drone_loopback *group)
+{
+    clear_error();
+    DRONE_REQUIRE(w && group, "null argument");
+    return drone_loopback_attach(group, w->self_id - 1, &w->comm);
 }
 
 // PRWorkerCUDA.go:52-65

@@ -22,8 +22,10 @@
 // affine in the row sum: Epi::row(r, s) is applied to the partial sum and Epi::fix(r, c) adds the
 // effect of the carry c.  Everything is order-deterministic: no floating-point atomics.
 //
-// The value type V is double for the fp64 PageRank and PushF2 (sum, non-zero count) for the float
-// delta-push state; it needs operator+ and the shuffle helpers below.
+// The value type V is double for the fp64 PageRank, PushF2 (sum, non-zero count) for the float delta-push
+// state, and MinI32 / MinF32 (operator+ is min) for label propagation and relaxation; it needs an associative
+// operator+, its identity vzero<V>() and the shuffle helpers below.  Epi::load(column, entry index) supplies the
+// value of one entry.
 #pragma once
 #include <climits>
 
@@ -49,7 +51,14 @@ struct PushF2 {
 };
 __device__ __forceinline__ PushF2 operator+(PushF2 a, PushF2 b) { return PushF2{a.s + b.s, a.c + b.c}; }
 
+struct MinI32 { int v; };
+struct MinF32 { float v; };
+__device__ __forceinline__ MinI32 operator+(MinI32 a, MinI32 b) { return MinI32{a.v < b.v ? a.v : b.v}; }
+__device__ __forceinline__ MinF32 operator+(MinF32 a, MinF32 b) { return MinF32{a.v < b.v ? a.v : b.v}; }
+
 template <typename V> __device__ __forceinline__ V vzero();
+template <> __device__ __forceinline__ MinI32 vzero<MinI32>() { return MinI32{INT_MAX}; }
+template <> __device__ __forceinline__ MinF32 vzero<MinF32>() { return MinF32{__builtin_huge_valf()}; }
 template <> __device__ __forceinline__ double vzero<double>() { return 0.0; }
 template <> __device__ __forceinline__ float vzero<float>() { return 0.0f; }
 template <> __device__ __forceinline__ PushF2 vzero<PushF2>() { return PushF2{0.0f, 0.0f}; }
@@ -60,6 +69,10 @@ __device__ __forceinline__ PushF2 shfl_up_v(PushF2 v, int d)
 {
     return PushF2{__shfl_up(v.s, d, kWave), __shfl_up(v.c, d, kWave)};
 }
+__device__ __forceinline__ MinI32 shfl_up_v(MinI32 v, int d) { return MinI32{__shfl_up(v.v, d, kWave)}; }
+__device__ __forceinline__ MinF32 shfl_up_v(MinF32 v, int d) { return MinF32{__shfl_up(v.v, d, kWave)}; }
+__device__ __forceinline__ MinI32 shfl_xor_v(MinI32 v, int m) { return MinI32{__shfl_xor(v.v, m, kWave)}; }
+__device__ __forceinline__ MinF32 shfl_xor_v(MinF32 v, int m) { return MinF32{__shfl_xor(v.v, m, kWave)}; }
 __device__ __forceinline__ double shfl_xor_v(double v, int m) { return __shfl_xor(v, m, kWave); }
 __device__ __forceinline__ float shfl_xor_v(float v, int m) { return __shfl_xor(v, m, kWave); }
 __device__ __forceinline__ PushF2 shfl_xor_v(PushF2 v, int m)
@@ -154,7 +167,7 @@ __global__ __launch_bounds__(kSpmvBlock) void spmv_merge_kernel(
         }
         V x[IPT];
 #pragma unroll
-        for (int k = 0; k < IPT; ++k) x[k] = c[k] >= 0 ? epi.load(c[k]) : vzero<V>();
+        for (int k = 0; k < IPT; ++k) x[k] = c[k] >= 0 ? epi.load(c[k], e0 + tid + k * kSpmvBlock) : vzero<V>();
 #pragma unroll
         for (int k = 0; k < IPT; ++k) {
             const int i = tid + k * kSpmvBlock;

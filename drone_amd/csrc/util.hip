@@ -136,6 +136,14 @@ extern "C" int drone_copy_to_host(void *dst_host, const void *src_device, size_t
     return DRONE_OK;
 }
 
+extern "C" int drone_copy_to_device(void *dst_device, const void *src_host, size_t bytes)
+{
+    clear_error();
+    DRONE_REQUIRE(bytes == 0 || (dst_device && src_host), "null operand");
+    if (bytes) DRONE_HIP_TRY(hipMemcpy(dst_device, src_host, bytes, hipMemcpyHostToDevice));
+    return DRONE_OK;
+}
+
 struct drone_timer {
     hipEvent_t a, b;
 };

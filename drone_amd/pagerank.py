@@ -26,6 +26,66 @@ def CUDA_build_graph(globalVertexSize, edgeSize, u, v, workerId, workerNum, comm
                              C.byref(comm))
 
 
+def CUDA_AddMasterRoute(g, masterVertex, mirrorNumber, mirrorWorkers):
+    """cuda_convert.go:35-38 (Go passes &slice[0]; empty tables are passed as one unused element here)"""
+    mv, pmv = _i32(masterVertex if len(masterVertex) else [0])
+    mn, pmn = _i32(mirrorNumber if len(mirrorNumber) else [0])
+    mw, pmw = _i32(mirrorWorkers if len(mirrorWorkers) else [0])
+    if int(np.sum(mirrorNumber)) != len(mirrorWorkers):
+        raise ValueError("mirrorNumber does not add up to len(mirrorWorkers)")
+    lib().addMasterRoute(g, pmv, pmn, pmw, len(masterVertex), len(mirrorWorkers))
+
+
+def CUDA_AddMirrorRoute(g, mirrorVertex, masterWorker):
+    """cuda_convert.go:40-42"""
+    if len(mirrorVertex) != len(masterWorker):
+        raise ValueError("mirrorVertex and masterWorker differ in length")
+    mv, pmv = _i32(mirrorVertex if len(mirrorVertex) else [0])
+    mw, pmw = _i32(masterWorker if len(masterWorker) else [0])
+    lib().addMirrorRoute(g, pmv, pmw, len(mirrorVertex))
+
+
+class Loopback:
+    """In-process transport for several subgraphs on one GPU (drone_loopback_*).  Every worker must be driven by
+    its own host thread: run_workers() does that."""
+
+    def __init__(self, workerNum, timeout_ms=120000):
+        self.h = C.c_void_p()
+        self.workerNum = workerNum
+        check(lib().drone_loopback_create(C.byref(self.h), int(workerNum), int(timeout_ms)))
+
+    def attach(self, workerId, comm):
+        check(lib().drone_loopback_attach(self.h, int(workerId), C.byref(comm)))
+
+    def close(self):
+        if self.h:
+            lib().drone_loopback_destroy(self.h)
+            self.h = None
+
+
+def run_workers(calls):
+    """Runs one callable per worker, each on its own thread (the foreign calls release the GIL), and returns their
+    results in order.  The first exception is re-raised."""
+    import threading
+    out, err = [None] * len(calls), [None] * len(calls)
+
+    def body(i):
+        try:
+            out[i] = calls[i]()
+        except BaseException as e:  # noqa: BLE001
+            err[i] = e
+
+    ts = [threading.Thread(target=body, args=(i,)) for i in range(len(calls))]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join()
+    for e in err:
+        if e is not None:
+            raise e
+    return out
+
+
 def CUDA_LoadOutDegree(g, values, globalOutDegree):
     """cuda_convert.go:85-87"""
     d, pd = _i32(globalOutDegree)
@@ -55,11 +115,19 @@ class PRWorkerCUDA:
     """Compute side of DRONE/src/worker/PRWorkerCUDA.go for one worker: newPRWorkerCUDA (:115-175) builds
     the graph and loads the out-degrees, peval (:52-65) / incEval (:76-88) make one call each."""
 
-    def __init__(self, globalVertexSize, u, v, globalOutDegree=None, workerId=0, workerNum=1):
+    def __init__(self, globalVertexSize, u, v, globalOutDegree=None, workerId=0, workerNum=1, routes=None,
+                 loopback=None):
+        """routes: dict with master_vertex, mirror_number, mirror_workers, mirror_vertex, master_worker (the contents
+        of Master.<i> / Mirror.<i>); loopback: the Loopback group that carries the exchange when workerNum > 1."""
         self.id, self.workerNum = workerId, workerNum
         self.comm = Comm()
         self.values = PRValues()
         self.g = CUDA_build_graph(globalVertexSize, len(u), u, v, workerId, workerNum, self.comm)
+        if routes is not None:
+            CUDA_AddMasterRoute(self.g, routes["master_vertex"], routes["mirror_number"], routes["mirror_workers"])
+            CUDA_AddMirrorRoute(self.g, routes["mirror_vertex"], routes["master_worker"])
+        if loopback is not None:
+            loopback.attach(workerId, self.comm)
         if globalOutDegree is None:
             globalOutDegree = np.bincount(np.asarray(u, np.int64), minlength=globalVertexSize)
         CUDA_LoadOutDegree(self.g, self.values, globalOutDegree)
@@ -82,7 +150,8 @@ class PRWorkerCUDA:
         v, g = self.values, self.g.contents
         return dict(pr=self._f32(v.prValue), acc=self._f32(v.accValue), diff=self._f32(v.diffValue),
                     globalAcc=float(self._f32(v.globalAcc, 1)[0]), globalDiff=float(self._f32(v.globalDiff, 1)[0]),
-                    active=self._i32(g.active), outDegree=self._i32(v.outDegree))
+                    active=self._i32(g.active), outDegree=self._i32(v.outDegree),
+                    updateByMessage=self._i32(g.updateByMessage))
 
     def graph_arrays(self):
         g = self.g.contents

@@ -52,6 +52,9 @@ class PRWorkerFromFiles:
         self.h = h
         self.n = lib().drone_pr_worker_local_size(h)
 
+    def attach_loopback(self, loopback):
+        check(lib().drone_pr_worker_attach_loopback(self.h, loopback.h))
+
     def peval(self):
         return lib().drone_pr_worker_peval(self.h)
 

@@ -67,7 +67,7 @@ typedef struct Graph {
 
 /* DRONE/src/cuda/graph.h:40-43: {ncclComm_t comm; cudaStream_t s}. */
 typedef struct Comm {
-    void *comm; /* RCCL communicator; NULL with one worker */
+    void *comm; /* a drone_transport* (section F); NULL with one worker */
     void *s;    /* hipStream_t created by build_graph      */
 } Comm;
 
@@ -280,6 +280,8 @@ int drone_stream_copy_f64(double *dst, const double *src, int64_t n, drone_strea
 
 /* Synchronous device-to-host copy (for hosts that have no HIP binding of their own, e.g. to read PRValues). */
 int drone_copy_to_host(void *dst_host, const void *src_device, size_t bytes);
+/* The other direction (e.g. to overwrite Graph::edgeLen with real edge lengths before SSSP_PEVal). */
+int drone_copy_to_device(void *dst_device, const void *src_host, size_t bytes);
 
 /* HIP-event stopwatch on a stream (bench harness plumbing). */
 typedef struct drone_timer drone_timer;
@@ -306,17 +308,82 @@ int drone_load_degree_file(const char *path, int **degree, int *count);         
 void drone_free_host(void *p);
 /* DRONE/src/worker/PRWorkerCUDA.go:115-175 (newPRWorkerCUDA) without the gRPC peers: reads
  * <data_path>/G.<self_id-1>, Master.<self_id-1>, Mirror.<self_id-1>, out_degree.txt, builds the graph, loads the
- * out-degrees.  self_id counts from 1 (0 is the master); worker_num must be 1 and the Master/Mirror files empty.
+ * out-degrees.  self_id counts from 1 (0 is the master).  With worker_num > 1 attach a transport before the first
+ * superstep (drone_pr_worker_attach_loopback for the workers of one process, each driven by its own thread).
  * peval / inceval are PRWorkerCUDA.go:52-65 / :76-88 minus the SuperStepFinish RPC. */
 typedef struct drone_pr_worker drone_pr_worker;
 int drone_pr_worker_create(drone_pr_worker **w, const char *data_path, int self_id, int worker_num,
                            int global_vertex_size);
+struct drone_loopback;
+int drone_pr_worker_attach_loopback(drone_pr_worker *w, struct drone_loopback *group); /* section F */
 Response drone_pr_worker_peval(drone_pr_worker *w);
 Response drone_pr_worker_inceval(drone_pr_worker *w);
 int drone_pr_worker_local_size(drone_pr_worker *w);
 int drone_pr_worker_read(drone_pr_worker *w, int *global_ids, float *pr); /* host [local size] each, may be NULL */
 int drone_pr_worker_run_f64(drone_pr_worker *w, double alpha, int iters, double *rank_out); /* host [local size] */
 int drone_pr_worker_destroy(drone_pr_worker *w);
+
+/* ====================================================================================== */
+/* F. Replica exchange between subgraphs, and the CC / SSSP jobs on the same boundary     */
+/* ====================================================================================== */
+/* With workerNum > 1 PR_PEVal / PR_IncEVal (and the CC / SSSP entry points below) end each superstep with the
+ * reference's two exchange phases, mirror -> master and master -> mirror (DRONE/src/cuda/algorithm/pr.cu:215-373,
+ * cc.cu:159-338), and fill Response's four send / receive counts.  Packing and applying run on the GPU; the
+ * wire is this function table, reached through Comm::comm (which holds an ncclComm_t in the reference,
+ * graph.h:40-43).  Calls block until the step is complete for this worker, like the reference's grouped
+ * ncclSend / ncclRecv followed by a stream synchronise.  All workers call in the same order. */
+typedef struct drone_transport {
+    void *ctx;
+    /* Worker `workerId` sends, to every other worker w, send_len[w] ids and 4-byte values starting at element
+     * send_index[w] of send_id / send_val (device), and receives into recv_id / recv_val (device, room for
+     * recv_capacity elements) what the others send to it, packed in ascending source-worker order;
+     * recv_len[w] (host [workerNum]) receives the count that came from w (0 for itself).  send_len and
+     * send_index are host arrays.  Returns 0 or a negative drone_status. */
+    int (*exchange)(void *ctx, int workerId, int workerNum, const int *send_len, const int *send_index,
+                    const int *send_id, const void *send_val, int *recv_len, int *recv_id, void *recv_val,
+                    int recv_capacity, drone_stream_t stream);
+    /* *device_scalar becomes the sum over all workers' values, added in worker order on every worker. */
+    int (*allreduce_sum_f32)(void *ctx, int workerId, int workerNum, float *device_scalar, drone_stream_t stream);
+} drone_transport;
+
+/* In-process transport for several subgraphs on one GPU: every worker of the group is driven by its own host
+ * thread (as the Go runtime drives one worker per process), and the calls above meet at a barrier and copy device
+ * to device.  drone_loopback_attach stores the worker's endpoint in comm->comm; call it after build_graph, which
+ * clears that field.  A worker that waits longer than timeout_ms for its peers fails with DRONE_ERR_INVALID
+ * instead of hanging (0 = wait for ever).  No counterpart in the reference. */
+typedef struct drone_loopback drone_loopback;
+int drone_loopback_create(drone_loopback **group, int workerNum, int timeout_ms);
+int drone_loopback_attach(drone_loopback *group, int workerId, Comm *comm);
+int drone_loopback_destroy(drone_loopback *group);
+
+/* DRONE/src/cuda/algorithm/cc.h:17-25.  Same fields; `ext` appended. */
+typedef struct CCValues {
+    int *sendID, *recvID;
+    int *sendCCValue, *recvCCValue;
+    int *ccValue; /* device [local] */
+    void *ext;
+} CCValues;
+/* cc.cu:340-447.  Label propagation to the local fixed point: ccValue starts as the LOCAL id (cc.cu:17) and
+ * becomes the minimum over everything that reaches the vertex along out-edges; then the exchange.  g->active
+ * is > 0 for vertices lowered by propagation in this call, 0 for vertices a message activated (and for every
+ * vertex at PEVal that was never lowered), -1 otherwise; VisitedSize counts active != 0 (common.cu:17-31). */
+Response CC_PEVal(Graph *g, CCValues *values, int workerId, int workerNum, Comm *comm);
+Response CC_IncEVal(Graph *g, CCValues *values, int workerId, int workerNum, Comm *comm);
+void drone_cc_values_destroy(Graph *g, CCValues *values);
+
+/* DRONE/src/cuda/algorithm/sssp.h:17-25.  Same fields; `ext` appended. */
+typedef struct SSSPValues {
+    int *sendID, *recvID;
+    float *sendDis, *recvDis;
+    float *distance; /* device [local]; 1e8 = not reached (sssp.cu:33) */
+    void *ext;
+} SSSPValues;
+/* sssp.cu:398-539.  Relaxation over g->edgeLen (1.0 after build_graph) from global vertex startId to the local
+ * fixed point, then the exchange.  A relaxation counts as an update when it lowers the distance by more than
+ * 1e-6 (sssp.cu:64). */
+Response SSSP_PEVal(Graph *g, SSSPValues *values, int startId, int workerId, int workerNum, Comm *comm);
+Response SSSP_IncEVal(Graph *g, SSSPValues *values, int workerId, int workerNum, Comm *comm);
+void drone_sssp_values_destroy(Graph *g, SSSPValues *values);
 
 #ifdef __cplusplus
 }

@@ -14,7 +14,7 @@ _SO = os.path.join(_HERE, "liboracle.so")
 
 
 def build(force=False):
-    srcs = [os.path.join(_HERE, f) for f in ("oracle_pr.c", "oracle_gcn.c", "Makefile")]
+    srcs = [os.path.join(_HERE, f) for f in ("oracle_pr.c", "oracle_gcn.c", "oracle_traverse.c", "Makefile")]
     stale = (not os.path.exists(_SO)) or any(os.path.getmtime(s) > os.path.getmtime(_SO) for s in srcs)
     if force or stale:
         subprocess.check_call(["make", "-C", _HERE, "-B", "liboracle.so"], stdout=subprocess.DEVNULL)
@@ -104,6 +104,177 @@ class PushState:
         return f(C.c_int(self.n), C.c_int(self.nglobal), _p(self.index), _p(self.dst), _p(self.outdeg),
                  _p(self.m2w), self.ct(alpha), self.ct(eps), _p(self.pr), _p(self.acc), _p(self.diff),
                  _p(self.gacc), _p(self.gdiff), _p(self.active))
+
+
+# ---- replica exchange between the subgraphs of a vertex cut ---------------------------------------------------
+class Part:
+    """Routing tables of one worker as DRONE/src/cuda/graph.cu:260-331 builds them: Mirror2Worker[local] (master
+    worker of a mirror, -1 otherwise) and, per local master, the list of workers that hold a mirror of it."""
+
+    def __init__(self, l2g, nglobal, master_vertex=(), mirror_number=(), mirror_workers=(), mirror_vertex=(),
+                 master_worker=()):
+        self.l2g = np.asarray(l2g, np.int64)
+        self.n = len(self.l2g)
+        self.g2l = np.full(nglobal, -1, np.int64)
+        self.g2l[self.l2g] = np.arange(self.n)
+        self.m2w = np.full(self.n, -1, np.int64)
+        for gv, w in zip(mirror_vertex, master_worker):
+            self.m2w[self.g2l[gv]] = w
+        self.master_workers = {}
+        k = 0
+        for gv, cnt in zip(master_vertex, mirror_number):
+            self.master_workers[int(self.g2l[gv])] = [int(w) for w in mirror_workers[k:k + cnt]]
+            k += cnt
+        self.active = np.zeros(self.n, np.int32)
+        self.ubm = np.zeros(self.n, np.int32)  # updateByMessage
+
+
+def exchange_phase(parts, vals, phase, send_mirror, send_master, combine):
+    """One phase of DRONE/src/cuda/algorithm/pr.cu:215-373 (the same skeleton in cc.cu:159-338 and sssp.cu) over
+    all workers at once.  phase 0: every mirror with send_mirror(active) sends its value to its master's worker
+    (pr.cu:89-102, :123-145); phase 1: every master with send_master(active, updateByMessage) sends its value to
+    all its mirror workers (pr.cu:104-121, :147-171).  Receivers apply combine(phase, old, value) -> (new, flag)
+    and OR the flag into updateByMessage (pr.cu:173-213), source workers in ascending order.  Returns
+    (sent[w], received[w])."""
+    W = len(parts)
+    box = [[[] for _ in range(W)] for _ in range(W)]  # box[src][dst] = [(global id, value)]
+    for w, p in enumerate(parts):
+        if phase == 0:
+            for v in np.nonzero(p.m2w != -1)[0]:
+                if send_mirror(p.active[v]):
+                    box[w][p.m2w[v]].append((p.l2g[v], vals[w][v]))
+        else:
+            for v in sorted(p.master_workers):
+                if send_master(p.active[v], p.ubm[v]):
+                    for dst in p.master_workers[v]:
+                        box[w][dst].append((p.l2g[v], vals[w][v]))
+    sent = [sum(len(box[w][d]) for d in range(W)) for w in range(W)]
+    recv = [sum(len(box[s][w]) for s in range(W)) for w in range(W)]
+    for dst, p in enumerate(parts):
+        for src in range(W):
+            for gid, val in box[src][dst]:
+                l = p.g2l[gid]
+                assert l >= 0, "message for a vertex that is not on the worker"
+                new, flag = combine(phase, vals[dst][l], val)
+                vals[dst][l] = new
+                if flag:
+                    p.ubm[l] = 1
+    return sent, recv
+
+
+class PushGroup:
+    """PR_PEVal / PR_IncEVal over several workers (pr.cu:375-428, :450-488): the single-worker restatement per
+    worker, then the two exchange phases and the sum of globalDiff over the workers (pr.cu:365)."""
+
+    def __init__(self, states, parts):
+        self.states, self.parts = states, parts
+
+    def _finish(self, visited):
+        sts, parts = self.states, self.parts
+        for st, p in zip(sts, parts):
+            p.active = st.active
+        diffs = [st.diff for st in sts]
+        dt = sts[0].dtype.type
+        add = lambda ph, old, v: ((dt(old) + dt(v)) if ph == 0 else dt(v), True)  # atomicAdd / atomicExch, flag always
+        s0, r0 = exchange_phase(parts, diffs, 0, lambda a: a != 0, None, add)
+        s1, r1 = exchange_phase(parts, diffs, 1, None, lambda a, u: a != 0 or u != 0, add)
+        total = dt(0)
+        for st in sts:
+            total = dt(total + st.gdiff[0])
+        for st in sts:
+            st.gdiff[0] = total
+        return [dict(VisitedSize=visited[w], Mirror2MasterSendSize=s0[w], Mirror2MasterRecvSize=r0[w],
+                     Master2MirrorSendSize=s1[w], Master2MirrorRecvSize=r1[w]) for w in range(len(sts))]
+
+    def peval(self):
+        for p in self.parts:
+            p.ubm[:] = 0
+        return self._finish([st.peval() for st in self.states])
+
+    def inceval(self, alpha=0.85, eps=1e-6):
+        for p in self.parts:
+            p.ubm[:] = 0  # pr.cu:440
+        return self._finish([st.inceval(alpha, eps) for st in self.states])
+
+
+class CCState:
+    """CC_PEVal / CC_IncEVal compute of one worker (cc.cu:340-447 without the exchange)."""
+
+    def __init__(self, index, dst):
+        self.index, self.dst = _i32(index), _i32(dst)
+        self.n = len(self.index) - 1
+        self.val = np.zeros(self.n, np.int32)
+        self.active = np.zeros(self.n, np.int32)
+
+    def peval(self):
+        lib().orc_cc_init(C.c_int(self.n), _p(self.val), _p(self.active))
+        self.rounds = lib().orc_cc_rounds(C.c_int(self.n), _p(self.index), _p(self.dst), _p(self.val),
+                                          _p(self.active), C.c_int(1 if self.n > 0 else 0))
+
+    def inceval(self, ubm):
+        up = lib().orc_process_messages(C.c_int(self.n), _p(self.active), _p(ubm))
+        self.rounds = lib().orc_cc_rounds(C.c_int(self.n), _p(self.index), _p(self.dst), _p(self.val),
+                                          _p(self.active), C.c_int(up))
+
+    def visited(self):
+        return lib().orc_count_active(C.c_int(self.n), _p(self.active))
+
+
+class SSSPState:
+    """SSSP_PEVal / SSSP_IncEVal compute of one worker (sssp.cu:398-539 without the exchange)."""
+
+    def __init__(self, index, dst, edge_len=None):
+        self.index, self.dst = _i32(index), _i32(dst)
+        self.n = len(self.index) - 1
+        self.len = _f32(edge_len) if edge_len is not None else np.ones(len(self.dst), np.float32)
+        self.val = np.zeros(self.n, np.float32)
+        self.active = np.zeros(self.n, np.int32)
+
+    def peval(self, start_local):
+        lib().orc_sssp_init(C.c_int(self.n), C.c_int(start_local), _p(self.val), _p(self.active))
+        self.rounds = lib().orc_sssp_rounds(C.c_int(self.n), _p(self.index), _p(self.dst), _p(self.len),
+                                            _p(self.val), _p(self.active), C.c_int(1 if start_local >= 0 else 0))
+
+    def inceval(self, ubm):
+        up = lib().orc_process_messages(C.c_int(self.n), _p(self.active), _p(ubm))
+        self.rounds = lib().orc_sssp_rounds(C.c_int(self.n), _p(self.index), _p(self.dst), _p(self.len),
+                                            _p(self.val), _p(self.active), C.c_int(up))
+
+    def visited(self):
+        return lib().orc_count_active(C.c_int(self.n), _p(self.active))
+
+
+class TraverseGroup:
+    """CC or SSSP over several workers: per-worker compute, then the two exchange phases with min-combine
+    (cc.cu:135-157 / sssp.cu:163-185: the replica is lowered and flagged when the message is smaller)."""
+
+    def __init__(self, states, parts):
+        self.states, self.parts = states, parts
+
+    def _finish(self):
+        sts, parts = self.states, self.parts
+        for st, p in zip(sts, parts):
+            p.active = st.active
+        vals = [st.val for st in sts]
+        lower = lambda ph, old, v: (min(old, v), old > v)
+        s0, r0 = exchange_phase(parts, vals, 0, lambda a: a > 0, None, lower)
+        s1, r1 = exchange_phase(parts, vals, 1, None, lambda a, u: a > 0 or u != 0, lower)
+        return [dict(VisitedSize=sts[w].visited(), Mirror2MasterSendSize=s0[w], Mirror2MasterRecvSize=r0[w],
+                     Master2MirrorSendSize=s1[w], Master2MirrorRecvSize=r1[w]) for w in range(len(sts))]
+
+    def peval(self, start_global=None):
+        for st, p in zip(self.states, self.parts):
+            p.ubm[:] = 0
+            if start_global is None:
+                st.peval()
+            else:
+                st.peval(int(p.g2l[start_global]))
+        return self._finish()
+
+    def inceval(self):
+        for st, p in zip(self.states, self.parts):
+            st.inceval(p.ubm)  # process_messages clears the flags it consumes
+        return self._finish()
 
 
 class GoPR:

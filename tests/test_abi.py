@@ -50,6 +50,9 @@ def test_struct_layouts_match_reference():
     assert (g.gridSize.offset, g.blockSize.offset, g.active.offset, g.updateByMessage.offset, g.GID.offset) == (104, 108, 112, 120, 128)
     # pr.h:7-16: ten pointers, then ext
     assert _lib.PRValues.outDegree.offset == 72 and _lib.PRValues.ext.offset == 80
+    # cc.h:17-25 / sssp.h:17-25: five pointers, then ext
+    assert _lib.CCValues.ccValue.offset == 32 and _lib.CCValues.ext.offset == 40
+    assert _lib.SSSPValues.distance.offset == 32 and _lib.SSSPValues.ext.offset == 40
 
 
 def test_version_and_error_channel():
@@ -125,3 +128,34 @@ def test_gcn_entry_points_validate_arguments_on_the_host():
     cfg = _lib.GcnConfig(0, 1, 1, 1, 0.5, 0.01, 0.0, 0, 1, 0, 1)
     assert L.drone_gcn_create(C.byref(h), C.byref(cfg), 0, None, None, None, None, None, 1, None, None, None, None, None) == -1
     assert L.drone_pr_plan_create_ex(C.byref(h), 10, 0, None, None, None, 4, None) == -1
+
+
+class _Transport(C.Structure):
+    """drone_transport of include/drone_hip.h"""
+    _EX = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                      C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p)
+    _AR = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p)
+    _fields_ = [("ctx", C.c_void_p), ("exchange", _EX), ("allreduce_sum_f32", _AR)]
+
+
+def test_loopback_transport_times_out_instead_of_hanging():
+    """A worker whose peer never arrives gets an error after timeout_ms; the group then stays broken.  Runs
+    without a GPU: the barrier comes before any device call."""
+    L = _lib.lib()
+    grp = C.c_void_p()
+    assert L.drone_loopback_create(C.byref(grp), 0, 10) == -1
+    assert L.drone_loopback_create(C.byref(grp), 2, -1) == -1
+    assert L.drone_loopback_create(C.byref(grp), 2, 50) == 0
+    comm = _lib.Comm()
+    assert L.drone_loopback_attach(grp, 2, C.byref(comm)) == -1      # workerId out of range
+    assert L.drone_loopback_attach(grp, 0, C.byref(comm)) == 0
+    tr = C.cast(comm.comm, C.POINTER(_Transport)).contents
+    send_len = (C.c_int * 2)(0, 0)
+    send_index = (C.c_int * 3)(0, 0, 0)
+    recv_len = (C.c_int * 2)(7, 7)
+    rc = tr.exchange(tr.ctx, 0, 2, send_len, send_index, None, None, recv_len, None, None, 1, None)
+    assert rc == -1 and b"did not arrive" in L.drone_last_error_string()
+    rc = tr.exchange(tr.ctx, 0, 2, send_len, send_index, None, None, recv_len, None, None, 1, None)
+    assert rc == -1                                                  # broken for good
+    assert tr.exchange(tr.ctx, 0, 3, send_len, send_index, None, None, recv_len, None, None, 1, None) == -1
+    assert L.drone_loopback_destroy(grp) == 0

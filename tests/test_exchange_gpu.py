@@ -1,0 +1,107 @@
+"""Several subgraphs of a vertex cut on one GPU: PR_PEVal / PR_IncEVal with the replica exchange over the
+in-process loopback transport, against the oracle's multi-worker restatement of pr.cu:215-488 and against the
+single-subgraph run of the whole graph."""
+import numpy as np
+import pytest
+
+from partition_util import vertex_cut
+
+pytestmark = pytest.mark.gpu
+
+
+def _graph(scale, ef, seed):
+    from drone_amd import rmat
+    s, d = rmat.rmat_edges(scale, ef << scale, seed=seed)
+    s, d = s.astype(np.int64), d.astype(np.int64)
+    keep = s != d
+    key = np.unique((s[keep] << 32) | d[keep])
+    return (key >> 32).astype(np.int32), (key & 0xFFFFFFFF).astype(np.int32)
+
+
+def _oracle_group(oracle, nglobal, parts, outdeg, dtype=np.float32):
+    states, tops = [], []
+    for p in parts:
+        n, g2l, l2g, index, dst = oracle.build_graph(nglobal, p["u"], p["v"])
+        top = oracle.Part(l2g, nglobal, p["master_vertex"], p["mirror_number"], p["mirror_workers"],
+                          p["mirror_vertex"], p["master_worker"])
+        states.append(oracle.PushState(index, dst, outdeg[l2g], nglobal, dtype=dtype, mirror2worker=top.m2w))
+        tops.append(top)
+    return oracle.PushGroup(states, tops)
+
+
+FIELDS = ["VisitedSize", "Mirror2MasterSendSize", "Mirror2MasterRecvSize", "Master2MirrorSendSize",
+          "Master2MirrorRecvSize"]
+
+
+@pytest.mark.parametrize("W,scale,seed", [(2, 8, 1), (3, 10, 2), (4, 12, 3), (7, 11, 4)])
+def test_pr_group_matches_oracle_group(oracle, W, scale, seed):
+    from drone_amd.pagerank import Loopback, PRWorkerCUDA, run_workers
+    nglobal = 1 << scale
+    u, v = _graph(scale, 8, seed)
+    outdeg = np.bincount(u, minlength=nglobal).astype(np.int32)
+    parts, _ = vertex_cut(u, v, W, seed)
+    grp = _oracle_group(oracle, nglobal, parts, outdeg)
+    lb = Loopback(W, timeout_ms=60000)
+    ws = [PRWorkerCUDA(nglobal, p["u"], p["v"], outdeg, workerId=i, workerNum=W, routes=p, loopback=lb)
+          for i, p in enumerate(parts)]
+    try:
+        for step in range(4):
+            want = grp.peval() if step == 0 else grp.inceval()
+            got = run_workers([(w.peval if step == 0 else w.incEval) for w in ws])
+            for i, w in enumerate(ws):
+                for f in FIELDS:
+                    assert getattr(got[i], f) == want[i][f], (step, i, f)
+                assert got[i].LocalVertexSize == grp.states[i].n
+                st = w.state()
+                np.testing.assert_allclose(st["diff"], grp.states[i].diff, rtol=2e-5, atol=1e-6)
+                np.testing.assert_allclose(st["pr"], grp.states[i].pr, rtol=2e-5, atol=1e-6)
+                np.testing.assert_allclose(st["globalDiff"], grp.states[i].gdiff[0], rtol=2e-5, atol=1e-7)
+                np.testing.assert_array_equal(st["updateByMessage"], grp.parts[i].ubm)
+    finally:
+        for w in ws:
+            w.close()
+        lb.close()
+
+
+def test_pr_group_equals_whole_graph(oracle):
+    """Every replica ends with the value the single-subgraph run gives the vertex."""
+    from drone_amd.pagerank import Loopback, PRWorkerCUDA, run_workers
+    scale, W = 12, 3
+    nglobal = 1 << scale
+    u, v = _graph(scale, 8, 7)
+    outdeg = np.bincount(u, minlength=nglobal).astype(np.int32)
+    parts, _ = vertex_cut(u, v, W, 5)
+    whole = PRWorkerCUDA(nglobal, u, v, outdeg)
+    lb = Loopback(W, timeout_ms=60000)
+    ws = [PRWorkerCUDA(nglobal, p["u"], p["v"], outdeg, workerId=i, workerNum=W, routes=p, loopback=lb)
+          for i, p in enumerate(parts)]
+    try:
+        whole.peval()
+        run_workers([w.peval for w in ws])
+        for _ in range(10):
+            whole.incEval()
+            run_workers([w.incEval for w in ws])
+        ref = np.zeros(nglobal, np.float32)
+        ref[whole.graph_arrays()["Local2Global"]] = whole.state()["pr"]
+        for w in ws:
+            l2g = w.graph_arrays()["Local2Global"]
+            np.testing.assert_allclose(w.state()["pr"], ref[l2g], rtol=1e-4, atol=1e-5)
+    finally:
+        whole.close()
+        for w in ws:
+            w.close()
+        lb.close()
+
+
+def test_exchange_without_transport_is_refused(oracle):
+    """workerNum > 1 with an empty Comm::comm must not silently skip the exchange."""
+    import ctypes as C
+    from drone_amd import _lib
+    from drone_amd.pagerank import PRWorkerCUDA
+    u, v = _graph(6, 4, 1)
+    w = PRWorkerCUDA(64, u, v, workerId=0, workerNum=1)
+    try:
+        w.peval()
+        assert w.values.sendID is None  # one subgraph: no staging, as before
+    finally:
+        w.close()

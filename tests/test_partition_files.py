@@ -75,8 +75,8 @@ def test_worker_create_rejects_bad_partitions(tmp_path):
     write_partition(tmp_path, [0, 1], [1, 2], [1, 1])
     with pytest.raises(_lib.DroneError, match="fewer than"):
         pf.PRWorkerFromFiles(tmp_path, 3)
-    with pytest.raises(_lib.DroneError, match="one worker"):
-        pf.PRWorkerFromFiles(tmp_path, 3, self_id=2, worker_num=2)
+    with pytest.raises(_lib.DroneError, match="self_id"):
+        pf.PRWorkerFromFiles(tmp_path, 3, self_id=3, worker_num=2)
 
 
 @pytest.mark.gpu
@@ -112,3 +112,48 @@ def test_worker_from_files_matches_oracle(tmp_path, oracle):
     got = w.run_f64(0.85, 20)
     assert np.max(np.abs(got - ref) / ref) <= 1e-9
     w.close()
+
+
+@pytest.mark.gpu
+def test_workers_from_files_with_replicas_match_oracle_group(tmp_path, oracle):
+    """Three subgraphs of a vertex cut read from G.i / Master.i / Mirror.i, driven as three workers of one process
+    over the loopback transport: same states and exchange counts as the oracle's multi-worker restatement."""
+    from partition_util import vertex_cut, write_partition_files
+    from drone_amd import rmat
+    from drone_amd.pagerank import Loopback, run_workers
+    s, d = rmat.rmat_edges(10, 1024 * 8, seed=9)
+    u, v = rmat.clean_directed_np(s, d)
+    gN, W = 1024, 3
+    outdeg = np.bincount(u, minlength=gN).astype(np.int32)
+    parts, _ = vertex_cut(u, v, W, 9)
+    write_partition_files(str(tmp_path), parts, outdeg)
+    states, tops = [], []
+    for p in parts:
+        n, g2l, l2g, index, dst = oracle.build_graph(gN, p["u"], p["v"])
+        top = oracle.Part(l2g, gN, p["master_vertex"], p["mirror_number"], p["mirror_workers"], p["mirror_vertex"],
+                          p["master_worker"])
+        states.append(oracle.PushState(index, dst, outdeg[l2g], gN, mirror2worker=top.m2w))
+        tops.append(top)
+    grp = oracle.PushGroup(states, tops)
+    lb = Loopback(W, timeout_ms=60000)
+    ws = [pf.PRWorkerFromFiles(str(tmp_path), gN, self_id=i + 1, worker_num=W) for i in range(W)]
+    try:
+        for w in ws:
+            w.attach_loopback(lb)
+        for step in range(4):
+            want = grp.peval() if step == 0 else grp.inceval()
+            got = run_workers([(w.peval if step == 0 else w.incEval) for w in ws])
+            for i in range(W):
+                for f in ("VisitedSize", "Mirror2MasterSendSize", "Mirror2MasterRecvSize", "Master2MirrorSendSize",
+                          "Master2MirrorRecvSize"):
+                    assert getattr(got[i], f) == want[i][f], (step, i, f)
+        for i, w in enumerate(ws):
+            ids, pr = w.read()
+            np.testing.assert_array_equal(ids, tops[i].l2g)
+            np.testing.assert_allclose(pr, states[i].pr, rtol=2e-5)
+            with pytest.raises(_lib.DroneError, match="replicated"):
+                w.run_f64(0.85, 2)
+    finally:
+        for w in ws:
+            w.close()
+        lb.close()

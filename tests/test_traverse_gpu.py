@@ -1,0 +1,160 @@
+"""CC_PEVal / CC_IncEVal and SSSP_PEVal / SSSP_IncEVal against the oracle's restatement of cc.cu / sssp.cu:
+bit-exact labels and distances, the sign class of g->active, VisitedSize and the four exchange counts."""
+import numpy as np
+import pytest
+
+from partition_util import vertex_cut
+
+pytestmark = pytest.mark.gpu
+
+FIELDS = ["VisitedSize", "Mirror2MasterSendSize", "Mirror2MasterRecvSize", "Master2MirrorSendSize",
+          "Master2MirrorRecvSize"]
+
+
+def _rmat(scale, ef, seed, symmetric=False):
+    from drone_amd import rmat
+    s, d = rmat.rmat_edges(scale, ef << scale, seed=seed)
+    s, d = s.astype(np.int64), d.astype(np.int64)
+    keep = s != d
+    s, d = s[keep], d[keep]
+    if symmetric:
+        s, d = np.concatenate([s, d]), np.concatenate([d, s])
+    key = np.unique((s << 32) | d)
+    return (key >> 32).astype(np.int32), (key & 0xFFFFFFFF).astype(np.int32)
+
+
+def _chain(n):
+    return np.arange(n - 1, dtype=np.int32), np.arange(1, n, dtype=np.int32)
+
+
+def _sign(a):
+    return np.sign(a)
+
+
+CASES = [("rmat10", lambda: _rmat(10, 8, 1)), ("rmat14_sym", lambda: _rmat(14, 8, 2, True)),
+         ("rmat16", lambda: _rmat(16, 16, 3)), ("chain300", lambda: _chain(300)),
+         ("one_edge", lambda: (np.array([3], np.int32), np.array([1], np.int32)))]
+
+
+@pytest.mark.parametrize("name,make", CASES, ids=[c[0] for c in CASES])
+def test_cc_single_worker(oracle, name, make):
+    from drone_amd.traverse import CCWorkerCUDA
+    u, v = make()
+    nglobal = int(max(u.max(), v.max())) + 1
+    n, g2l, l2g, index, dst = oracle.build_graph(nglobal, u, v)
+    st = oracle.CCState(index, dst)
+    st.peval()
+    w = CCWorkerCUDA(nglobal, u, v)
+    try:
+        res = w.peval()
+        np.testing.assert_array_equal(w.read(), st.val)
+        np.testing.assert_array_equal(_sign(w.flags()["active"]), _sign(st.active))
+        assert res.VisitedSize == st.visited() and res.LocalVertexSize == n
+        assert res.Mirror2MasterSendSize == 0 and res.Master2MirrorRecvSize == 0
+        # IncEVal without messages: nothing runs, every vertex is "untouched" (-1) and counted (cc.cu:398-400)
+        res = w.incEval()
+        st.inceval(np.zeros(n, np.int32))
+        np.testing.assert_array_equal(w.read(), st.val)
+        np.testing.assert_array_equal(w.flags()["active"], st.active)
+        assert res.VisitedSize == n
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("name,make", CASES, ids=[c[0] for c in CASES])
+def test_sssp_single_worker(oracle, name, make):
+    from drone_amd.traverse import SSSPWorkerCUDA
+    u, v = make()
+    nglobal = int(max(u.max(), v.max())) + 1
+    n, g2l, l2g, index, dst = oracle.build_graph(nglobal, u, v)
+    start = int(u[0])
+    st = oracle.SSSPState(index, dst)
+    st.peval(int(g2l[start]))
+    w = SSSPWorkerCUDA(nglobal, u, v, startId=start)
+    try:
+        res = w.peval()
+        np.testing.assert_array_equal(w.read(), st.val)
+        np.testing.assert_array_equal(_sign(w.flags()["active"]), _sign(st.active))
+        assert res.VisitedSize == st.visited() and res.LocalVertexSize == n
+    finally:
+        w.close()
+
+
+def test_sssp_start_vertex_absent(oracle):
+    """Global2Local[startId] == -1: nothing is reached, every vertex counts as visited (active == -1)."""
+    from drone_amd.traverse import SSSPWorkerCUDA
+    u, v = np.array([5, 6], np.int32), np.array([6, 7], np.int32)
+    w = SSSPWorkerCUDA(10, u, v, startId=0)
+    try:
+        res = w.peval()
+        np.testing.assert_array_equal(w.read(), np.full(3, 1e8, np.float32))
+        assert res.VisitedSize == 3
+    finally:
+        w.close()
+
+
+def test_sssp_edge_lengths(oracle):
+    """g->edgeLen is honoured (build_graph fills it with 1.0; a caller may overwrite it)."""
+    from drone_amd.traverse import SSSPWorkerCUDA
+    u, v = _rmat(12, 8, 5)
+    nglobal = 1 << 12
+    n, g2l, l2g, index, dst = oracle.build_graph(nglobal, u, v)
+    length = np.random.default_rng(0).integers(1, 9, len(dst)).astype(np.float32)
+    st = oracle.SSSPState(index, dst, length)
+    st.peval(int(g2l[u[0]]))
+    w = SSSPWorkerCUDA(nglobal, u, v, startId=int(u[0]))
+    try:
+        w.set_edge_len(length)
+        w.peval()
+        np.testing.assert_array_equal(w.read(), st.val)
+    finally:
+        w.close()
+
+
+def _group(oracle, kind, nglobal, parts):
+    states, tops = [], []
+    for p in parts:
+        n, g2l, l2g, index, dst = oracle.build_graph(nglobal, p["u"], p["v"])
+        tops.append(oracle.Part(l2g, nglobal, p["master_vertex"], p["mirror_number"], p["mirror_workers"],
+                                p["mirror_vertex"], p["master_worker"]))
+        states.append(oracle.CCState(index, dst) if kind == "cc" else oracle.SSSPState(index, dst))
+    return oracle.TraverseGroup(states, tops)
+
+
+@pytest.mark.parametrize("kind", ["cc", "sssp"])
+@pytest.mark.parametrize("W,scale,seed", [(2, 9, 1), (3, 12, 2), (5, 11, 3)])
+def test_group_matches_oracle_group(oracle, kind, W, scale, seed):
+    from drone_amd.pagerank import Loopback, run_workers
+    from drone_amd.traverse import CCWorkerCUDA, SSSPWorkerCUDA
+    nglobal = 1 << scale
+    u, v = _rmat(scale, 8, seed, symmetric=(kind == "cc"))
+    parts, _ = vertex_cut(u, v, W, seed)
+    grp = _group(oracle, kind, nglobal, parts)
+    start = int(u[0])
+    lb = Loopback(W, timeout_ms=60000)
+    if kind == "cc":
+        ws = [CCWorkerCUDA(nglobal, p["u"], p["v"], workerId=i, workerNum=W, routes=p, loopback=lb)
+              for i, p in enumerate(parts)]
+    else:
+        ws = [SSSPWorkerCUDA(nglobal, p["u"], p["v"], workerId=i, workerNum=W, routes=p, loopback=lb, startId=start)
+              for i, p in enumerate(parts)]
+    try:
+        for step in range(12):
+            if step == 0:
+                want = grp.peval(start) if kind == "sssp" else grp.peval()
+            else:
+                want = grp.inceval()
+            got = run_workers([(w.peval if step == 0 else w.incEval) for w in ws])
+            for i, w in enumerate(ws):
+                for f in FIELDS:
+                    assert getattr(got[i], f) == want[i][f], (step, i, f)
+                np.testing.assert_array_equal(w.read(), grp.states[i].val)
+                fl = w.flags()
+                np.testing.assert_array_equal(_sign(fl["active"]), _sign(grp.states[i].active))
+                np.testing.assert_array_equal(fl["updateByMessage"], grp.parts[i].ubm)
+            if sum(r["Mirror2MasterSendSize"] + r["Master2MirrorSendSize"] for r in want) == 0:
+                break
+    finally:
+        for w in ws:
+            w.close()
+        lb.close()
