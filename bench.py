@@ -238,6 +238,55 @@ def bench_spmm_sweep():
     return out
 
 
+def bench_traverse(cpu_baseline=True):
+    """SSSP_PEVal (unit lengths, directed R-MAT scale 22 ef 16 seed 2) and CC_PEVal (the same graph symmetrised) through
+    the Go worker's boundary: one subgraph to its local fixed point.  TEPS = edges of the subgraph / time of the call.
+    The CPU figure is the oracle's serial restatement of sssp.cu / cc.cu, one thread."""
+    import numpy as np
+    from drone_amd import rmat
+    from drone_amd.traverse import CCWorkerCUDA, SSSPWorkerCUDA
+    scale = 22
+    s, d = rmat.rmat_edges(scale, 16 << scale, seed=2)
+    u, v = rmat.clean_directed_np(s, d)
+    n = 1 << scale
+    out = {"workload": f"SSSP / CC to the local fixed point, R-MAT scale {scale} ef 16 seed 2, one subgraph"}
+
+    def run(worker, edges, name):
+        worker.peval()
+        ms = min(timed_ms(worker.peval) for _ in range(3))
+        out[name] = {"edges": int(edges), "local_vertices": int(worker.n), "peval_ms": ms,
+                     "GTEPS": edges / (ms * 1e-3) / 1e9}
+        return worker.read()
+
+    def timed_ms(fn):
+        t = time.perf_counter()
+        fn()
+        return (time.perf_counter() - t) * 1e3
+
+    w = SSSPWorkerCUDA(n, u, v, startId=int(u[0]))
+    dist = run(w, len(u), "sssp")
+    w.close()
+    us, vs = np.concatenate([u, v]).astype(np.int64), np.concatenate([v, u]).astype(np.int64)
+    key = np.unique((us << 32) | vs)
+    us, vs = (key >> 32).astype(np.int32), (key & 0xFFFFFFFF).astype(np.int32)
+    w = CCWorkerCUDA(n, us, vs)
+    lab = run(w, len(us), "cc")
+    w.close()
+    if cpu_baseline:
+        from oracle import oracle
+        nl, g2l, l2g, index, dst = oracle.build_graph(n, u, v)
+        st = oracle.SSSPState(index, dst)
+        ms = timed_ms(lambda: st.peval(int(g2l[u[0]])))
+        out["sssp"]["cpu_baseline"] = {"value": len(u) / (ms * 1e-3) / 1e9, "unit": "GTEPS", "cores": 1, "kind": "port",
+                                       "ms": ms, "identical": bool(np.array_equal(st.val, dist))}
+        nl, g2l, l2g, index, dst = oracle.build_graph(n, us, vs)
+        st = oracle.CCState(index, dst)
+        ms = timed_ms(st.peval)
+        out["cc"]["cpu_baseline"] = {"value": len(us) / (ms * 1e-3) / 1e9, "unit": "GTEPS", "cores": 1, "kind": "port",
+                                     "ms": ms, "identical": bool(np.array_equal(st.val, lab))}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -249,8 +298,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="launch the 1 GiB stream-copy kernel exactly once (a dispatch of known traffic to scale "
                          "rocprofv3 byte counters by)")
-    ap.add_argument("--suite", default="default", choices=["pr", "default", "full", "gcn", "sweep"],
-                    help="pr: PageRank only; default: + GCN training step (configs[3]); full: + configs[2] and [4]")
+    ap.add_argument("--suite", default="default", choices=["pr", "default", "full", "gcn", "sweep", "traverse"],
+                    help="pr: PageRank only; default: + GCN training step (configs[3]); full: + configs[2], [4] and the "
+                         "SSSP / CC jobs; gcn, sweep, traverse: that part alone")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs one subgraph on ONE GPU; there is no multi-GPU path to time "
@@ -273,8 +323,11 @@ def main():
     del a, b
     torch.cuda.empty_cache()
 
-    if args.suite in ("gcn", "sweep"):      # profiling helpers: GCN parts alone, no headline line
-        part = bench_gcn_step(steps=max(3, args.steps), warmup=max(1, args.warmup)) if args.suite == "gcn" else bench_spmm_sweep()
+    if args.suite in ("gcn", "sweep", "traverse"):      # profiling helpers: one part alone, no headline line
+        if args.suite == "traverse":
+            part = bench_traverse(cpu_baseline=not args.no_cpu_baseline)
+        else:
+            part = bench_gcn_step(steps=max(3, args.steps), warmup=max(1, args.warmup)) if args.suite == "gcn" else bench_spmm_sweep()
         print(json.dumps(part), flush=True)
         return
 
@@ -348,6 +401,8 @@ def main():
         result["gcn_layer"] = bench_gcn_layer()
         torch.cuda.empty_cache()
         result["spmm_sweep"] = bench_spmm_sweep()
+        torch.cuda.empty_cache()
+        result["traverse"] = bench_traverse(cpu_baseline=not args.no_cpu_baseline)
     print(json.dumps(result), flush=True)
 
 
