@@ -225,8 +225,11 @@ int drone::exchange_phase(Graph *g, int phase, typename Policy::T *vals, int *se
     std::vector<int> send_len((size_t)workerNum), recv_len((size_t)workerNum, 0);
     for (int w = 0; w < workerNum; ++w) send_len[w] = r.send_index_h[w + 1] - r.send_index_h[w];
     DRONE_REQUIRE(send_len[workerId] == 0, "the routing tables name this worker as its own peer");
-    rc = tr->exchange(tr->ctx, workerId, workerNum, send_len.data(), r.send_index_h, send_id, send_val,
-                      recv_len.data(), recv_id, recv_val, r.capacity, comm->s);
+    const void *send[2] = {send_id, send_val};
+    void *recv[2] = {recv_id, recv_val};
+    const size_t elem[2] = {sizeof(int), sizeof(T)};
+    rc = tr->exchange(tr->ctx, workerId, workerNum, send_len.data(), r.send_index_h, 2, send, recv, elem,
+                      recv_len.data(), r.capacity, comm->s);
     if (rc != DRONE_OK) return rc;
 
     int *unknown = r.unknown;
@@ -273,9 +276,12 @@ struct drone_loopback {
     int waiting = 0;
     uint64_t generation = 0;
     bool broken = false;
+    static constexpr int kMaxArrays = 4;
     struct Slot {
-        const int *send_len = nullptr, *send_index = nullptr, *send_id = nullptr;
-        const void *send_val = nullptr;
+        const int *send_len = nullptr, *send_index = nullptr;
+        int n_arrays = 0;
+        const void *send[kMaxArrays] = {};
+        size_t elem_bytes[kMaxArrays] = {};
         float *scalar = nullptr;
     };
     std::vector<Slot> slot;
@@ -320,16 +326,21 @@ int loopback_fail(const char *what)
 }
 
 int loopback_exchange(void *ctx, int workerId, int workerNum, const int *send_len, const int *send_index,
-                      const int *send_id, const void *send_val, int *recv_len, int *recv_id, void *recv_val,
-                      int recv_capacity, drone_stream_t stream)
+                      int n_arrays, const void *const *send, void *const *recv, const size_t *elem_bytes,
+                      int *recv_len, int recv_capacity, drone_stream_t stream)
 {
     drone_loopback *grp = static_cast<drone_loopback::Endpoint *>(ctx)->group;
     DRONE_REQUIRE(workerNum == grp->workers && workerId >= 0 && workerId < workerNum, "worker id / count");
+    DRONE_REQUIRE(n_arrays >= 1 && n_arrays <= drone_loopback::kMaxArrays, "n_arrays");
     hipStream_t s = as_stream(stream);
-    grp->slot[workerId].send_len = send_len;
-    grp->slot[workerId].send_index = send_index;
-    grp->slot[workerId].send_id = send_id;
-    grp->slot[workerId].send_val = send_val;
+    drone_loopback::Slot &mine = grp->slot[workerId];
+    mine.send_len = send_len;
+    mine.send_index = send_index;
+    mine.n_arrays = n_arrays;
+    for (int a = 0; a < n_arrays; ++a) {
+        mine.send[a] = send[a];
+        mine.elem_bytes[a] = elem_bytes[a];
+    }
     if (!grp->barrier()) return loopback_fail("exchange");
     int total = 0, rc = DRONE_OK;
     for (int w = 0; w < workerNum && rc == DRONE_OK; ++w) {
@@ -338,6 +349,11 @@ int loopback_exchange(void *ctx, int workerId, int workerNum, const int *send_le
         const drone_loopback::Slot &src = grp->slot[w];
         const int len = src.send_len[workerId];
         if (len <= 0) continue;
+        if (src.n_arrays != n_arrays) {
+            set_error(DRONE_ERR_INVALID, "loopback transport: workers %d and %d are in different exchange steps", workerId, w);
+            rc = DRONE_ERR_INVALID;
+            break;
+        }
         if (total + len > recv_capacity) {
             set_error(DRONE_ERR_INVALID, "loopback transport: worker %d receives more than its %d staging elements",
                       workerId, recv_capacity);
@@ -345,12 +361,16 @@ int loopback_exchange(void *ctx, int workerId, int workerNum, const int *send_le
             break;
         }
         const size_t off = (size_t)src.send_index[workerId];
-        if (hipMemcpyAsync(recv_id + total, src.send_id + off, sizeof(int) * (size_t)len, hipMemcpyDeviceToDevice, s) != hipSuccess ||
-            hipMemcpyAsync(static_cast<char *>(recv_val) + 4 * (size_t)total, static_cast<const char *>(src.send_val) + 4 * off,
-                           4 * (size_t)len, hipMemcpyDeviceToDevice, s) != hipSuccess) {
-            set_error(DRONE_ERR_HIP, "loopback transport: device copy failed");
-            rc = DRONE_ERR_HIP;
-            break;
+        for (int a = 0; a < n_arrays; ++a) {
+            const size_t eb = elem_bytes[a];
+            if (src.elem_bytes[a] != eb ||
+                hipMemcpyAsync(static_cast<char *>(recv[a]) + eb * (size_t)total,
+                               static_cast<const char *>(src.send[a]) + eb * off, eb * (size_t)len,
+                               hipMemcpyDeviceToDevice, s) != hipSuccess) {
+                set_error(DRONE_ERR_HIP, "loopback transport: device copy failed (or element sizes differ)");
+                rc = DRONE_ERR_HIP;
+                break;
+            }
         }
         recv_len[w] = len;
         total += len;

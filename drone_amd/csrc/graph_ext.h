@@ -28,6 +28,17 @@ struct RouteLists {
     int *unknown = nullptr;        // device scalar: received ids that are not on this worker
 };
 
+// Staging of the K-wide row synchronisation (grow-only).
+struct RowSync {
+    int capacity = 0;        // rows
+    size_t row_elems = 0;    // capacity * K the row buffers were sized for
+    int *send_id = nullptr, *recv_id = nullptr;
+    float *send_rows = nullptr, *recv_rows = nullptr;
+    uint8_t *send_u8 = nullptr, *recv_u8 = nullptr;
+    float *send_maxmin = nullptr, *recv_maxmin = nullptr;
+};
+void row_sync_release(RowSync *rs);
+
 struct GraphExt {
     int n = 0;
     int edges = 0;
@@ -43,6 +54,7 @@ struct GraphExt {
     double *inv64 = nullptr;
     double *rank64 = nullptr;
     RouteLists routes;
+    RowSync row_sync;
     // SSSP: edge lengths in in-edge order
     int *in_eid = nullptr;    // device [edges]: position in the out-edge CSR (g->dst / g->edgeLen) of each in-edge
     float *in_len = nullptr;  // device [edges]: g->edgeLen gathered through in_eid at every SSSP_PEVal

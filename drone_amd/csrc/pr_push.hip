@@ -199,6 +199,7 @@ void drone::graph_ext_release(GraphExt *x)
     if (x->inv64) (void)hipFree(x->inv64);
     if (x->rank64) (void)hipFree(x->rank64);
     routes_release(&x->routes);
+    row_sync_release(&x->row_sync);
     if (x->in_eid) (void)hipFree(x->in_eid);
     if (x->in_len) (void)hipFree(x->in_len);
     *x = GraphExt{};

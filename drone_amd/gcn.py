@@ -197,3 +197,33 @@ class GcnModel:
         if self.h:
             lib().drone_gcn_destroy(self.h)
             self.h = None
+
+
+def compress_rows_u8(x):
+    """drone_compress_rows_u8 (cuda_compress.cu:92-105 compressFloat2Uint8): x float32 [rows, K] on the device ->
+    (uint8 [rows, K], float32 [rows, 2] = {max, min})."""
+    import torch
+    rows, K = x.shape
+    q = torch.empty((rows, K), dtype=torch.uint8, device=x.device)
+    mm = torch.empty((rows, 2), dtype=torch.float32, device=x.device)
+    check(lib().drone_compress_rows_u8(x.data_ptr(), x.stride(0) if rows else K, rows, K, q.data_ptr(), mm.data_ptr(), None))
+    return q, mm
+
+
+def decompress_rows_u8(q, maxmin):
+    """drone_decompress_rows_u8 (cuda_compress.cu:76-90 de_convert)."""
+    import torch
+    rows, K = q.shape
+    out = torch.empty((rows, K), dtype=torch.float32, device=q.device)
+    check(lib().drone_decompress_rows_u8(q.data_ptr(), maxmin.data_ptr(), rows, K, out.data_ptr(), K, None))
+    return out
+
+
+def graphsum_sync_rows(g, data, workerId, workerNum, comm, compress=False):
+    """drone_graphsum_sync_rows_f32 (cuda_communicate.cu:374-448 GraphSum_sync_value_nccl): data float32
+    [local, K] on the device, updated in place.  Returns (mirror2master_recv, master2mirror_recv)."""
+    import ctypes as C
+    a, b = C.c_int(0), C.c_int(0)
+    check(lib().drone_graphsum_sync_rows_f32(g, data.data_ptr(), data.stride(0), data.shape[1], int(workerId),
+                                             int(workerNum), C.byref(comm), int(bool(compress)), C.byref(a), C.byref(b)))
+    return a.value, b.value

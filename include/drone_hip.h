@@ -334,14 +334,15 @@ int drone_pr_worker_destroy(drone_pr_worker *w);
  * ncclSend / ncclRecv followed by a stream synchronise.  All workers call in the same order. */
 typedef struct drone_transport {
     void *ctx;
-    /* Worker `workerId` sends, to every other worker w, send_len[w] ids and 4-byte values starting at element
-     * send_index[w] of send_id / send_val (device), and receives into recv_id / recv_val (device, room for
-     * recv_capacity elements) what the others send to it, packed in ascending source-worker order;
-     * recv_len[w] (host [workerNum]) receives the count that came from w (0 for itself).  send_len and
-     * send_index are host arrays.  Returns 0 or a negative drone_status. */
+    /* Moves n_arrays parallel device arrays in one step.  Worker `workerId` sends, to every other worker w,
+     * elements [send_index[w], send_index[w] + send_len[w]) of each send[a] (element size elem_bytes[a]), and
+     * receives into each recv[a] (room for recv_capacity elements) what the others send to it, packed in
+     * ascending source-worker order; recv_len[w] (host [workerNum]) receives the count that came from w (0 for
+     * itself).  send_len, send_index, send, recv and elem_bytes are host arrays.  Returns 0 or a negative
+     * drone_status. */
     int (*exchange)(void *ctx, int workerId, int workerNum, const int *send_len, const int *send_index,
-                    const int *send_id, const void *send_val, int *recv_len, int *recv_id, void *recv_val,
-                    int recv_capacity, drone_stream_t stream);
+                    int n_arrays, const void *const *send, void *const *recv, const size_t *elem_bytes,
+                    int *recv_len, int recv_capacity, drone_stream_t stream);
     /* *device_scalar becomes the sum over all workers' values, added in worker order on every worker. */
     int (*allreduce_sum_f32)(void *ctx, int workerId, int workerNum, float *device_scalar, drone_stream_t stream);
 } drone_transport;
@@ -384,6 +385,23 @@ typedef struct SSSPValues {
 Response SSSP_PEVal(Graph *g, SSSPValues *values, int startId, int workerId, int workerNum, Comm *comm);
 Response SSSP_IncEVal(Graph *g, SSSPValues *values, int workerId, int workerNum, Comm *comm);
 void drone_sssp_values_destroy(Graph *g, SSSPValues *values);
+
+/* cuda_gcn/src/cuda/cuda_compress.cu:8-105 (findMinMax + convert, de_convert): one (max, min) pair and K bytes per
+ * row, q = uint8((x - min) / (max - min) * 255 + 0.5), x' = min + (max - min) * q / 255.  in / out rows have
+ * leading dimension ld, the byte rows are dense (K), maxmin is [rows][2] = {max, min}.  A constant row, which
+ * divides by zero in the reference, is encoded as zeros and decodes to its value. */
+int drone_compress_rows_u8(const float *in, int ld, int rows, int K, uint8_t *out, float *maxmin,
+                           drone_stream_t stream);
+int drone_decompress_rows_u8(const uint8_t *in, const float *maxmin, int rows, int K, float *out, int ld,
+                             drone_stream_t stream);
+/* cuda_gcn/src/cuda/cuda_communicate.cu:374-448 (GraphSum_sync_value_nccl, full-batch branch): data is [local][ld]
+ * with K used columns; the rows of all mirrors are added into their masters' rows (source workers in ascending
+ * order), then every replicated master's row is assigned to its mirrors.  compress != 0 sends rows as uint8 with
+ * the (max, min) pairs (the reference's `compress` switch, cuda_communicate.cu:317-351).  The two outputs receive
+ * the row counts that arrived in each phase (the reference's mirror2master / master2mirror counters); they may be
+ * NULL.  Blocks like the entry points above; the routing tables are those of addMasterRoute / addMirrorRoute. */
+int drone_graphsum_sync_rows_f32(Graph *g, float *data, int ld, int K, int workerId, int workerNum, Comm *comm,
+                                 int compress, int *mirror2master_recv, int *master2mirror_recv);
 
 #ifdef __cplusplus
 }

@@ -446,3 +446,55 @@ def gcn_forward_backward(rp, ci, v, rpT, ciT, vT, X, W1, W2, truth, keep1=None, 
         _p(ciT), _p(vT), _p(X), _p(W1), _p(W2), _p(truth), _p(keep1), C.c_float(p_drop), _p(Z), _p(H1),
         _p(dW1), _p(dW2), _p(dT1))
     return dict(loss=loss, Z=Z, H1=H1, dW1=dW1, dW2=dW2, dT1=dT1)
+
+
+# ---- GraphSum replica sync of K-wide rows and the uint8 row compression ----------------------------------------
+def compress_rows_u8(x):
+    """cuda_gcn/src/cuda/cuda_compress.cu:8-74: per-row max / min, q = uint8((x - min) / (max - min) * 255 + 0.5)
+    with the quotient and product in float and the + 0.5 in double.  A constant row (0 / 0 in the reference) is
+    encoded as zeros.  Returns (q uint8 [rows, K], maxmin float32 [rows, 2] = {max, min})."""
+    x = np.ascontiguousarray(x, np.float32)
+    mx, mn = x.max(axis=1), x.min(axis=1)
+    rng = (mx - mn).astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        t = ((x - mn[:, None]).astype(np.float32) / rng[:, None]).astype(np.float32) * np.float32(255)
+    q = np.where(rng[:, None] == 0, 0.0, t.astype(np.float64) + 0.5)
+    return np.floor(q).astype(np.uint8), np.stack([mx, mn], axis=1).astype(np.float32)
+
+
+def decompress_rows_u8(q, maxmin):
+    """cuda_compress.cu:76-90: x' = min + (max - min) * q / 255 in float."""
+    mx, mn = maxmin[:, 0:1].astype(np.float32), maxmin[:, 1:2].astype(np.float32)
+    return (mn + ((mx - mn).astype(np.float32) * q.astype(np.float32)).astype(np.float32) / np.float32(255)).astype(np.float32)
+
+
+def graphsum_sync_rows(parts, data, compress=False):
+    """cuda_gcn/src/cuda/cuda_communicate.cu:374-448 over all workers at once: every mirror's row is added into its
+    master's row (apply_sum, source workers in ascending order, rows of one worker in ascending local id), then
+    every replicated master's row is assigned to its mirrors (apply_assign).  data[w] is worker w's [local, K]
+    float32 array, updated in place.  With compress the rows pass through compress_rows_u8 / decompress_rows_u8
+    on the way (cuda_compress.cu:108-138).  Returns (mirror2master_recv[w], master2mirror_recv[w])."""
+    W = len(parts)
+    wire = (lambda r: decompress_rows_u8(*compress_rows_u8(r[None, :]))[0]) if compress else (lambda r: r.copy())
+    recv0, recv1 = [0] * W, [0] * W
+    box = [[[] for _ in range(W)] for _ in range(W)]
+    for w, p in enumerate(parts):
+        for v in np.nonzero(p.m2w != -1)[0]:
+            box[w][p.m2w[v]].append((p.l2g[v], wire(data[w][v])))
+    for dst, p in enumerate(parts):
+        for src in range(W):
+            for gid, row in box[src][dst]:
+                l = p.g2l[gid]
+                data[dst][l] = (data[dst][l] + row).astype(np.float32)
+                recv0[dst] += 1
+    box = [[[] for _ in range(W)] for _ in range(W)]
+    for w, p in enumerate(parts):
+        for v in sorted(p.master_workers):
+            for dst in p.master_workers[v]:
+                box[w][dst].append((p.l2g[v], wire(data[w][v])))
+    for dst, p in enumerate(parts):
+        for src in range(W):
+            for gid, row in box[src][dst]:
+                data[dst][p.g2l[gid]] = row
+                recv1[dst] += 1
+    return recv0, recv1

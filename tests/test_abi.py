@@ -132,8 +132,8 @@ def test_gcn_entry_points_validate_arguments_on_the_host():
 
 class _Transport(C.Structure):
     """drone_transport of include/drone_hip.h"""
-    _EX = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
-                      C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p)
+    _EX = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p,
+                      C.c_void_p, C.c_void_p, C.c_int, C.c_void_p)
     _AR = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p)
     _fields_ = [("ctx", C.c_void_p), ("exchange", _EX), ("allreduce_sum_f32", _AR)]
 
@@ -153,9 +153,13 @@ def test_loopback_transport_times_out_instead_of_hanging():
     send_len = (C.c_int * 2)(0, 0)
     send_index = (C.c_int * 3)(0, 0, 0)
     recv_len = (C.c_int * 2)(7, 7)
-    rc = tr.exchange(tr.ctx, 0, 2, send_len, send_index, None, None, recv_len, None, None, 1, None)
+    send = (C.c_void_p * 2)(None, None)
+    recv = (C.c_void_p * 2)(None, None)
+    elem = (C.c_size_t * 2)(4, 4)
+    args = (send_len, send_index, 2, send, recv, elem, recv_len, 1, None)
+    rc = tr.exchange(tr.ctx, 0, 2, *args)
     assert rc == -1 and b"did not arrive" in L.drone_last_error_string()
-    rc = tr.exchange(tr.ctx, 0, 2, send_len, send_index, None, None, recv_len, None, None, 1, None)
-    assert rc == -1                                                  # broken for good
-    assert tr.exchange(tr.ctx, 0, 3, send_len, send_index, None, None, recv_len, None, None, 1, None) == -1
+    assert tr.exchange(tr.ctx, 0, 2, *args) == -1                    # broken for good
+    assert tr.exchange(tr.ctx, 0, 3, *args) == -1                    # wrong worker count
+    assert tr.exchange(tr.ctx, 0, 2, send_len, send_index, 9, send, recv, elem, recv_len, 1, None) == -1
     assert L.drone_loopback_destroy(grp) == 0
