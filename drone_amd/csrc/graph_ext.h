@@ -57,7 +57,8 @@ struct GraphExt {
     RowSync row_sync;
     // SSSP: edge lengths in in-edge order
     int *in_eid = nullptr;    // device [edges]: position in the out-edge CSR (g->dst / g->edgeLen) of each in-edge
-    float *in_len = nullptr;  // device [edges]: g->edgeLen gathered through in_eid at every SSSP_PEVal
+    float *in_len = nullptr;  // device [edges]: g->edgeLen in in-edge order, refreshed at every SSSP_PEVal
+    bool in_len_ones = false; // in_len is known to hold 1.0 everywhere
 };
 
 void graph_ext_release(GraphExt *x);  // frees everything but the struct itself

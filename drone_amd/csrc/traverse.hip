@@ -5,7 +5,7 @@
 // and atomicMin's its label / distance into the targets) until nothing changes, with a device synchronise per
 // round.
 //
-// Here a round is one sweep of the merge-path aggregation over the IN-edge CSR with min as the combining
+// Here a dense round is one sweep of the merge-path aggregation over the IN-edge CSR with min as the combining
 // operator: value[v] <- min(value[v], min over in-edges u->v of f(value[u])), f = identity for labels and
 // + edge length for distances.  No atomics, hub rows are spread over tiles, and the sweep updates in place,
 // so a change can travel several hops in one sweep.  Both iterations descend monotonically to the same least
@@ -13,6 +13,12 @@
 // reference's three classes (> 0 lowered by propagation in this call, 0 activated by a message or initial,
 // -1 untouched), which is all the exchange and countActive (common.cu:17-31) look at.  The round number
 // stored in g->active by the reference depends on its thread schedule and is not reproduced.
+//
+// A full sweep costs E however few vertices changed, so rounds with a sparse frontier run the other way round:
+// one wavefront per frontier vertex walks its out-edges and lowers the targets with atomicMin (what the
+// reference does for every round), appending each newly lowered vertex once to the next frontier.  The direction
+// is chosen per round from the number of out-edges of the frontier: push below E / 16, pull above.  Both
+// directions move towards the same fixed point, so switching between them does not change the result.
 #include <chrono>
 #include <rocprim/device/device_radix_sort.hpp>
 
@@ -118,9 +124,29 @@ __global__ __launch_bounds__(kSpmvBlock) void count_active_kernel(int n, const i
     if (threadIdx.x == 0) block_part[blockIdx.x] = total;
 }
 
+__global__ void clear_counters_kernel(unsigned long long *c)
+{
+    if (threadIdx.x < 2 && blockIdx.x == 0) c[threadIdx.x] = 0ull;
+}
+
 __global__ void iota_kernel(int *out, int n)
 {
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) out[i] = i;
+}
+
+__global__ __launch_bounds__(kSpmvBlock) void count_not_one_kernel(int n, const float *__restrict__ len,
+                                                                   double *__restrict__ block_part)
+{
+    __shared__ double s_red[kSpmvBlock / kWave];
+    double cnt = 0.0;
+    for (int i = blockIdx.x * kSpmvBlock + threadIdx.x; i < n; i += gridDim.x * kSpmvBlock) cnt += len[i] != 1.0f;
+    const double total = block_sum_256(cnt, s_red);
+    if (threadIdx.x == 0) block_part[blockIdx.x] = total;
+}
+
+__global__ void fill_f32_kernel(float *out, float v, int n)
+{
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) out[i] = v;
 }
 
 __global__ void gather_len_kernel(int n, const int *__restrict__ eid, const float *__restrict__ len,
@@ -134,6 +160,9 @@ struct TraverseExt {
     double *stat = nullptr;        // device scalar
     double *block_part = nullptr;  // device [blocks]
     int blocks = 0;
+    int *frontier[2] = {nullptr, nullptr};  // device [n] each: vertex lists of the push rounds
+    unsigned long long *counters = nullptr; // device [2]: {vertices << 32 | out-edges, largest out-degree} of the list being built
+    unsigned long long *host = nullptr;     // pinned [2]: landing place of the statistic and of the counters
 };
 
 double seconds_since(std::chrono::steady_clock::time_point t0)
@@ -154,6 +183,10 @@ TraverseExt *traverse_ext_create(int n)
     if (t->blocks > 4096) t->blocks = 4096;
     DRONE_HIP_OR_DIE(hipMalloc(&t->stat, sizeof(double)));
     DRONE_HIP_OR_DIE(hipMalloc(&t->block_part, sizeof(double) * (size_t)t->blocks));
+    DRONE_HIP_OR_DIE(hipMalloc(&t->frontier[0], sizeof(int) * (size_t)(n > 0 ? n : 1)));
+    DRONE_HIP_OR_DIE(hipMalloc(&t->frontier[1], sizeof(int) * (size_t)(n > 0 ? n : 1)));
+    DRONE_HIP_OR_DIE(hipMalloc(&t->counters, sizeof(unsigned long long) * 2));
+    DRONE_HIP_OR_DIE(hipHostMalloc(&t->host, sizeof(unsigned long long) * 2));
     return t;
 }
 
@@ -163,15 +196,19 @@ void traverse_ext_destroy(void *ext)
     if (!t) return;
     (void)hipFree(t->stat);
     (void)hipFree(t->block_part);
+    (void)hipFree(t->frontier[0]);
+    (void)hipFree(t->frontier[1]);
+    (void)hipFree(t->counters);
+    (void)hipHostFree(t->host);
     delete t;
 }
 
 double read_stat(TraverseExt *t, hipStream_t s)
 {
-    double v = 0.0;
-    DRONE_HIP_OR_DIE(hipMemcpyAsync(&v, t->stat, sizeof(double), hipMemcpyDeviceToHost, s));
+    double *landing = reinterpret_cast<double *>(t->host);  // pinned: the copy does not go through a staging buffer
+    DRONE_HIP_OR_DIE(hipMemcpyAsync(landing, t->stat, sizeof(double), hipMemcpyDeviceToHost, s));
     DRONE_HIP_OR_DIE(hipStreamSynchronize(s));
-    return v;
+    return *landing;
 }
 
 double reduce_parts(TraverseExt *t, hipStream_t s)
@@ -186,19 +223,194 @@ int count_active(Graph *g, TraverseExt *t, hipStream_t s)
     return (int)reduce_parts(t, s);
 }
 
-// Sweeps until a sweep lowers nothing.  Returns the number of sweeps.
-template <typename V, typename Epi>
-int sweep_to_fixed_point(Graph *g, TraverseExt *t, Epi epi, hipStream_t s)
+// ---- push direction ---------------------------------------------------------------------------------------
+struct CcPush {
+    int *cc;
+    __device__ __forceinline__ int load(int v) const { return __atomic_load_n(cc + v, __ATOMIC_RELAXED); }
+    __device__ __forceinline__ int relax(int val, int) const { return val; }
+    __device__ __forceinline__ bool lower(int t, int nv) const { return atomicMin(cc + t, nv) > nv; }  // cc.cu:35-36
+};
+
+struct SsspPush {
+    float *dist;
+    const float *__restrict__ len;  // out-edge order (g->edgeLen)
+    __device__ __forceinline__ float load(int v) const
+    {
+        return __uint_as_float(__atomic_load_n(reinterpret_cast<unsigned int *>(dist + v), __ATOMIC_RELAXED));
+    }
+    __device__ __forceinline__ float relax(float val, int e) const { return val + len[e]; }
+    __device__ __forceinline__ bool lower(int t, float nv) const
+    {
+        // sssp.cu:11-21 fatomicMin: compare-and-swap until the stored value is not larger; returns the value seen
+        // first.  The target counts as updated past the tolerance (sssp.cu:64).
+        unsigned int *addr = reinterpret_cast<unsigned int *>(dist + t);
+        const float first = __uint_as_float(__atomic_load_n(addr, __ATOMIC_RELAXED));
+        float old = first;
+        while (old > nv) {
+            const unsigned int seen = atomicCAS(addr, __float_as_uint(old), __float_as_uint(nv));
+            if (seen == __float_as_uint(old)) break;
+            old = __uint_as_float(seen);
+        }
+        return first > nv + kRelaxEps;
+    }
+};
+
+// Appends v for every lane with `take` to the list and adds the lanes' out-degrees to the counters.  The vertex
+// count and the edge sum share one 64-bit word (both stay below 2^31), so a wavefront issues one atomic that returns
+// its position in the list; the largest degree is only written when it grows.  Must be reached by all lanes.
+__device__ __forceinline__ void frontier_append(bool take, int v, int degree, int *__restrict__ list,
+                                                unsigned long long *__restrict__ counters)
+{
+    const unsigned long long mask = __ballot(take);
+    if (mask == 0) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    unsigned long long sum = take ? (unsigned long long)degree : 0ull;
+    int mx = take ? degree : 0;
+#pragma unroll
+    for (int m = kWave / 2; m > 0; m >>= 1) {
+        sum += __shfl_xor(sum, m, kWave);
+        const int o = __shfl_xor(mx, m, kWave);
+        mx = o > mx ? o : mx;
+    }
+    const int leader = __ffsll((long long)mask) - 1;
+    unsigned long long base = 0;
+    if (lane == leader) {
+        base = atomicAdd(counters, ((unsigned long long)__popcll(mask) << 32) + sum) >> 32;
+        if ((unsigned long long)mx > __atomic_load_n(counters + 1, __ATOMIC_RELAXED))
+            atomicMax(counters + 1, (unsigned long long)mx);
+    }
+    base = __shfl(base, leader, kWave);
+    if (take) list[base + __popcll(mask & ((1ull << lane) - 1ull))] = v;
+}
+
+// list <- vertices whose active flag equals `value`.  A work-group first compacts its matches in LDS, then the
+// first wavefront appends them, so the shared counter sees one atomic per 256 vertices that hold a match.
+__global__ __launch_bounds__(kSpmvBlock) void collect_frontier_kernel(int n, const int *__restrict__ active, int value,
+                                                                      const int *__restrict__ index, int *__restrict__ list,
+                                                                      unsigned long long *__restrict__ counters)
+{
+    __shared__ int s_v[kSpmvBlock];
+    __shared__ int s_count;
+    for (int base = blockIdx.x * kSpmvBlock; base < n; base += gridDim.x * kSpmvBlock) {
+        if (threadIdx.x == 0) s_count = 0;
+        __syncthreads();
+        const int v = base + threadIdx.x;
+        if (v < n && active[v] == value) s_v[atomicAdd(&s_count, 1)] = v;
+        __syncthreads();
+        const int cnt = s_count;
+        if (threadIdx.x < kWave) {
+            for (int k = 0; k < cnt; k += kWave) {  // cnt is the same for the whole wavefront
+                const bool take = k + (int)threadIdx.x < cnt;
+                const int u = take ? s_v[k + threadIdx.x] : 0;
+                frontier_append(take, u, take ? index[u + 1] - index[u] : 0, list, counters);
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// One wavefront per (frontier vertex, chunk of kPushChunk out-edges); blockIdx.y is the chunk, so a hub's edges are
+// spread over many wavefronts and a wavefront whose chunk lies past the vertex's degree leaves at once.  A target
+// lowered in this round is appended to `next` once: its active flag is swapped to this round's mark, and only the
+// lane that changes it appends.
+constexpr int kPushChunk = 1024;
+
+template <typename Push>
+__global__ __launch_bounds__(256) void push_round_kernel(int count, const int *__restrict__ frontier,
+                                                         const int *__restrict__ index, const int *__restrict__ dst,
+                                                         Push push, int *__restrict__ active, int mark,
+                                                         int *__restrict__ next, unsigned long long *__restrict__ counters)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int waves = gridDim.x * (blockDim.x / kWave);
+    for (int i = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave; i < count; i += waves) {
+        const int v = frontier[i];
+        const int e0 = index[v] + blockIdx.y * kPushChunk;
+        int e1 = index[v + 1];
+        if (e0 >= e1) continue;  // the same for all lanes
+        if (e1 > e0 + kPushChunk) e1 = e0 + kPushChunk;
+        const auto val = push.load(v);
+        for (int eb = e0; eb < e1; eb += kWave) {
+            const int e = eb + lane;
+            bool take = false;
+            int t = 0;
+            if (e < e1) {
+                t = dst[e];
+                take = push.lower(t, push.relax(val, e)) && atomicExch(active + t, mark) != mark;
+            }
+            frontier_append(take, t, take ? index[t + 1] - index[t] : 0, next, counters);
+        }
+    }
+}
+
+struct Frontier {
+    unsigned long long count = 0, edges = 0, max_degree = 0;
+};
+
+Frontier read_counters(TraverseExt *t, hipStream_t s)
+{
+    DRONE_HIP_OR_DIE(hipMemcpyAsync(t->host, t->counters, sizeof(unsigned long long) * 2, hipMemcpyDeviceToHost, s));
+    DRONE_HIP_OR_DIE(hipStreamSynchronize(s));
+    return Frontier{t->host[0] >> 32, t->host[0] & 0xFFFFFFFFull, t->host[1]};
+}
+
+Frontier collect_frontier(Graph *g, TraverseExt *t, int value, int *list, hipStream_t s)
+{
+    const int n = getLocalVertexSize(g);
+    clear_counters_kernel<<<1, 64, 0, s>>>(t->counters);
+    collect_frontier_kernel<<<t->blocks, kSpmvBlock, 0, s>>>(n, g->active, value, g->index, list, t->counters);
+    return read_counters(t, s);
+}
+
+// Runs rounds until nothing changes.  `fr` describes the vertices that still have to propagate and sit in
+// t->frontier[0] (count 0 with all_active = true means "every vertex": the first round is a sweep).  Returns the
+// number of rounds, or -1 when the bound of n + 1 rounds is exceeded (a cycle of negative length).
+template <typename V, typename Epi, typename Push>
+int run_to_fixed_point(Graph *g, TraverseExt *t, Epi epi, Push push, Frontier fr, bool all_active, hipStream_t s)
 {
     GraphExt *x = static_cast<GraphExt *>(g->ext);
-    int sweeps = 0;
+    const int n = x->n;
+    const unsigned long long push_limit = (unsigned long long)x->edges / 16;
+    int cur = 0, rounds = 0, mark = 0;
+    bool pull = all_active || fr.edges > push_limit;
+    if (!pull && fr.count == 0) return 0;
     for (;;) {
-        epi.mark = sweeps + 1;  // cc.cu:37 `active[v] = step + 1`
-        spmv_merge_launch<V, int, kIpt, Epi>(x->mt, x->ms, x->in_index, x->in_src, epi, t->stat, s);
-        DRONE_HIP_OR_DIE(hipGetLastError());
-        ++sweeps;
-        if (read_stat(t, s) == 0.0) return sweeps;
+        if (rounds > n + 1) return -1;
+        ++rounds;
+        ++mark;  // cc.cu:37 `active[v] = step + 1`: positive, and different in every round
+        if (pull) {
+            epi.mark = mark;
+            spmv_merge_launch<V, int, kIpt, Epi>(x->mt, x->ms, x->in_index, x->in_src, epi, t->stat, s);
+            DRONE_HIP_OR_DIE(hipGetLastError());
+            const double changed = read_stat(t, s);
+            if (changed == 0.0) return rounds;
+            if (changed <= (double)n / 16) {  // few enough to be worth listing
+                cur = 0;
+                fr = collect_frontier(g, t, mark, t->frontier[0], s);
+                pull = fr.edges > push_limit;
+            }
+        } else {
+            clear_counters_kernel<<<1, 64, 0, s>>>(t->counters);
+            const int waves_per_block = 256 / kWave;
+            const int gx = (int)(ceil_div((int64_t)fr.count, waves_per_block) < 16384 ? ceil_div((int64_t)fr.count, waves_per_block) : 16384);
+            const int gy = (int)ceil_div((int64_t)(fr.max_degree > 0 ? fr.max_degree : 1), kPushChunk);
+            push_round_kernel<Push><<<dim3(gx, gy), 256, 0, s>>>((int)fr.count, t->frontier[cur], g->index, g->dst, push, g->active,
+                                                         mark, t->frontier[cur ^ 1], t->counters);
+            DRONE_HIP_OR_DIE(hipGetLastError());
+            fr = read_counters(t, s);
+            cur ^= 1;
+            if (fr.count == 0) return rounds;
+            pull = fr.edges > push_limit;  // a sweep covers whatever the listed vertices still had to propagate
+        }
     }
+}
+
+void report_rounds(int rounds, const char *who)
+{
+    if (rounds >= 0) return;
+    set_error(DRONE_ERR_INVALID, "%s: no fixed point after n + 1 rounds (a cycle of negative length); the values are "
+              "not converged", who);
+    printf("%s: no fixed point after n + 1 rounds (a cycle of negative length)\n", who);
 }
 
 // Position in the out-edge CSR of every in-edge: a stable sort of the edge numbers by target keeps the
@@ -229,6 +441,23 @@ void ensure_in_edge_ids(Graph *g, hipStream_t s)
     (void)hipFree(tmp);
     (void)hipFree(keys_out);
     (void)hipFree(iota);
+}
+
+// Brings x->in_len (edge lengths in in-edge order) up to date with g->edgeLen.  build_graph leaves every length at
+// 1.0 and few callers change that, so a streaming check for "all ones" comes first: it avoids the random gather
+// through in_eid, which costs more than a whole sweep.
+void refresh_in_edge_lengths(Graph *g, TraverseExt *t, hipStream_t s)
+{
+    GraphExt *x = static_cast<GraphExt *>(g->ext);
+    if (x->edges == 0) return;
+    count_not_one_kernel<<<t->blocks, kSpmvBlock, 0, s>>>(x->edges, g->edgeLen, t->block_part);
+    if (reduce_parts(t, s) == 0.0) {
+        if (!x->in_len_ones) fill_f32_kernel<<<1024, 256, 0, s>>>(x->in_len, 1.0f, x->edges);
+        x->in_len_ones = true;
+        return;
+    }
+    gather_len_kernel<<<1024, 256, 0, s>>>(x->edges, x->in_eid, g->edgeLen, x->in_len);
+    x->in_len_ones = false;
 }
 
 template <typename Policy, typename T>
@@ -275,7 +504,8 @@ extern "C" Response CC_PEVal(Graph *g, CCValues *values, int workerId, int worke
     }
     TraverseExt *t = static_cast<TraverseExt *>(values->ext);
     cc_init_kernel<<<t->blocks, kSpmvBlock, 0, s>>>(n, g->active, values->ccValue, g->updateByMessage);
-    sweep_to_fixed_point<MinI32>(g, t, CcEpi{values->ccValue, g->active, 1}, s);
+    if (n > 0)  // every vertex starts active (cc.cu:16): the first round is a sweep
+        run_to_fixed_point<MinI32>(g, t, CcEpi{values->ccValue, g->active, 1}, CcPush{values->ccValue}, Frontier{}, true, s);
     res.LocalVertexSize = n;
     res.CalTime = (float)seconds_since(t0);
     const auto t1 = std::chrono::steady_clock::now();
@@ -300,8 +530,10 @@ extern "C" Response CC_IncEVal(Graph *g, CCValues *values, int workerId, int wor
     TraverseExt *t = static_cast<TraverseExt *>(values->ext);
     const int n = getLocalVertexSize(g);
     process_messages_kernel<<<t->blocks, kSpmvBlock, 0, s>>>(n, g->active, g->updateByMessage, t->block_part);
-    if (reduce_parts(t, s) > 0.0)  // cc.cu:425: no message, no round
-        sweep_to_fixed_point<MinI32>(g, t, CcEpi{values->ccValue, g->active, 1}, s);
+    if (reduce_parts(t, s) > 0.0) {  // cc.cu:425: no message, no round
+        const Frontier fr = collect_frontier(g, t, 0, t->frontier[0], s);  // the vertices a message activated
+        run_to_fixed_point<MinI32>(g, t, CcEpi{values->ccValue, g->active, 1}, CcPush{values->ccValue}, fr, false, s);
+    }
     res.LocalVertexSize = n;
     res.CalTime = (float)seconds_since(t0);
     const auto t1 = std::chrono::steady_clock::now();
@@ -344,15 +576,18 @@ extern "C" Response SSSP_PEVal(Graph *g, SSSPValues *values, int startId, int wo
     ensure_flags(g);
     ensure_in_edge_ids(g, s);
     GraphExt *x = static_cast<GraphExt *>(g->ext);
-    if (x->edges > 0) gather_len_kernel<<<1024, 256, 0, s>>>(x->edges, x->in_eid, g->edgeLen, x->in_len);
     if (!values->ext) {  // sssp.cu:408-411
         DRONE_HIP_OR_DIE(hipMalloc(&values->distance, sizeof(float) * (size_t)(n > 0 ? n : 1)));
         values->ext = traverse_ext_create(n);
     }
     TraverseExt *t = static_cast<TraverseExt *>(values->ext);
+    refresh_in_edge_lengths(g, t, s);
     sssp_init_kernel<<<t->blocks, kSpmvBlock, 0, s>>>(n, start, g->active, values->distance, g->updateByMessage);
-    if (start >= 0)  // sssp.cu:30: only the worker that holds the start vertex has anything to do
-        sweep_to_fixed_point<MinF32>(g, t, SsspEpi{values->distance, x->in_len, g->active, 1}, s);
+    if (start >= 0) {  // sssp.cu:30: only the worker that holds the start vertex has anything to do
+        const Frontier fr = collect_frontier(g, t, 0, t->frontier[0], s);  // the start vertex
+        report_rounds(run_to_fixed_point<MinF32>(g, t, SsspEpi{values->distance, x->in_len, g->active, 1},
+                                                 SsspPush{values->distance, g->edgeLen}, fr, false, s), "SSSP_PEVal");
+    }
     res.LocalVertexSize = n;
     res.CalTime = (float)seconds_since(t0);
     const auto t1 = std::chrono::steady_clock::now();
@@ -378,8 +613,11 @@ extern "C" Response SSSP_IncEVal(Graph *g, SSSPValues *values, int workerId, int
     GraphExt *x = static_cast<GraphExt *>(g->ext);
     const int n = getLocalVertexSize(g);
     process_messages_kernel<<<t->blocks, kSpmvBlock, 0, s>>>(n, g->active, g->updateByMessage, t->block_part);
-    if (reduce_parts(t, s) > 0.0)
-        sweep_to_fixed_point<MinF32>(g, t, SsspEpi{values->distance, x->in_len, g->active, 1}, s);
+    if (reduce_parts(t, s) > 0.0) {
+        const Frontier fr = collect_frontier(g, t, 0, t->frontier[0], s);
+        report_rounds(run_to_fixed_point<MinF32>(g, t, SsspEpi{values->distance, x->in_len, g->active, 1},
+                                                 SsspPush{values->distance, g->edgeLen}, fr, false, s), "SSSP_IncEVal");
+    }
     res.LocalVertexSize = n;
     res.CalTime = (float)seconds_since(t0);
     const auto t1 = std::chrono::steady_clock::now();

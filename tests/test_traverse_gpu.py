@@ -158,3 +158,68 @@ def test_group_matches_oracle_group(oracle, kind, W, scale, seed):
         for w in ws:
             w.close()
         lb.close()
+
+
+def test_sssp_negative_cycle_terminates_with_an_error(oracle):
+    """The reference would relax for ever; here the rounds are bounded by n + 1 and the error channel says why."""
+    from drone_amd import _lib
+    from drone_amd.traverse import SSSPWorkerCUDA
+    u, v = np.array([0, 1, 2], np.int32), np.array([1, 2, 0], np.int32)
+    w = SSSPWorkerCUDA(3, u, v, startId=0)
+    try:
+        w.set_edge_len(np.array([1.0, -3.0, 1.0], np.float32))
+        w.peval()
+        assert _lib.lib().drone_last_error() != 0
+        assert b"negative" in _lib.lib().drone_last_error_string()
+    finally:
+        w.close()
+
+
+def test_long_chain_uses_sparse_rounds(oracle):
+    """20,000 hops: one push round per hop, not one sweep over all edges per hop; same result as the oracle."""
+    import time
+    from drone_amd.traverse import CCWorkerCUDA, SSSPWorkerCUDA
+    n = 20000
+    u, v = _chain(n)
+    perm = np.random.default_rng(3).permutation(n).astype(np.int32)     # hop order unrelated to vertex order
+    u, v = perm[u], perm[v]
+    nl, g2l, l2g, index, dst = oracle.build_graph(n, u, v)
+    st = oracle.SSSPState(index, dst)
+    st.peval(int(g2l[u[0]]))
+    w = SSSPWorkerCUDA(n, u, v, startId=int(u[0]))
+    try:
+        t0 = time.time()
+        w.peval()
+        assert time.time() - t0 < 20.0
+        np.testing.assert_array_equal(w.read(), st.val)
+        assert float(st.val.max()) == n - 1
+    finally:
+        w.close()
+    sc = oracle.CCState(index, dst)
+    sc.peval()
+    w = CCWorkerCUDA(n, u, v)
+    try:
+        res = w.peval()
+        np.testing.assert_array_equal(w.read(), sc.val)
+        assert res.VisitedSize == sc.visited()
+    finally:
+        w.close()
+
+
+def test_graph_without_edges(oracle):
+    from drone_amd.traverse import CCWorkerCUDA, SSSPWorkerCUDA
+    e = np.zeros(0, np.int32)
+    w = CCWorkerCUDA(5, e, e)
+    try:
+        res = w.peval()
+        assert res.LocalVertexSize == 0 and res.VisitedSize == 0
+        res = w.incEval()
+        assert res.VisitedSize == 0
+    finally:
+        w.close()
+    w = SSSPWorkerCUDA(5, e, e, startId=2)
+    try:
+        res = w.peval()
+        assert res.LocalVertexSize == 0 and res.VisitedSize == 0
+    finally:
+        w.close()
