@@ -11,7 +11,9 @@
 // lanes read adjacent addresses in whichever dimension is contiguous in memory.
 // A long reduction with a small output (the weight gradient: K = vertex count) is split over grid.z; the
 // partial tiles go to a scratch buffer and are summed in split order by a second kernel.
+#include <map>
 #include <mutex>
+#include <utility>
 
 #include "common.h"
 
@@ -162,28 +164,31 @@ __global__ void sgemm_reduce_kernel(int M, int N, int splits, const float *__res
     }
 }
 
-// Grow-only scratch for split-K partials, one per device.  Calls that use it must not overlap on a device.
+// Grow-only scratch for split-K partials, one per (device, stream): calls on one stream are ordered, so they can
+// share a buffer; calls on different streams may overlap and get their own.
+struct SplitScratch {
+    float *ptr = nullptr;
+    size_t bytes = 0;
+};
 std::mutex g_ws_mutex;
-float *g_ws[16] = {};
-size_t g_ws_bytes[16] = {};
+std::map<std::pair<int, hipStream_t>, SplitScratch> g_ws;
 
-int workspace(size_t bytes, float **out)
+int workspace(size_t bytes, hipStream_t s, float **out)
 {
     int dev = 0;
     DRONE_HIP_TRY(hipGetDevice(&dev));
-    DRONE_REQUIRE(dev >= 0 && dev < 16, "device ordinal");
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    if (g_ws_bytes[dev] < bytes) {
-        if (g_ws[dev]) {
-            DRONE_HIP_TRY(hipDeviceSynchronize());
-            (void)hipFree(g_ws[dev]);
-            g_ws[dev] = nullptr;
-            g_ws_bytes[dev] = 0;
+    SplitScratch &w = g_ws[std::make_pair(dev, s)];
+    if (w.bytes < bytes) {
+        if (w.ptr) {
+            DRONE_HIP_TRY(hipStreamSynchronize(s));  // earlier calls on this stream may still read it
+            (void)hipFree(w.ptr);
+            w = SplitScratch{};
         }
-        DRONE_HIP_TRY(hipMalloc(&g_ws[dev], bytes));
-        g_ws_bytes[dev] = bytes;
+        DRONE_HIP_TRY(hipMalloc(&w.ptr, bytes));
+        w.bytes = bytes;
     }
-    *out = g_ws[dev];
+    *out = w.ptr;
     return DRONE_OK;
 }
 
@@ -227,7 +232,7 @@ extern "C" int drone_sgemm_rm_f32(int transA, int transB, int M, int N, int K, f
     splits = (int)ceil_div(K > 0 ? K : 1, k_chunk);
     float *partial = nullptr;
     if (splits > 1) {
-        int rc = workspace(sizeof(float) * (size_t)splits * M * N, &partial);
+        int rc = workspace(sizeof(float) * (size_t)splits * M * N, s, &partial);
         if (rc != DRONE_OK) return rc;
     }
     dim3 grid((unsigned)ceil_div(N, bn), (unsigned)ceil_div(M, BM), (unsigned)splits);

@@ -1,7 +1,9 @@
 // Element-wise and per-row kernels on the measured GCN step, semantics as in cuda_gcn/src/cuda/cuda_kernel.cu:
 // ReLU (:384-399), dropout with an explicit keep mask (:403-420), soft-max cross-entropy (:295-379 with the
 // host logic of cuda_module.cu:406-483), Adam (:450-460), plus SGD, accuracy (cuda_gcn.cu:226-246) and arg-max.
+#include <map>
 #include <mutex>
+#include <utility>
 
 #include "common.h"
 
@@ -204,10 +206,10 @@ __global__ void fill_f32_kernel(float *__restrict__ x, int64_t n, float value)
         x[i] = value;
 }
 
-// scratch for the cross-entropy block partials, one per device (grow-only)
+// scratch for the cross-entropy block partials (2048 blocks), one per (device, stream): calls on one stream are
+// ordered and share it, calls on different streams may overlap
 std::mutex g_mutex;
-void *g_ce_ws[16] = {};
-int g_ce_blocks[16] = {};
+std::map<std::pair<int, hipStream_t>, void *> g_ce_ws;
 
 }  // namespace
 }  // namespace drone
@@ -264,21 +266,18 @@ extern "C" int drone_cross_entropy_f32(int n, int classes, const float *logits, 
     DRONE_REQUIRE(grad == nullptr || ldg >= classes, "ldg < classes");
     int dev = 0;
     DRONE_HIP_TRY(hipGetDevice(&dev));
-    DRONE_REQUIRE(dev >= 0 && dev < 16, "device ordinal");
     int blocks = (int)ceil_div(n, kThreads / kWave);
     if (blocks > 2048) blocks = 2048;
+    hipStream_t s = as_stream(stream);
     void *ws = nullptr;
     {
         std::lock_guard<std::mutex> lock(g_mutex);
-        if (g_ce_blocks[dev] < 2048) {
-            DRONE_HIP_TRY(hipMalloc(&g_ce_ws[dev], 2048 * (sizeof(double) + sizeof(int))));
-            g_ce_blocks[dev] = 2048;
-        }
-        ws = g_ce_ws[dev];
+        void *&slot = g_ce_ws[std::make_pair(dev, s)];
+        if (!slot) DRONE_HIP_TRY(hipMalloc(&slot, 2048 * (sizeof(double) + sizeof(int))));
+        ws = slot;
     }
     double *bl = static_cast<double *>(ws);
     int *bc = reinterpret_cast<int *>(bl + 2048);
-    hipStream_t s = as_stream(stream);
     cross_entropy_kernel<<<blocks, kThreads, 0, s>>>(n, classes, logits, ld, truth, grad, ldg, grad_scale, bl, bc);
     cross_entropy_finish_kernel<<<1, kThreads, 0, s>>>(blocks, bl, bc, loss_out, count_out);
     DRONE_HIP_TRY(hipGetLastError());

@@ -159,8 +159,8 @@ int drone_pr_run_graph_f64(Graph *g, PRValues *values, double alpha, int iters, 
 /* All dense operands are row-major fp32 with explicit leading dimensions (in elements); CSR arrays are
  * int32 offsets / int32 columns / fp32 values, base 0 - the descriptors of cuda_module.cu:166-194.
  * Calls are asynchronous on `stream`.  Apart from plan creation, the transpose (a set-up step) and
- * grow-only scratch kept per device by drone_sgemm_rm_f32 (split reductions) and
- * drone_cross_entropy_f32, nothing allocates; calls that use that scratch must not overlap on a device. */
+ * grow-only scratch kept per (device, stream) by drone_sgemm_rm_f32 (split reductions) and
+ * drone_cross_entropy_f32, nothing allocates; calls on different streams may overlap. */
 
 /* cuda_gcn/src/cuda/cuda_kernel.cu:145-155 (launched at cuda_module.cu:163):
  * v[e(u->col)] = 1 / sqrtf(1.0 * out_deg[u] * in_deg[col]) for every entry of row u. */

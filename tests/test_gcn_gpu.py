@@ -288,3 +288,22 @@ def test_sgd_adam(T, oracle):
         gcn.adam_step(wd, dev(T, g), md, vd, True, 5e-4, 0.01, 0.9, 0.999, 1e-8, t)
         oracle.adam_step(wa, g, m, v, True, 5e-4, 0.01, 0.9, 0.999, 1e-8, t)
         np.testing.assert_allclose(wd.cpu().numpy(), wa, rtol=1e-5, atol=1e-6)
+
+
+def test_split_reductions_on_two_streams_do_not_share_scratch(T):
+    """Two weight-gradient GEMMs and two cross-entropies issued back to back on different streams (so they may run
+    at the same time) give the results of the serial calls."""
+    from drone_amd import gcn
+    rng = np.random.default_rng(11)
+    X1, G1 = dev(T, rng.normal(size=(60000, 64)).astype(np.float32)), dev(T, rng.normal(size=(60000, 41)).astype(np.float32))
+    X2, G2 = dev(T, rng.normal(size=(50000, 48)).astype(np.float32)), dev(T, rng.normal(size=(50000, 33)).astype(np.float32))
+    want1, want2 = gcn.sgemm(1, 0, X1, G1).clone(), gcn.sgemm(1, 0, X2, G2).clone()
+    T.cuda.synchronize()
+    s1, s2 = T.cuda.Stream(), T.cuda.Stream()
+    for _ in range(5):
+        o1 = T.empty_like(want1)
+        o2 = T.empty_like(want2)
+        gcn.sgemm(1, 0, X1, G1, out=o1, stream=s1.cuda_stream)
+        gcn.sgemm(1, 0, X2, G2, out=o2, stream=s2.cuda_stream)
+        T.cuda.synchronize()
+        assert T.equal(o1, want1) and T.equal(o2, want2)
