@@ -108,6 +108,17 @@ __global__ __launch_bounds__(kWave * kRowsPerBlock) void rows_apply_kernel(
     }
 }
 
+// cuda_module.cu:50-62
+__global__ __launch_bounds__(kWave * kRowsPerBlock) void clear_mirror_rows_kernel(int rows, int K, float *__restrict__ grad,
+                                                                                  int ld, const int *__restrict__ m2w)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    for (int r = blockIdx.x * kRowsPerBlock + threadIdx.x / kWave; r < rows; r += gridDim.x * kRowsPerBlock) {
+        if (m2w[r] == -1) continue;
+        for (int k = lane; k < K; k += kWave) grad[(size_t)r * ld + k] = 0.0f;
+    }
+}
+
 int row_grid(int rows) { return rows > 0 ? (int)(ceil_div(rows, kRowsPerBlock) < 8192 ? ceil_div(rows, kRowsPerBlock) : 8192) : 1; }
 
 int ensure_row_staging(RowSync *rs, int capacity, int K)
@@ -141,6 +152,18 @@ void drone::row_sync_release(RowSync *rs)
     (void)hipFree(rs->send_maxmin);
     (void)hipFree(rs->recv_maxmin);
     *rs = RowSync{};
+}
+
+extern "C" int drone_clear_mirror_rows_f32(float *grad, int ld, int rows, int K, const int *mirror2worker,
+                                           drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(rows >= 0 && K >= 1 && ld >= K, "rows / K / ld");
+    DRONE_REQUIRE(rows == 0 || (grad && mirror2worker), "null operand");
+    if (rows == 0) return DRONE_OK;
+    clear_mirror_rows_kernel<<<row_grid(rows), kWave * kRowsPerBlock, 0, as_stream(stream)>>>(rows, K, grad, ld, mirror2worker);
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
 }
 
 extern "C" int drone_compress_rows_u8(const float *in, int ld, int rows, int K, uint8_t *out, float *maxmin,

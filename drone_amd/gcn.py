@@ -227,3 +227,10 @@ def graphsum_sync_rows(g, data, workerId, workerNum, comm, compress=False):
     check(lib().drone_graphsum_sync_rows_f32(g, data.data_ptr(), data.stride(0), data.shape[1], int(workerId),
                                              int(workerNum), C.byref(comm), int(bool(compress)), C.byref(a), C.byref(b)))
     return a.value, b.value
+
+
+def clear_mirror_rows(grad, mirror2worker, stream=0):
+    """drone_clear_mirror_rows_f32 (cuda_module.cu:50-62): zero the rows of mirrors in place."""
+    rows, K = grad.shape
+    check(lib().drone_clear_mirror_rows_f32(grad.data_ptr(), grad.stride(0), rows, K, mirror2worker.data_ptr(), stream))
+    return grad

@@ -94,9 +94,13 @@ class Matmul : public Module {
     Variable *a, *b, *c;
     int m, n, p;
     drone_stream_t s;
+    const int *mirror2worker;  // device [m] or null: rows of mirrors are left out of the weight gradient
 public:
-    Matmul(Variable *a_, Variable *b_, Variable *c_, int m_, int n_, int p_, std::string name, drone_stream_t stream)
-        : a(a_), b(b_), c(c_), m(m_), n(n_), p(p_), s(stream) { ModuleName = std::move(name); }
+    // cuda_module.cu:10-11: the reference passes graph->Mirror2Worker; with one subgraph there are no mirrors and
+    // null skips the clearing kernel.
+    Matmul(Variable *a_, Variable *b_, Variable *c_, int m_, int n_, int p_, std::string name, drone_stream_t stream,
+           const int *mirror2worker_ = nullptr)
+        : a(a_), b(b_), c(c_), m(m_), n(n_), p(p_), s(stream), mirror2worker(mirror2worker_) { ModuleName = std::move(name); }
     void forward(bool) override
     {
         DRONE_GCN_CHECK(drone_sgemm_rm_f32(0, 0, m, p, n, 1.0f, a->data, a->ld, b->data, b->ld, 0.0f, c->data, c->ld, s));
@@ -105,8 +109,11 @@ public:
     {
         if (a->requires_grad)
             DRONE_GCN_CHECK(drone_sgemm_rm_f32(0, 1, m, n, p, 1.0f, c->grad, c->ld, b->data, b->ld, 0.0f, a->grad, a->ld, s));
-        if (b->requires_grad)
+        if (b->requires_grad) {
+            if (mirror2worker)  // cuda_module.cu:89-90: zero the mirrors' rows of c->grad in place, after a->grad used them
+                DRONE_GCN_CHECK(drone_clear_mirror_rows_f32(c->grad, c->ld, m, p, mirror2worker, s));
             DRONE_GCN_CHECK(drone_sgemm_rm_f32(1, 0, n, p, m, 1.0f, a->data, a->ld, c->grad, c->ld, 0.0f, b->grad, b->ld, s));
+        }
     }
 };
 

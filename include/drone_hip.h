@@ -196,6 +196,10 @@ int64_t drone_spmm_bytes(int n_rows, int64_t nnz, int K);
 int drone_sgemm_rm_f32(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,
                        const float *B, int ldb, float beta, float *C, int ldc, drone_stream_t stream);
 int64_t drone_sgemm_flops(int M, int N, int K);
+/* cuda_module.cu:50-62 clear_mirror_grad, launched between the two GEMMs of CUDAMatmul::backward (:89-90): rows
+ * of grad [rows][ld] (K used columns) whose vertex is a mirror (mirror2worker[row] != -1) are set to zero, so a
+ * replicated vertex contributes to the weight gradient on its master's worker only. */
+int drone_clear_mirror_rows_f32(float *grad, int ld, int rows, int K, const int *mirror2worker, drone_stream_t stream);
 /* cuda_kernel.cu:384-392 / :394-399: in-place ReLU with a byte mask recorded when training. */
 int drone_relu_forward_f32(float *x, uint8_t *mask, int64_t n, int training, drone_stream_t stream);
 int drone_relu_backward_f32(float *grad, const uint8_t *mask, int64_t n, drone_stream_t stream);

@@ -98,3 +98,17 @@ def test_graphsum_sync_one_worker_is_a_no_op(oracle):
     assert gcn.graphsum_sync_rows(w.g, x, 0, 1, w.comm) == (0, 0)
     assert torch.equal(x, keep)
     lib_close(w)
+
+
+def test_clear_mirror_rows(oracle):
+    """cuda_module.cu:50-62: rows of mirrors become zero, everything else (including padding columns) is untouched."""
+    import torch
+    from drone_amd import gcn
+    rng = np.random.default_rng(5)
+    rows, K, ld = 1000, 41, 44
+    full = torch.from_numpy(rng.standard_normal((rows, ld)).astype(np.float32)).cuda()
+    m2w = np.where(rng.random(rows) < 0.3, rng.integers(0, 4, rows), -1).astype(np.int32)
+    want = full.cpu().numpy().copy()
+    want[m2w != -1, :K] = 0.0
+    gcn.clear_mirror_rows(full[:, :K], torch.from_numpy(m2w).cuda())
+    np.testing.assert_array_equal(full.cpu().numpy(), want)
