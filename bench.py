@@ -146,7 +146,8 @@ def bench_gcn_step(steps, warmup, cpu_baseline=False):
         B = torch.rand((N, ld), device="cuda") * 2 - 1
         out = torch.empty((N, ld), device="cuda")
         ms = time_call(lambda: gcn.spmm(plan, rp, ci, val, B[:, :K], K=K, out=out[:, :K]), reps=5)
-        kernels.append(spmm_report(f"spmm (rows + band pieces) K={K} ld={ld}", N, nnz, K, ms))
+        kernels.append(spmm_report(f"spmm (rows + band pieces + dense core) K={K} ld={ld}", N, nnz, K, ms))
+    plan_info = plan.info()
     spmm_ms = 2 * sum(k["ms"] for k in kernels[:2])
     spmm_bytes = 2 * sum(k["algorithmic_bytes"] for k in kernels[:2])
     gemms = []
@@ -180,7 +181,7 @@ def bench_gcn_step(steps, warmup, cpu_baseline=False):
             "workload": f"2-layer GCN training step (configs[3]): N={N}, nnz={nnz}, 602->128->41, ReLU, dropout 0.5, "
                         "softmax cross-entropy, SGD lr 0.01, fp32",
             "step_ms": step_ms, "steps": steps, "setup_ms_one_off": setup_s * 1e3, "spmm_kernels": kernels,
-            "spmm_ms_per_step": spmm_ms,
+            "spmm_ms_per_step": spmm_ms, "spmm_plan": plan_info,
             "spmm_frac_of_hbm_peak": spmm_bytes / (spmm_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "gemms": gemms}
 
 
@@ -209,7 +210,7 @@ def bench_gcn_layer():
     ms_gemm = time_call(lambda: gcn.sgemm(0, 0, H, W, out=T1), reps=10)
     plan.close()
     return {"workload": f"GCN layer forward (configs[2]): R-MAT scale 20 undirected + self-loops, N={N}, nnz={nnz}, K=128",
-            "layer_ms": ms, "spmm": spmm_report("spmm (rows + band pieces) K=128", N, nnz, K, ms_spmm),
+            "layer_ms": ms, "spmm": spmm_report("spmm (rows + band pieces + dense core) K=128", N, nnz, K, ms_spmm),
             "gemm_ms": ms_gemm, "gemm_tflops": 2.0 * N * K * K / (ms_gemm * 1e-3) / 1e12}
 
 

@@ -156,6 +156,7 @@ SIGNATURES = {
     "drone_timer_destroy": (_I, [_P]),
     "drone_device_synchronize": (_I, []),
     "drone_pr_worker_attach_loopback": (_I, [_P, _P]),
+    "drone_spmm_plan_info": (_I, [_P, C.POINTER(_I64), C.POINTER(_I64), C.POINTER(_I64), C.POINTER(_I), C.POINTER(_I)]),
     "drone_clear_mirror_rows_f32": (_I, [_P, _I, _I, _I, _P, _P]),
     "drone_compress_rows_u8": (_I, [_P, _I, _I, _I, _P, _P, _P]),
     "drone_decompress_rows_u8": (_I, [_P, _P, _I, _I, _P, _I, _P]),

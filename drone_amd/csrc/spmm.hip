@@ -18,8 +18,21 @@
 // list in that order.  Work-groups are dispatched in list order, so at any moment the resident wavefronts
 // work inside one band whose feature rows stay in L2.  A piece writes its partial row to plan-owned scratch;
 // a second kernel adds each long row's partials in (band, position) order - no atomics, bitwise repeatable.
+//
+// Dense core: power-law graphs with a high edge factor have a core (most frequent columns x longest rows) that is
+// tens of percent dense.  There a gather per non-zero moves K*4 bytes through L2 for every entry, while a dense
+// tile product moves each feature row once per 128 rows and runs on the matrix cores.  The plan therefore ranks
+// the long rows by length, takes row groups [0,4096), [4096,8192), [8192,16384), ... in that order and, per
+// group, the leading 2048-column chunks (in column-frequency order) whose density is at least kDenseThreshold;
+// the entries of these rectangles are kept out of the band pieces, stored as dense fp32 blocks, and multiplied
+// by drone_sgemm_rm_f32 against the frequency-ordered copy of B's leading rows.  The threshold is near the ratio
+// of the two kernels' measured costs (about 3 ps per dense cell, 24 ps per gathered entry at K = 128, both
+// proportional to K) and was then set by measurement on the 232,965-vertex / 229 M-entry graph (ms for K = 128 /
+// K = 41: no dense part 6.33 / 3.57; threshold 0.30: 5.39 / 3.02; 0.16: 4.94 / 2.72; 0.12: 4.90 / 2.70; 0.06:
+// 5.17 / 2.81).  Graphs without such a core (every chunk below the threshold) get no dense part.
 #include <algorithm>
 #include <cstring>
+#include <numeric>
 #include <vector>
 
 #include <rocprim/device/device_radix_sort.hpp>
@@ -42,6 +55,22 @@ struct drone_spmm_plan {
     unsigned *perm = nullptr;                                                // device [long_nnz]: sorted position -> entry
     float *partial = nullptr;                                                // device [num_pieces x max_k]
     int num_bands = 0, band_cols = 0;
+    // dense core (see the file comment); rows and columns below are in rank order
+    struct Rect { int row0, rows, width; size_t a_off; };
+    int num_rects = 0;
+    Rect rects[8] = {};
+    int dense_rows = 0, dense_wmax = 0;
+    int64_t dense_nnz = 0;
+    int *dense_row = nullptr;        // device [dense_rows]: matrix row of each ranked row
+    int *dense_seg_begin = nullptr;  // device [dense_rows]: the row's dense entries in ci2 / val2
+    int *dense_seg_end = nullptr;
+    int *dense_row_width = nullptr;  // device [dense_rows]: width of the rectangle the row belongs to
+    int64_t *dense_row_off = nullptr;// device [dense_rows]: first cell of the row in dense_a
+    int *col_rank = nullptr;         // device [n_cols]: column -> frequency rank
+    unsigned *col_order = nullptr;   // device [n_cols]: frequency rank -> column
+    float *dense_a = nullptr;        // device: the rectangles, row-major, one after the other
+    float *dense_b = nullptr;        // device [dense_wmax x ldk]: B's rows in rank order
+    float *dense_t = nullptr;        // device [dense_rows x ldk]: products in rank order
 };
 
 namespace drone {
@@ -52,6 +81,15 @@ constexpr int kChunk = 2048;            // most non-zeros in one piece
 constexpr int kHotBands = 16;           // bands kept apart; colder columns share one more band
 constexpr size_t kBandBytes = 2u << 20; // feature rows of one band (half of an XCD's L2)
 constexpr int kRowsPerBlock = 4;
+constexpr int kDenseChunk = 2048;       // column granularity of the dense rectangles
+constexpr int kDenseMaxCols = 32768;    // widest rectangle
+constexpr int kDenseFirstRows = 4096;   // rows of the first group; every further group doubles the covered rows
+constexpr int kDenseGroups = 5;         // up to 65,536 rows
+constexpr float kDenseThreshold = 0.12f;  // for feature widths that fill 128-column tiles
+constexpr double kGatherMsPerEntry = 0.19e-9;  // band-piece kernel: 24 ps per entry at K = 128
+constexpr double kDenseMsPerCell = 0.025e-9;   // dense product: 3.2 ps per cell at K = 128
+constexpr double kDenseMinGainMs = 0.25;
+static_assert(kDenseMaxCols / kDenseChunk <= 32, "the density histogram keeps at most 32 chunks per wavefront");
 
 template <int VEC> struct VecT;
 template <> struct VecT<4> { using type = float4; };
@@ -249,21 +287,96 @@ __global__ void assign_bands_kernel(const unsigned *__restrict__ order, int n_co
     }
 }
 
-// One wavefront per long row: key = band(col) * num_long + long index, value = entry index, written to the
-// row's compact range [long_offset[i], long_offset[i+1]).
+// col_rank[order[rank]] = rank
+__global__ void col_rank_kernel(const unsigned *__restrict__ order, int n_cols, int *__restrict__ col_rank)
+{
+    for (int r = blockIdx.x * blockDim.x + threadIdx.x; r < n_cols; r += gridDim.x * blockDim.x) col_rank[order[r]] = r;
+}
+
+// hist[group(row) * chunks + col_rank / kDenseChunk] += 1 over the entries of the ranked long rows whose column rank
+// is below chunks * kDenseChunk.  One wavefront per long row, counting in LDS first (the few global counters would
+// serialise 10^8 atomics); group_of_long[i] < 0 = row outside the groups.  chunks <= 32.
+__global__ __launch_bounds__(256) void dense_histogram_kernel(int num_long, const int *__restrict__ long_row,
+                                                              const int *__restrict__ group_of_long,
+                                                              const int *__restrict__ rp, const int *__restrict__ ci,
+                                                              const int *__restrict__ col_rank, int chunks,
+                                                              unsigned *__restrict__ hist)
+{
+    __shared__ unsigned s_cnt[256 / kWave][32];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    for (int i = (blockIdx.x * blockDim.x + threadIdx.x) / kWave; i < num_long; i += gridDim.x * blockDim.x / kWave) {
+        const int g = group_of_long[i];
+        if (g < 0) continue;  // the same for the whole wavefront
+        if (lane < 32) s_cnt[wave][lane] = 0;
+        __builtin_amdgcn_wave_barrier();
+        const int r = long_row[i], e0 = rp[r], e1 = rp[r + 1];
+        for (int e = e0 + lane; e < e1; e += kWave) {
+            const int c = col_rank[ci[e]] / kDenseChunk;
+            if (c < chunks) atomicAdd(&s_cnt[wave][c], 1u);
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (lane < chunks && s_cnt[wave][lane]) atomicAdd(&hist[g * chunks + lane], s_cnt[wave][lane]);
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+// One wavefront per long row: key = band * num_long + long index, value = entry index, written to the row's
+// compact range [long_offset[i], long_offset[i+1]).  band = band(col), or num_bands (past every real band) for
+// the entries that live in a dense rectangle: column rank below the row's dense width.
 __global__ __launch_bounds__(256) void band_keys_kernel(int num_long, const int *__restrict__ long_row,
                                                         const int *__restrict__ long_offset, const int *__restrict__ rp,
                                                         const int *__restrict__ ci,
-                                                        const unsigned char *__restrict__ band_of_col,
+                                                        const unsigned char *__restrict__ band_of_col, int num_bands,
+                                                        const int *__restrict__ dense_width_of_long,
+                                                        const int *__restrict__ col_rank,
                                                         unsigned *__restrict__ keys, unsigned *__restrict__ idx)
 {
     const int lane = threadIdx.x & (kWave - 1);
     for (int i = (blockIdx.x * blockDim.x + threadIdx.x) / kWave; i < num_long; i += gridDim.x * blockDim.x / kWave) {
         const int r = long_row[i], e0 = rp[r], len = rp[r + 1] - e0, o = long_offset[i];
+        const int w = dense_width_of_long[i];
         for (int k = lane; k < len; k += kWave) {
-            keys[o + k] = (unsigned)band_of_col[ci[e0 + k]] * (unsigned)num_long + (unsigned)i;
+            const int c = ci[e0 + k];
+            const unsigned band = col_rank[c] < w ? (unsigned)num_bands : (unsigned)band_of_col[c];
+            keys[o + k] = band * (unsigned)num_long + (unsigned)i;
             idx[o + k] = (unsigned)(e0 + k);
         }
+    }
+}
+
+// dense_a[row_off[rr] + col_rank[col]] = value over the dense entries of ranked row rr (one wavefront per row).
+// Cells without an entry keep the zero they were created with.
+__global__ __launch_bounds__(256) void dense_fill_kernel(int dense_rows, const int *__restrict__ seg_begin,
+                                                         const int *__restrict__ seg_end, const int64_t *__restrict__ row_off,
+                                                         const int *__restrict__ ci2, const float *__restrict__ val2,
+                                                         const int *__restrict__ col_rank, float *__restrict__ a)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    for (int rr = (blockIdx.x * blockDim.x + threadIdx.x) / kWave; rr < dense_rows; rr += gridDim.x * blockDim.x / kWave)
+        for (int p = seg_begin[rr] + lane; p < seg_end[rr]; p += kWave) a[row_off[rr] + col_rank[ci2[p]]] = val2[p];
+}
+
+// dense_b[r, 0..K) = B[order[r], 0..K) for the leading ranks (one wavefront per row)
+__global__ __launch_bounds__(256) void dense_gather_b_kernel(int rows, const unsigned *__restrict__ order,
+                                                             const float *__restrict__ B, int ldb, int K,
+                                                             float *__restrict__ out, int ldo)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    for (int r = (blockIdx.x * blockDim.x + threadIdx.x) / kWave; r < rows; r += gridDim.x * blockDim.x / kWave) {
+        const float *src = B + (size_t)order[r] * ldb;
+        for (int k = lane; k < ldo; k += kWave) out[(size_t)r * ldo + k] = k < K ? src[k] : 0.0f;
+    }
+}
+
+// C[dense_row[rr], :] += alpha * T[rr, :]
+__global__ __launch_bounds__(256) void dense_add_kernel(int dense_rows, const int *__restrict__ dense_row,
+                                                        const float *__restrict__ t, int ldt, float *__restrict__ C,
+                                                        int ldc, int K, float alpha)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    for (int rr = (blockIdx.x * blockDim.x + threadIdx.x) / kWave; rr < dense_rows; rr += gridDim.x * blockDim.x / kWave) {
+        float *dst = C + (size_t)dense_row[rr] * ldc;
+        for (int k = lane; k < K; k += kWave) dst[k] += alpha * t[(size_t)rr * ldt + k];
     }
 }
 
@@ -290,9 +403,28 @@ void launch_spmm(const drone_spmm_plan *plan, const int *rp, const int *ci, cons
     if (blocks > 0)
         spmm_rows_kernel<G, VEC><<<blocks, kWave * kRowsPerBlock, 0, s>>>(plan->n_rows, rp, ci, v, B, ldb, C, ldc, K,
                                                                          alpha, beta);
-    if (plan->num_pieces > 0)
+    if (plan->num_long > 0)  // also when every entry of the long rows went to the dense part: C = beta * C there
         spmm_combine_kernel<<<plan->num_long, 128, 0, s>>>(plan->num_long, plan->long_row, plan->first_slot,
                                                           plan->partial, plan->max_k, C, ldc, K, alpha, beta);
+}
+
+// The dense rectangles' share of C: B's leading rows in rank order, one product per rectangle, rows added back.
+int launch_dense(const drone_spmm_plan *plan, const float *B, int ldb, float *C, int ldc, int K, float alpha,
+                 hipStream_t s)
+{
+    if (plan->dense_rows == 0) return DRONE_OK;
+    const int ldk = (plan->max_k + 3) / 4 * 4;
+    dense_gather_b_kernel<<<(int)ceil_div(plan->dense_wmax, 4), 256, 0, s>>>(plan->dense_wmax, plan->col_order, B, ldb, K,
+                                                                           plan->dense_b, ldk);
+    for (int i = 0; i < plan->num_rects; ++i) {
+        const drone_spmm_plan::Rect &rc = plan->rects[i];
+        const int status = drone_sgemm_rm_f32(0, 0, rc.rows, K, rc.width, 1.0f, plan->dense_a + rc.a_off, rc.width,
+                                              plan->dense_b, ldk, 0.0f, plan->dense_t + (size_t)rc.row0 * ldk, ldk, s);
+        if (status != DRONE_OK) return status;
+    }
+    dense_add_kernel<<<(int)ceil_div(plan->dense_rows, 4), 256, 0, s>>>(plan->dense_rows, plan->dense_row, plan->dense_t,
+                                                                      ldk, C, ldc, K, alpha);
+    return DRONE_OK;
 }
 
 int build_band_pieces(drone_spmm_plan *p, const std::vector<int> &h_rp, const std::vector<int> &long_row,
@@ -312,11 +444,26 @@ int build_band_pieces(drone_spmm_plan *p, const std::vector<int> &h_rp, const st
     if (num_bands < 1) num_bands = 1;
     p->band_cols = band_cols;
     p->num_bands = num_bands;
-    DRONE_REQUIRE((int64_t)num_bands * num_long < (int64_t)UINT32_MAX, "too many long rows for 32-bit band keys");
+    DRONE_REQUIRE(((int64_t)num_bands + 1) * num_long < (int64_t)UINT32_MAX, "too many long rows for 32-bit band keys");
+
+    // long rows ranked by length (stable, descending): candidates for the dense rectangles
+    std::vector<int> by_rank((size_t)num_long), rank_of_long((size_t)num_long);
+    std::iota(by_rank.begin(), by_rank.end(), 0);
+    std::stable_sort(by_rank.begin(), by_rank.end(), [&](int a, int b) {
+        return long_offset[a + 1] - long_offset[a] > long_offset[b + 1] - long_offset[b];
+    });
+    for (int r = 0; r < num_long; ++r) rank_of_long[by_rank[r]] = r;
+    int group_begin[kDenseGroups + 1];
+    int groups = 0;
+    group_begin[0] = 0;
+    for (int g = 0, end = kDenseFirstRows; g < kDenseGroups && end <= num_long; ++g, end *= 2) group_begin[++groups] = end;
+    const int chunks = std::min(kDenseMaxCols, p->n_cols) / kDenseChunk;
+    std::vector<int> dense_width_of_long((size_t)num_long, 0), group_width((size_t)kDenseGroups, 0);
 
     unsigned *counts = nullptr, *counts_sorted = nullptr, *col_ids = nullptr, *col_order = nullptr;
     unsigned char *band_of_col = nullptr;
-    int *d_long_offset = nullptr;
+    int *d_long_offset = nullptr, *d_group_of_long = nullptr, *d_dense_width = nullptr;
+    unsigned *d_hist = nullptr;
     unsigned *keys = nullptr, *keys_sorted = nullptr, *idx = nullptr, *run_keys = nullptr, *run_counts = nullptr, *run_total = nullptr;
     void *temp = nullptr;
     size_t temp_bytes = 0, need = 0;
@@ -345,7 +492,7 @@ int build_band_pieces(drone_spmm_plan *p, const std::vector<int> &h_rp, const st
         count_columns_kernel<<<2048, 256, 0, s>>>(ci, p->nnz, counts);
         iota_u32_kernel<<<1024, 256, 0, s>>>(col_ids, (int64_t)nc);
         int key_bits = 1;
-        while (key_bits < 32 && (1ull << key_bits) < (unsigned long long)num_bands * (unsigned long long)num_long) ++key_bits;
+        while (key_bits < 32 && (1ull << key_bits) < ((unsigned long long)num_bands + 1) * (unsigned long long)num_long) ++key_bits;
         DRONE_HIP_TRY(rocprim::radix_sort_pairs_desc(nullptr, temp_bytes, counts, counts_sorted, col_ids, col_order, nc, 0, 32, s));
         DRONE_HIP_TRY(rocprim::radix_sort_pairs(nullptr, need, keys, keys_sorted, idx, p->perm, ln, 0, key_bits, s));
         if (need > temp_bytes) temp_bytes = need;
@@ -354,10 +501,50 @@ int build_band_pieces(drone_spmm_plan *p, const std::vector<int> &h_rp, const st
         DRONE_HIP_TRY(hipMalloc(&temp, temp_bytes ? temp_bytes : 1));
         DRONE_HIP_TRY(rocprim::radix_sort_pairs_desc(temp, temp_bytes, counts, counts_sorted, col_ids, col_order, nc, 0, 32, s));
         assign_bands_kernel<<<1024, 256, 0, s>>>(col_order, p->n_cols, band_cols, num_bands, band_of_col);
-        // 2. stable sort of the long rows' entries by (band, row)
+        DRONE_HIP_TRY(hipMalloc(&p->col_rank, sizeof(int) * nc));
+        col_rank_kernel<<<1024, 256, 0, s>>>(col_order, p->n_cols, p->col_rank);
         int kb = (int)ceil_div(num_long, 4);
         if (kb > 65536) kb = 65536;
-        band_keys_kernel<<<kb, 256, 0, s>>>(num_long, p->long_row, d_long_offset, rp, ci, band_of_col, keys, idx);
+        // 1b. dense rectangles: density of every (row group, column chunk) in rank order
+        if (groups > 0 && chunks > 0) {
+            std::vector<int> group_of_long((size_t)num_long, -1);
+            for (int g = 0; g < groups; ++g)
+                for (int r = group_begin[g]; r < group_begin[g + 1]; ++r) group_of_long[by_rank[r]] = g;
+            DRONE_HIP_TRY(hipMalloc(&d_group_of_long, sizeof(int) * (size_t)num_long));
+            DRONE_HIP_TRY(hipMalloc(&d_hist, sizeof(unsigned) * (size_t)groups * chunks));
+            DRONE_HIP_TRY(hipMemcpyAsync(d_group_of_long, group_of_long.data(), sizeof(int) * (size_t)num_long, hipMemcpyHostToDevice, s));
+            DRONE_HIP_TRY(hipMemsetAsync(d_hist, 0, sizeof(unsigned) * (size_t)groups * chunks, s));
+            dense_histogram_kernel<<<kb, 256, 0, s>>>(num_long, p->long_row, d_group_of_long, rp, ci, p->col_rank, chunks, d_hist);
+            std::vector<unsigned> hist((size_t)groups * chunks);
+            DRONE_HIP_TRY(hipMemcpyAsync(hist.data(), d_hist, sizeof(unsigned) * hist.size(), hipMemcpyDeviceToHost, s));
+            DRONE_HIP_TRY(hipStreamSynchronize(s));
+            // The product of a rectangle runs in column tiles of 64 (K <= 64, at about half the rate) or 128, so
+            // narrow feature widths need a denser core before the matrix cores win.
+            const int tile = p->max_k <= 64 ? 64 : (p->max_k + 127) / 128 * 128;
+            const double efficiency = (double)p->max_k / tile * (tile == 64 ? 0.5 : 1.0);
+            const double threshold = kDenseThreshold / efficiency;
+            double dense_entries = 0.0, dense_cells = 0.0;
+            for (int g = 0; g < groups; ++g) {
+                const double cells = (double)(group_begin[g + 1] - group_begin[g]) * kDenseChunk;
+                int w = 0;
+                while (w < chunks && hist[(size_t)g * chunks + w] / cells >= threshold) ++w;
+                if (w == 0) break;  // density falls with rank: later groups are sparser still
+                group_width[g] = w * kDenseChunk;
+                for (int c = 0; c < w; ++c) dense_entries += hist[(size_t)g * chunks + c];
+                dense_cells += cells * w;
+            }
+            // Worth it only when the estimated saving clears the fixed costs (gathering B's leading rows, the
+            // launches, adding the rows back): measured rates, ms per entry and per cell at feature width 1.
+            const double gain_ms = dense_entries * p->max_k * kGatherMsPerEntry - dense_cells * (p->max_k / efficiency) * kDenseMsPerCell;
+            if (gain_ms < kDenseMinGainMs) std::fill(group_width.begin(), group_width.end(), 0);
+            for (int g = 0; g < groups && group_width[g] > 0; ++g)
+                for (int r = group_begin[g]; r < group_begin[g + 1]; ++r) dense_width_of_long[by_rank[r]] = group_width[g];
+        }
+        DRONE_HIP_TRY(hipMalloc(&d_dense_width, sizeof(int) * (size_t)num_long));
+        DRONE_HIP_TRY(hipMemcpyAsync(d_dense_width, dense_width_of_long.data(), sizeof(int) * (size_t)num_long, hipMemcpyHostToDevice, s));
+        // 2. stable sort of the long rows' entries by (band, row); dense entries sort behind every band
+        band_keys_kernel<<<kb, 256, 0, s>>>(num_long, p->long_row, d_long_offset, rp, ci, band_of_col, num_bands,
+                                            d_dense_width, p->col_rank, keys, idx);
         DRONE_HIP_TRY(rocprim::radix_sort_pairs(temp, temp_bytes, keys, keys_sorted, idx, p->perm, ln, 0, key_bits, s));
         gather_sorted_kernel<<<4096, 256, 0, s>>>(long_nnz, p->perm, ci, v, p->ci2, p->val2);
         // 3. runs of equal key = (band, row) pieces
@@ -370,16 +557,28 @@ int build_band_pieces(drone_spmm_plan *p, const std::vector<int> &h_rp, const st
         DRONE_HIP_TRY(hipMemcpy(h_counts.data(), run_counts, sizeof(unsigned) * runs, hipMemcpyDeviceToHost));
         // 4. pieces in band-major order; slots row-major (a row's pieces in band order, then position)
         std::vector<int> pieces_of_row((size_t)num_long, 0);
-        for (unsigned k = 0; k < runs; ++k) pieces_of_row[h_keys[k] % (unsigned)num_long] += (int)ceil_div(h_counts[k], kChunk);
+        const auto is_dense_run = [&](unsigned k) { return h_keys[k] / (unsigned)num_long == (unsigned)num_bands; };
+        for (unsigned k = 0; k < runs; ++k)
+            if (!is_dense_run(k)) pieces_of_row[h_keys[k] % (unsigned)num_long] += (int)ceil_div(h_counts[k], kChunk);
         std::vector<int> first_slot((size_t)num_long + 1, 0);
         for (int i = 0; i < num_long; ++i) first_slot[i + 1] = first_slot[i] + pieces_of_row[i];
         const int num_pieces = first_slot[num_long];
         std::vector<int> cursor(first_slot.begin(), first_slot.end() - 1), pb, pe, ps;
         pb.reserve(num_pieces); pe.reserve(num_pieces); ps.reserve(num_pieces);
+        int dense_rows = 0;
+        while (dense_rows < num_long && dense_width_of_long[by_rank[dense_rows]] > 0) ++dense_rows;
+        std::vector<int> seg_begin((size_t)dense_rows, 0), seg_end((size_t)dense_rows, 0);
         int64_t pos = 0;
         for (unsigned k = 0; k < runs; ++k) {
             const int i = (int)(h_keys[k] % (unsigned)num_long);
             const int64_t end = pos + h_counts[k];
+            if (is_dense_run(k)) {
+                seg_begin[rank_of_long[i]] = (int)pos;
+                seg_end[rank_of_long[i]] = (int)end;
+                p->dense_nnz += h_counts[k];
+                pos = end;
+                continue;
+            }
             for (int64_t b = pos; b < end; b += kChunk) {
                 pb.push_back((int)b);
                 pe.push_back((int)(b + kChunk < end ? b + kChunk : end));
@@ -398,12 +597,54 @@ int build_band_pieces(drone_spmm_plan *p, const std::vector<int> &h_rp, const st
         DRONE_HIP_TRY(hipMemcpy(p->piece_begin, pb.data(), sizeof(int) * (size_t)num_pieces, hipMemcpyHostToDevice));
         DRONE_HIP_TRY(hipMemcpy(p->piece_end, pe.data(), sizeof(int) * (size_t)num_pieces, hipMemcpyHostToDevice));
         DRONE_HIP_TRY(hipMemcpy(p->piece_slot, ps.data(), sizeof(int) * (size_t)num_pieces, hipMemcpyHostToDevice));
+        // 5. the dense rectangles
+        if (dense_rows > 0) {
+            std::vector<int> h_row((size_t)dense_rows), h_width((size_t)dense_rows);
+            std::vector<int64_t> h_off((size_t)dense_rows);
+            size_t cells = 0;
+            for (int g = 0; g < groups && group_width[g] > 0; ++g) {
+                drone_spmm_plan::Rect &rc = p->rects[p->num_rects++];
+                rc.row0 = group_begin[g];
+                rc.rows = group_begin[g + 1] - group_begin[g];
+                rc.width = group_width[g];
+                rc.a_off = cells;
+                for (int r = 0; r < rc.rows; ++r) {
+                    h_row[rc.row0 + r] = long_row[by_rank[rc.row0 + r]];
+                    h_width[rc.row0 + r] = rc.width;
+                    h_off[rc.row0 + r] = (int64_t)(cells + (size_t)r * rc.width);
+                }
+                cells += (size_t)rc.rows * rc.width;
+                if (rc.width > p->dense_wmax) p->dense_wmax = rc.width;
+            }
+            p->dense_rows = dense_rows;
+            const size_t ldk = (size_t)(p->max_k + 3) / 4 * 4;
+            DRONE_HIP_TRY(hipMalloc(&p->dense_row, sizeof(int) * (size_t)dense_rows));
+            DRONE_HIP_TRY(hipMalloc(&p->dense_seg_begin, sizeof(int) * (size_t)dense_rows));
+            DRONE_HIP_TRY(hipMalloc(&p->dense_seg_end, sizeof(int) * (size_t)dense_rows));
+            DRONE_HIP_TRY(hipMalloc(&p->dense_row_width, sizeof(int) * (size_t)dense_rows));
+            DRONE_HIP_TRY(hipMalloc(&p->dense_row_off, sizeof(int64_t) * (size_t)dense_rows));
+            DRONE_HIP_TRY(hipMalloc(&p->dense_a, sizeof(float) * cells));
+            DRONE_HIP_TRY(hipMalloc(&p->dense_b, sizeof(float) * (size_t)p->dense_wmax * ldk));
+            DRONE_HIP_TRY(hipMalloc(&p->dense_t, sizeof(float) * (size_t)dense_rows * ldk));
+            DRONE_HIP_TRY(hipMemcpy(p->dense_row, h_row.data(), sizeof(int) * (size_t)dense_rows, hipMemcpyHostToDevice));
+            DRONE_HIP_TRY(hipMemcpy(p->dense_seg_begin, seg_begin.data(), sizeof(int) * (size_t)dense_rows, hipMemcpyHostToDevice));
+            DRONE_HIP_TRY(hipMemcpy(p->dense_seg_end, seg_end.data(), sizeof(int) * (size_t)dense_rows, hipMemcpyHostToDevice));
+            DRONE_HIP_TRY(hipMemcpy(p->dense_row_width, h_width.data(), sizeof(int) * (size_t)dense_rows, hipMemcpyHostToDevice));
+            DRONE_HIP_TRY(hipMemcpy(p->dense_row_off, h_off.data(), sizeof(int64_t) * (size_t)dense_rows, hipMemcpyHostToDevice));
+            DRONE_HIP_TRY(hipMemsetAsync(p->dense_a, 0, sizeof(float) * cells, s));
+            dense_fill_kernel<<<(int)ceil_div(dense_rows, 4), 256, 0, s>>>(dense_rows, p->dense_seg_begin, p->dense_seg_end,
+                                                                          p->dense_row_off, p->ci2, p->val2, p->col_rank, p->dense_a);
+            p->col_order = col_order;  // kept: the SpMM gathers B's leading rows through it
+            col_order = nullptr;
+            DRONE_HIP_TRY(hipStreamSynchronize(s));
+        }
         DRONE_HIP_TRY(hipGetLastError());
         return DRONE_OK;
     };
     const int rc = body();
     (void)hipFree(counts); (void)hipFree(counts_sorted); (void)hipFree(col_ids); (void)hipFree(col_order);
     (void)hipFree(band_of_col); (void)hipFree(d_long_offset); (void)hipFree(keys); (void)hipFree(keys_sorted);
+    (void)hipFree(d_group_of_long); (void)hipFree(d_dense_width); (void)hipFree(d_hist);
     (void)hipFree(idx); (void)hipFree(run_keys); (void)hipFree(run_counts); (void)hipFree(run_total); (void)hipFree(temp);
     return rc;
 }
@@ -449,6 +690,9 @@ extern "C" int drone_spmm_plan_update_values(drone_spmm_plan *p, const float *v,
     DRONE_REQUIRE(p != nullptr && (p->nnz == 0 || v), "null argument");
     if (p->long_nnz > 0) {
         gather_sorted_kernel<<<4096, 256, 0, as_stream(stream)>>>(p->long_nnz, p->perm, nullptr, v, nullptr, p->val2);
+        if (p->dense_rows > 0)  // cells without an entry stay zero, the others are overwritten
+            dense_fill_kernel<<<(int)ceil_div(p->dense_rows, 4), 256, 0, as_stream(stream)>>>(
+                p->dense_rows, p->dense_seg_begin, p->dense_seg_end, p->dense_row_off, p->ci2, p->val2, p->col_rank, p->dense_a);
         DRONE_HIP_TRY(hipGetLastError());
     }
     return DRONE_OK;
@@ -466,7 +710,32 @@ extern "C" int drone_spmm_plan_destroy(drone_spmm_plan *p)
     (void)hipFree(p->val2);
     (void)hipFree(p->perm);
     (void)hipFree(p->partial);
+    (void)hipFree(p->dense_row);
+    (void)hipFree(p->dense_seg_begin);
+    (void)hipFree(p->dense_seg_end);
+    (void)hipFree(p->dense_row_width);
+    (void)hipFree(p->dense_row_off);
+    (void)hipFree(p->col_rank);
+    (void)hipFree(p->col_order);
+    (void)hipFree(p->dense_a);
+    (void)hipFree(p->dense_b);
+    (void)hipFree(p->dense_t);
     delete p;
+    return DRONE_OK;
+}
+
+extern "C" int drone_spmm_plan_info(const drone_spmm_plan *p, int64_t *long_nnz, int64_t *dense_nnz, int64_t *dense_cells,
+                                    int *dense_rows, int *dense_cols)
+{
+    clear_error();
+    DRONE_REQUIRE(p != nullptr, "plan");
+    int64_t cells = 0;
+    for (int i = 0; i < p->num_rects; ++i) cells += (int64_t)p->rects[i].rows * p->rects[i].width;
+    if (long_nnz) *long_nnz = p->long_nnz;
+    if (dense_nnz) *dense_nnz = p->dense_nnz;
+    if (dense_cells) *dense_cells = cells;
+    if (dense_rows) *dense_rows = p->dense_rows;
+    if (dense_cols) *dense_cols = p->dense_wmax;
     return DRONE_OK;
 }
 
@@ -503,6 +772,8 @@ extern "C" int drone_spmm_csr_f32(const drone_spmm_plan *plan, const int *rp, co
         else if (K <= 32) launch_spmm<32, 1>(plan, rp, ci, v, B, ldb, C, ldc, K, alpha, beta, s);
         else launch_spmm<64, 1>(plan, rp, ci, v, B, ldb, C, ldc, K, alpha, beta, s);
     }
+    const int dense_status = launch_dense(plan, B, ldb, C, ldc, K, alpha, s);
+    if (dense_status != DRONE_OK) return dense_status;
     DRONE_HIP_TRY(hipGetLastError());
     return DRONE_OK;
 }

@@ -49,6 +49,13 @@ class SpmmPlan:
     def update_values(self, val, stream=0):
         check(lib().drone_spmm_plan_update_values(self.h, _ptr(val), stream))
 
+    def info(self):
+        """drone_spmm_plan_info: what went to the band pieces and what to the dense rectangles."""
+        a, b, c = C.c_int64(0), C.c_int64(0), C.c_int64(0)
+        d, e = C.c_int(0), C.c_int(0)
+        check(lib().drone_spmm_plan_info(self.h, C.byref(a), C.byref(b), C.byref(c), C.byref(d), C.byref(e)))
+        return dict(long_nnz=a.value, dense_nnz=b.value, dense_cells=c.value, dense_rows=d.value, dense_cols=e.value)
+
     def close(self):
         if self.h:
             lib().drone_spmm_plan_destroy(self.h)

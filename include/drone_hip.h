@@ -173,7 +173,9 @@ int drone_csr_transpose_f32(int n_rows, int n_cols, int64_t nnz, const int *rp, 
 /* Schedule for the SpMM of one CSR with feature widths up to max_k.  Rows of at most 512 entries run one
  * wavefront each.  Longer rows are cut by column band (columns ranked by frequency; a band's feature rows fill
  * about 2 MB of L2) and the plan keeps a (band,row)-sorted copy of their entries - columns AND values as
- * passed here - plus the scratch for their partial rows.  The rp / ci / v later passed to
+ * passed here - plus the scratch for their partial rows.  Where the longest rows meet the most frequent
+ * columns densely enough (at least 12 % of the cells of a 2048-column chunk), those entries are stored as dense
+ * fp32 rectangles instead and multiplied on the matrix cores (drone_spmm_plan_info reports how much).  The rp / ci / v later passed to
  * drone_spmm_csr_f32 must be the arrays the plan was built from; after changing values in place call
  * drone_spmm_plan_update_values.  Set-up step (the counterpart of cusparseSpMM_bufferSize + the
  * preprocessing cuSPARSE hides, cuda_module.cu:232-243); synchronises `stream`. */
@@ -182,6 +184,10 @@ int drone_spmm_plan_create(drone_spmm_plan **plan, int n_rows, int n_cols, int64
                            const int *ci, const float *v, int max_k, drone_stream_t stream);
 int drone_spmm_plan_update_values(drone_spmm_plan *plan, const float *v, drone_stream_t stream);
 int drone_spmm_plan_destroy(drone_spmm_plan *plan);
+/* What the plan decided: entries in rows longer than 512, entries moved to dense rectangles, the cells of those
+ * rectangles, and the rows / columns (in rank order) the rectangles span.  Any output may be NULL. */
+int drone_spmm_plan_info(const drone_spmm_plan *plan, int64_t *long_nnz, int64_t *dense_nnz, int64_t *dense_cells,
+                         int *dense_rows, int *dense_cols);
 /* cusparseSpMM(NON_TRANSPOSE, NON_TRANSPOSE, alpha, A, B, beta, C, ALG_DEFAULT) at cuda_module.cu:245
  * (forward: A = transposed CSR) and :335 (backward: A = original CSR):
  * C[n_rows x K] = alpha * A * B + beta * C. */

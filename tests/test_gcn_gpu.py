@@ -307,3 +307,49 @@ def test_split_reductions_on_two_streams_do_not_share_scratch(T):
         gcn.sgemm(1, 0, X2, G2, out=o2, stream=s2.cuda_stream)
         T.cuda.synchronize()
         assert T.equal(o1, want1) and T.equal(o2, want2)
+
+
+def test_spmm_dense_core_matches_oracle(T, oracle):
+    """A graph with a dense core (a 6000-vertex near-clique inside a sparse graph): the plan moves the core to dense
+    rectangles; the product and the product after update_values still match the fp64-accumulated oracle, and alpha /
+    beta are honoured on the rows the rectangles touch."""
+    from drone_amd import gcn
+    rng = np.random.default_rng(21)
+    n, core = 12000, 6000
+    perm = rng.permutation(n)
+    dense = rng.random((core, core)) < 0.8
+    r, c = np.nonzero(dense)
+    rs, cs = rng.integers(0, n, 60000), rng.integers(0, n, 60000)
+    key = np.unique(np.concatenate([perm[r].astype(np.int64) * n + perm[c], rs * n + cs]))
+    rows, cols = (key // n).astype(np.int32), (key % n).astype(np.int32)
+    rp = np.zeros(n + 1, np.int32)
+    rp[1:] = np.cumsum(np.bincount(rows, minlength=n))
+    val = rng.uniform(-1, 1, len(cols)).astype(np.float32)
+    d_rp, d_ci, d_val = dev(T, rp), dev(T, cols), dev(T, val)
+    plan = gcn.SpmmPlan(d_rp, d_ci, d_val, n, max_k=128)
+    info = plan.info()
+    assert info["dense_rows"] == 4096 and info["dense_cols"] >= 4096 and info["dense_nnz"] > 10_000_000
+    narrow = gcn.SpmmPlan(d_rp, d_ci, d_val, n, max_k=16)      # too narrow for the matrix cores to pay: no dense part
+    assert narrow.info()["dense_nnz"] == 0
+    narrow.close()
+    for K in (128, 41, 7):
+        B = rng.uniform(-1, 1, (n, K)).astype(np.float32)
+        want = oracle.spmm_f64acc(rp, cols, val, B)
+        got = gcn.spmm(plan, d_rp, d_ci, d_val, dev(T, B)).cpu().numpy()
+        assert np.max(np.abs(got - want)) <= 1e-4 * np.max(np.abs(want))
+        C0 = rng.uniform(-1, 1, (n, K)).astype(np.float32)
+        out = dev(T, C0)
+        gcn.spmm(plan, d_rp, d_ci, d_val, dev(T, B), out=out, alpha=0.5, beta=-2.0)
+        ref = 0.5 * want - 2.0 * C0
+        assert np.max(np.abs(out.cpu().numpy() - ref)) <= 1e-4 * np.max(np.abs(ref))
+    val2 = rng.uniform(-1, 1, len(cols)).astype(np.float32)
+    d_val.copy_(dev(T, val2))
+    plan.update_values(d_val)
+    B = rng.uniform(-1, 1, (n, 128)).astype(np.float32)
+    want = oracle.spmm_f64acc(rp, cols, val2, B)
+    got = gcn.spmm(plan, d_rp, d_ci, d_val, dev(T, B)).cpu().numpy()
+    assert np.max(np.abs(got - want)) <= 1e-4 * np.max(np.abs(want))
+    a = gcn.spmm(plan, d_rp, d_ci, d_val, dev(T, B))
+    b = gcn.spmm(plan, d_rp, d_ci, d_val, dev(T, B))
+    assert T.equal(a, b)                       # repeatable bit for bit
+    plan.close()
