@@ -78,7 +78,7 @@ namespace {
 
 constexpr int kSplitRow = 512;          // rows with more non-zeros are cut into band pieces
 constexpr int kChunk = 2048;            // most non-zeros in one piece
-constexpr int kHotBands = 16;           // bands kept apart; colder columns share one more band
+constexpr int kHotBands = 24;           // bands kept apart; colder columns share one more band
 constexpr size_t kBandBytes = 2u << 20; // feature rows of one band (half of an XCD's L2)
 constexpr int kRowsPerBlock = 4;
 constexpr int kDenseChunk = 2048;       // column granularity of the dense rectangles
