@@ -288,6 +288,57 @@ def bench_traverse(cpu_baseline=True):
     return out
 
 
+def bench_exchange():
+    """Four subgraphs of a random vertex cut of R-MAT scale 20 (ef 16, seed 2) on one GPU, each worker on its own host
+    thread over the in-process loopback transport: PR_PEVal + 5 x PR_IncEVal with the two exchange phases per
+    superstep, and the K-wide row sync of the GCN (K = 128) with and without uint8 compression.  Bytes = ids +
+    values packed once and applied once."""
+    import numpy as np
+    import torch
+    from drone_amd import gcn, rmat
+    from drone_amd.pagerank import Loopback, PRWorkerCUDA, run_workers
+    from drone_amd.partition import random_vertex_cut
+    scale, W, K = 20, 4, 128
+    s, d = rmat.rmat_edges(scale, 16 << scale, seed=2)
+    u, v = rmat.clean_directed_np(s, d)
+    n = 1 << scale
+    outdeg = np.bincount(u, minlength=n).astype(np.int32)
+    parts = random_vertex_cut(u, v, n, W, seed=2)
+    lb = Loopback(W, timeout_ms=120000)
+    ws = [PRWorkerCUDA(n, p["u"], p["v"], outdeg, workerId=i, workerNum=W, routes=p, loopback=lb) for i, p in enumerate(parts)]
+    out = {"workload": f"replica exchange, {W} subgraphs of a random vertex cut of R-MAT scale {scale} on one GPU, loopback "
+                       f"transport; mirrors {sum(len(p['mirror_vertex']) for p in parts)}, local vertices "
+                       f"{[w.n for w in ws]}, edges {[len(p['u']) for p in parts]}"}
+    run_workers([w.peval for w in ws])                         # builds the send lists, staging, tilings
+    steps = []
+    for step in range(6):
+        t = time.perf_counter()
+        res = run_workers([(w.peval if step == 0 else w.incEval) for w in ws])
+        wall = (time.perf_counter() - t) * 1e3
+        sent = sum(r.Mirror2MasterSendSize + r.Master2MirrorSendSize for r in res)
+        steps.append({"superstep": step, "wall_ms": wall, "cal_ms_max": max(r.CalTime for r in res) * 1e3,
+                      "send_ms_max": max(r.SendTime for r in res) * 1e3, "elements_sent": int(sent),
+                      "exchange_GBps": sent * 8 * 2 / (max(r.SendTime for r in res) + 1e-12) / 1e9})
+    out["pagerank_supersteps"] = steps
+    # GCN row sync on the same graphs
+    dev = [torch.rand((w.n, K), device="cuda") for w in ws]
+    rows = sum(len(p["mirror_vertex"]) for p in parts)
+    for compress in (False, True):
+        run_workers([(lambda i=i: gcn.graphsum_sync_rows(ws[i].g, dev[i], i, W, ws[i].comm, compress)) for i in range(W)])
+        t = time.perf_counter()
+        reps = 5
+        for _ in range(reps):
+            run_workers([(lambda i=i: gcn.graphsum_sync_rows(ws[i].g, dev[i], i, W, ws[i].comm, compress)) for i in range(W)])
+        ms = (time.perf_counter() - t) * 1e3 / reps
+        wire = rows * 2 * (4 + (K + 8 if compress else 4 * K))
+        out["graphsum_sync_K128_" + ("uint8" if compress else "f32")] = {
+            "ms": ms, "rows_per_phase": rows, "wire_bytes": wire, "row_GBps": rows * 2 * 4 * K * 2 / (ms * 1e-3) / 1e9}
+    for w in ws:
+        w.close()
+    lb.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -299,9 +350,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="launch the 1 GiB stream-copy kernel exactly once (a dispatch of known traffic to scale "
                          "rocprofv3 byte counters by)")
-    ap.add_argument("--suite", default="default", choices=["pr", "default", "full", "gcn", "sweep", "traverse"],
+    ap.add_argument("--suite", default="default", choices=["pr", "default", "full", "gcn", "sweep", "traverse", "exchange"],
                     help="pr: PageRank only; default: + GCN training step (configs[3]); full: + configs[2], [4] and the "
-                         "SSSP / CC jobs; gcn, sweep, traverse: that part alone")
+                         "SSSP / CC jobs and the replica exchange; gcn, sweep, traverse, exchange: that part alone")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs one subgraph on ONE GPU; there is no multi-GPU path to time "
@@ -324,8 +375,10 @@ def main():
     del a, b
     torch.cuda.empty_cache()
 
-    if args.suite in ("gcn", "sweep", "traverse"):      # profiling helpers: one part alone, no headline line
-        if args.suite == "traverse":
+    if args.suite in ("gcn", "sweep", "traverse", "exchange"):      # profiling helpers: one part alone, no headline line
+        if args.suite == "exchange":
+            part = bench_exchange()
+        elif args.suite == "traverse":
             part = bench_traverse(cpu_baseline=not args.no_cpu_baseline)
         else:
             part = bench_gcn_step(steps=max(3, args.steps), warmup=max(1, args.warmup)) if args.suite == "gcn" else bench_spmm_sweep()
@@ -404,6 +457,8 @@ def main():
         result["spmm_sweep"] = bench_spmm_sweep()
         torch.cuda.empty_cache()
         result["traverse"] = bench_traverse(cpu_baseline=not args.no_cpu_baseline)
+        torch.cuda.empty_cache()
+        result["exchange"] = bench_exchange()
     print(json.dumps(result), flush=True)
 
 
