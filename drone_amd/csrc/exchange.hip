@@ -108,6 +108,7 @@ void drone::routes_release(RouteLists *r)
     if (r->send_index_d) (void)hipFree(r->send_index_d);
     if (r->send_index_h) (void)hipHostFree(r->send_index_h);
     if (r->unknown) (void)hipFree(r->unknown);
+    if (r->unknown_h) (void)hipHostFree(r->unknown_h);
     *r = RouteLists{};
 }
 
@@ -172,6 +173,7 @@ int drone::routes_prepare(Graph *g, int workerNum)
     DRONE_HIP_TRY(hipMalloc(&r.send_index_d, sizeof(int) * ((size_t)workerNum + 1)));
     DRONE_HIP_TRY(hipHostMalloc(&r.send_index_h, sizeof(int) * ((size_t)workerNum + 1)));
     DRONE_HIP_TRY(hipMalloc(&r.unknown, sizeof(int)));
+    DRONE_HIP_TRY(hipHostMalloc(&r.unknown_h, sizeof(int)));
     r.workers = workerNum;
     r.ready = true;
     return DRONE_OK;
@@ -244,10 +246,9 @@ int drone::exchange_phase(Graph *g, int phase, typename Policy::T *vals, int *se
         total += len;
     }
     DRONE_HIP_TRY(hipGetLastError());
-    int bad = 0;
-    DRONE_HIP_TRY(hipMemcpyAsync(&bad, unknown, sizeof(int), hipMemcpyDeviceToHost, s));
+    DRONE_HIP_TRY(hipMemcpyAsync(r.unknown_h, unknown, sizeof(int), hipMemcpyDeviceToHost, s));
     DRONE_HIP_TRY(hipStreamSynchronize(s));
-    if (bad > 0) printf("error global id: %d received ids are not on worker %d\n", bad, workerId);
+    if (*r.unknown_h > 0) printf("error global id: %d received ids are not on worker %d\n", *r.unknown_h, workerId);
     *sent = r.send_index_h[workerNum];
     *received = total;
     return DRONE_OK;
@@ -290,6 +291,7 @@ struct drone_loopback {
         drone_loopback *group;
     };
     std::vector<Endpoint> endpoint;
+    float *scalars = nullptr, *sums = nullptr;  // pinned [workers] each: staging of the all-reduce
 
     // Returns false when a peer did not arrive in time (the group is then unusable).
     bool barrier()
@@ -387,23 +389,18 @@ int loopback_allreduce(void *ctx, int workerId, int workerNum, float *device_sca
 {
     drone_loopback *grp = static_cast<drone_loopback::Endpoint *>(ctx)->group;
     DRONE_REQUIRE(workerNum == grp->workers && workerId >= 0 && workerId < workerNum, "worker id / count");
+    DRONE_REQUIRE(grp->scalars != nullptr, "the group has no pinned staging");
     hipStream_t s = as_stream(stream);
-    DRONE_HIP_TRY(hipStreamSynchronize(s));  // the scalar is final before the peers read it
-    grp->slot[workerId].scalar = device_scalar;
+    // every worker lands its own value in the group's pinned array, then all of them add the array in worker order
+    DRONE_HIP_TRY(hipMemcpyAsync(grp->scalars + workerId, device_scalar, sizeof(float), hipMemcpyDeviceToHost, s));
+    DRONE_HIP_TRY(hipStreamSynchronize(s));
     if (!grp->barrier()) return loopback_fail("allreduce");
     float sum = 0.0f;
-    int rc = DRONE_OK;
-    for (int w = 0; w < workerNum; ++w) {
-        float v = 0.0f;
-        if (hipMemcpy(&v, grp->slot[w].scalar, sizeof(float), hipMemcpyDeviceToHost) != hipSuccess) {
-            set_error(DRONE_ERR_HIP, "loopback transport: reading a peer's scalar failed");
-            rc = DRONE_ERR_HIP;
-        }
-        sum += v;
-    }
-    if (!grp->barrier()) return loopback_fail("allreduce");  // everyone has read before anyone writes
-    if (rc != DRONE_OK) return rc;
-    DRONE_HIP_TRY(hipMemcpy(device_scalar, &sum, sizeof(float), hipMemcpyHostToDevice));
+    for (int w = 0; w < workerNum; ++w) sum += grp->scalars[w];
+    grp->sums[workerId] = sum;
+    if (!grp->barrier()) return loopback_fail("allreduce");  // everyone has read before the next call overwrites
+    DRONE_HIP_TRY(hipMemcpyAsync(device_scalar, grp->sums + workerId, sizeof(float), hipMemcpyHostToDevice, s));
+    DRONE_HIP_TRY(hipStreamSynchronize(s));
     return DRONE_OK;
 }
 
@@ -418,6 +415,9 @@ extern "C" int drone_loopback_create(drone_loopback **group, int workerNum, int 
     drone_loopback *g = new drone_loopback();
     g->workers = workerNum;
     g->timeout_ms = timeout_ms;
+    // pinned staging; without a device (host-only checks of the barrier logic) the group works except for the all-reduce
+    if (hipHostMalloc(&g->scalars, sizeof(float) * 2 * (size_t)workerNum) == hipSuccess) g->sums = g->scalars + workerNum;
+    else g->scalars = nullptr;
     g->slot.resize((size_t)workerNum);
     g->endpoint.resize((size_t)workerNum);
     for (int w = 0; w < workerNum; ++w) {
@@ -441,6 +441,7 @@ extern "C" int drone_loopback_attach(drone_loopback *group, int workerId, Comm *
 
 extern "C" int drone_loopback_destroy(drone_loopback *group)
 {
+    if (group && group->scalars) (void)hipHostFree(group->scalars);
     delete group;
     return DRONE_OK;
 }

@@ -26,6 +26,7 @@ struct RouteLists {
     int *send_index_d = nullptr;   // device [workers + 1]
     int *send_index_h = nullptr;   // pinned [workers + 1]
     int *unknown = nullptr;        // device scalar: received ids that are not on this worker
+    int *unknown_h = nullptr;      // pinned landing place of that scalar
 };
 
 // Staging of the K-wide row synchronisation (grow-only).

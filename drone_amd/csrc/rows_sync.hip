@@ -264,11 +264,10 @@ extern "C" int drone_graphsum_sync_rows_f32(Graph *g, float *data, int ld, int K
             total += len;
         }
         DRONE_HIP_TRY(hipGetLastError());
-        int bad = 0;
-        DRONE_HIP_TRY(hipMemcpyAsync(&bad, r.unknown, sizeof(int), hipMemcpyDeviceToHost, s));
+        DRONE_HIP_TRY(hipMemcpyAsync(r.unknown_h, r.unknown, sizeof(int), hipMemcpyDeviceToHost, s));
         DRONE_HIP_TRY(hipStreamSynchronize(s));
-        if (bad > 0) {
-            set_error(DRONE_ERR_INVALID, "%d received rows name vertices that are not on worker %d", bad, workerId);
+        if (*r.unknown_h > 0) {
+            set_error(DRONE_ERR_INVALID, "%d received rows name vertices that are not on worker %d", *r.unknown_h, workerId);
             return DRONE_ERR_INVALID;
         }
         if (up && mirror2master_recv) *mirror2master_recv = total;
