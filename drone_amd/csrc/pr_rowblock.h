@@ -23,13 +23,13 @@
 namespace drone {
 
 constexpr int kRbThreads = 1024;
-// Shape chosen by measurement on R-MAT scale 24 (ms per iteration): 512 K entries / unroll 8: 1.07; 1 M / 8: 0.96;
-// 1 M / 4: 0.92; 1 M / 2: 0.88; 1 M / 1: 1.00; 2 M / 4: 1.02 (too few heavy blocks for 256 CUs).  Larger blocks reuse
-// popular lines more often; a small unroll keeps a wavefront's gathers close together in the sorted order.
+// Shape chosen by measurement on R-MAT scale 24 (ms per iteration, with the slice layout of rb_accumulate): 16,384
+// rows / 1 M entries 0.685; 16,384 / 512 K 0.72; 16,384 / 2 M 0.87 (too few heavy blocks for 256 CUs); 8,192 rows (two
+// blocks per CU) / 1 M 0.85, / 512 K 0.99.  Larger blocks reuse popular lines more often.
 constexpr int kRbRows = 16384;       // most rows ending in one block (LDS accumulators: 128 KB)
 constexpr int kRbItems = 1 << 20;    // most entries in one block
 constexpr int kRbWeight = kRbItems / kRbRows;
-constexpr int kRbUnroll = 2;
+constexpr int kRbUnroll = 4;
 constexpr int kRbLdsBytes = (kRbRows + 8) * (int)sizeof(double);  // rows ending in a block <= kRbRows + 1, + the open row
 
 struct RowBlocks {
@@ -54,6 +54,8 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
                       hipStream_t stream);
 void row_blocks_destroy(RowBlocks *rb);
 
+__device__ __forceinline__ int64_t ceil_div_dev(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
 // Sum of `v` over the 1024 threads of the block, valid in thread 0.  s_red: 16 doubles of LDS.
 __device__ __forceinline__ double block_sum_1024(double v, double *s_red)
 {
@@ -69,24 +71,33 @@ __device__ __forceinline__ double block_sum_1024(double v, double *s_red)
 }
 
 // Adds the block's entries [e0, e1) into the LDS accumulators.  kWide reads the 6-byte layout, otherwise the packed
-// one.  Indices past the end are clamped to the last entry (gathered, then added as 0.0), which keeps the loop free
-// of divergent branches.  Measured on R-MAT scale 24 (ms per iteration): this form 0.86; the same with the next
-// step's entries requested ahead of the adds 0.89 (more gathers in flight spread a wavefront's accesses over more
-// lines); the 6-byte layout 0.88 - 0.90.
+// one.  Every wavefront sweeps its own contiguous slice of the (source-sorted) entries, 64 * kRbUnroll at a time.
+// With the 16 wavefronts interleaved at 64-entry granularity instead, neighbouring wavefronts ask for the same
+// popular line while its fill is still pending, and the L1 serialises them behind that fill (counters: the L1
+// stalled on pending data for 74 % of the kernel's cycles, the address unit held up by it for 35 %); with slices
+// the wavefronts work at 16 different places of the source vector and a line is waited for by one wavefront only.
+// Measured on R-MAT scale 24 (ms per iteration): interleaved, unroll 2: 0.857; slices, unroll 2 / 3 / 4 / 6 / 8:
+// 0.732 / 0.684 / 0.687 / 0.701 / 0.718; slices with the next step's entries requested ahead of the adds: 0.689.
+// Indices past the end of a slice are clamped to the block's last entry (gathered, then added as 0.0), which keeps
+// the loop free of divergent branches.
 template <bool kWide, typename Epi>
 __device__ __forceinline__ void rb_accumulate(int64_t e0, int64_t e1, int tid, const int32_t *__restrict__ col,
                                               const uint16_t *__restrict__ lrow, const uint32_t *__restrict__ packed,
                                               const int32_t *__restrict__ bases, const Epi &epi, double *s_acc)
 {
     if (e0 >= e1) return;
-    constexpr int64_t kStep = (int64_t)kRbThreads * kRbUnroll;
+    constexpr int kWaves = kRbThreads / kWave;
+    const int lane = tid & (kWave - 1), wave = tid / kWave;
+    const int64_t slice = ceil_div_dev(e1 - e0, (int64_t)kWaves * kWave) * kWave;  // a multiple of 64: batches stay whole
+    const int64_t s0 = e0 + wave * slice;
+    const int64_t s1 = s0 + slice < e1 ? s0 + slice : e1;
     const int64_t last = e1 - 1;
-    uint32_t a[kRbUnroll];
-    int32_t g[kRbUnroll];
-    auto fetch = [&](int64_t base) {
+    for (int64_t base = s0; base < s1; base += kWave * kRbUnroll) {
+        uint32_t a[kRbUnroll];
+        int32_t g[kRbUnroll];
 #pragma unroll
         for (int k = 0; k < kRbUnroll; ++k) {
-            int64_t e = base + tid + (int64_t)k * kRbThreads;
+            int64_t e = base + k * kWave + lane;
             e = e < last ? e : last;
             if (kWide) {
                 a[k] = (uint32_t)__builtin_nontemporal_load(col + e);
@@ -96,9 +107,6 @@ __device__ __forceinline__ void rb_accumulate(int64_t e0, int64_t e1, int tid, c
                 g[k] = bases[(e - e0) >> 6];  // same address for all lanes of a wavefront
             }
         }
-    };
-    for (int64_t base = e0; base < e1; base += kStep) {
-        fetch(base);
         int c[kRbUnroll], l[kRbUnroll];
 #pragma unroll
         for (int k = 0; k < kRbUnroll; ++k) {
@@ -110,7 +118,7 @@ __device__ __forceinline__ void rb_accumulate(int64_t e0, int64_t e1, int tid, c
         for (int k = 0; k < kRbUnroll; ++k) v[k] = epi.load(c[k]);
 #pragma unroll
         for (int k = 0; k < kRbUnroll; ++k)
-            atomicAdd(&s_acc[l[k]], base + tid + (int64_t)k * kRbThreads < e1 ? v[k] : 0.0);  // clamped entries add 0
+            atomicAdd(&s_acc[l[k]], base + k * kWave + lane < s1 ? v[k] : 0.0);  // clamped entries add 0
     }
 }
 
