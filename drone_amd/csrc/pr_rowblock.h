@@ -77,7 +77,10 @@ __device__ __forceinline__ double block_sum_1024(double v, double *s_red)
 // stalled on pending data for 74 % of the kernel's cycles, the address unit held up by it for 35 %); with slices
 // the wavefronts work at 16 different places of the source vector and a line is waited for by one wavefront only.
 // Measured on R-MAT scale 24 (ms per iteration): interleaved, unroll 2: 0.857; slices, unroll 2 / 3 / 4 / 6 / 8:
-// 0.732 / 0.684 / 0.687 / 0.701 / 0.718; slices with the next step's entries requested ahead of the adds: 0.689.
+// 0.732 / 0.684 / 0.687 / 0.701 / 0.718; slices with the next step's entries requested ahead of the adds: 0.689;
+// chunks of 1 K / 4 K / 16 K entries dealt round-robin to the wavefronts: 0.83 / 0.86 / 0.86; the same chunks with
+// every wavefront starting at a different place of the sweep: 0.76 / 0.74 / 0.77.  With slices a CU always runs a
+// mix of wavefronts that hit L1 (popular sources, the first slices) and wavefronts that miss (the cold tail).
 // Indices past the end of a slice are clamped to the block's last entry (gathered, then added as 0.0), which keeps
 // the loop free of divergent branches.
 template <bool kWide, typename Epi>
