@@ -162,6 +162,13 @@ SIGNATURES = {
     "drone_decompress_rows_u8": (_I, [_P, _P, _I, _I, _P, _I, _P]),
     "drone_graphsum_sync_rows_f32": (_I, [C.POINTER(Graph), _P, _I, _I, _I, _I, C.POINTER(Comm), _I,
                                           C.POINTER(_I), C.POINTER(_I)]),
+    "drone_row_cache_create": (_I, [C.POINTER(_P), C.POINTER(Graph), _I, _I]),
+    "drone_row_cache_destroy": (None, [_P]),
+    "drone_row_cache_size": (_I, [_P]),
+    "drone_graphsum_refresh_rows_cached_f32": (_I, [C.POINTER(Graph), _P, _I, _P, _I, _I, _I, _I, C.POINTER(Comm), _I,
+                                                    C.POINTER(_I), C.POINTER(_I)]),
+    "drone_graphsum_sync_rows_cached_f32": (_I, [C.POINTER(Graph), _P, _I, C.c_float, _P, _I, _I, _I, _I,
+                                                 C.POINTER(Comm), _I, C.POINTER(_I), C.POINTER(_I)]),
     "drone_loopback_create": (_I, [C.POINTER(_P), _I, _I]),
     "drone_loopback_attach": (_I, [_P, _I, C.POINTER(Comm)]),
     "drone_loopback_destroy": (_I, [_P]),

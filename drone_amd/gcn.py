@@ -2,6 +2,8 @@
 (torch only owns the memory; every operation below is one C-ABI call into libdrone_hip.so)."""
 import ctypes as C
 
+import numpy as np
+
 from ._lib import check, lib
 
 
@@ -234,6 +236,64 @@ def graphsum_sync_rows(g, data, workerId, workerNum, comm, compress=False):
     check(lib().drone_graphsum_sync_rows_f32(g, data.data_ptr(), data.stride(0), data.shape[1], int(workerId),
                                              int(workerNum), C.byref(comm), int(bool(compress)), C.byref(a), C.byref(b)))
     return a.value, b.value
+
+
+class RowCache:
+    """CacheBuffer plus the step schedule of CUDAGraphSum (cuda_gcn/src/cuda/cuda_communicate.cuh:48-58,
+    cuda_module.cu:156-159, :268-272, :364-368): the stale-row synchronisation of one GraphSum layer.
+
+    sync_value(data) / sync_grad(data) pick the full or the incremental synchronisation from train_step as the
+    reference does (values: full at step 0 and when step % 100 == 5; gradients: full when step % 10 == 0);
+    sync_grad ends the step (cuda_module.cu:388).  error_rate = [0.1, 0.0] (cuda_cache.cu:70-71); with
+    update_threshold set, every incremental value sync multiplies error_rate[0] by 0.9 (cuda_cache.cu:416-418).
+    refresh() and sync() are the two entry points without the schedule."""
+
+    def __init__(self, g, workerId, workerNum, comm, K, compress=False):
+        import ctypes as C
+        self.g, self.workerId, self.workerNum, self.comm, self.K = g, int(workerId), int(workerNum), comm, int(K)
+        self.compress = bool(compress)
+        self.error_rate = [0.1, 0.0]
+        self.train_step = 0
+        self.update_threshold = False
+        self.h = C.c_void_p()
+        check(lib().drone_row_cache_create(C.byref(self.h), g, self.workerNum, self.K))
+
+    @property
+    def size(self):
+        return lib().drone_row_cache_size(self.h)
+
+    def _call(self, fn, data, *lead):
+        import ctypes as C
+        a, b = C.c_int(0), C.c_int(0)
+        check(fn(self.g, self.h, *lead, data.data_ptr(), data.stride(0), data.shape[1], self.workerId, self.workerNum,
+                 C.byref(self.comm), int(self.compress), C.byref(a), C.byref(b)))
+        return a.value, b.value
+
+    def refresh(self, kind, data):
+        """drone_graphsum_refresh_rows_cached_f32: full synchronisation, both caches re-seeded."""
+        return self._call(lib().drone_graphsum_refresh_rows_cached_f32, data, int(kind))
+
+    def sync(self, kind, data, error_rate):
+        """drone_graphsum_sync_rows_cached_f32: incremental synchronisation with the given threshold."""
+        return self._call(lib().drone_graphsum_sync_rows_cached_f32, data, int(kind), float(error_rate))
+
+    def sync_value(self, data):
+        if self.train_step == 0 or self.train_step % 100 == 5:
+            return self.refresh(0, data)
+        r = self.sync(0, data, self.error_rate[0])
+        if self.update_threshold:
+            self.error_rate[0] = float(np.float32(self.error_rate[0]) * np.float32(0.9))
+        return r
+
+    def sync_grad(self, data):
+        r = self.refresh(1, data) if self.train_step % 10 == 0 else self.sync(1, data, self.error_rate[1])
+        self.train_step += 1
+        return r
+
+    def close(self):
+        if self.h:
+            lib().drone_row_cache_destroy(self.h)
+            self.h = None
 
 
 def clear_mirror_rows(grad, mirror2worker, stream=0):

@@ -413,6 +413,38 @@ int drone_decompress_rows_u8(const uint8_t *in, const float *maxmin, int rows, i
 int drone_graphsum_sync_rows_f32(Graph *g, float *data, int ld, int K, int workerId, int workerNum, Comm *comm,
                                  int compress, int *mirror2master_recv, int *master2mirror_recv);
 
+/* The stale-row ("SEMI_BATCH") synchronisation, cuda_gcn/src/cuda/cuda_cache.cu.  A drone_row_cache replaces
+ * CacheBuffer (cuda_communicate.cuh:48-58, constructor cuda_cache.cu:45-72): for every replicated vertex of the
+ * subgraph (mirror, or master with a mirror somewhere; cuda_cache.cu:13-43) it keeps, per kind (0 = values,
+ * 1 = gradients), the partial row this worker last contributed and the row all replicas last agreed on, K floats
+ * each, zero at creation.  Create it after addMasterRoute / addMirrorRoute; it belongs to (g, workerNum, K).
+ * drone_row_cache_size returns the reference's cacheSize (MasterSize + MirrorSize). */
+typedef struct drone_row_cache drone_row_cache;
+int drone_row_cache_create(drone_row_cache **out, Graph *g, int workerNum, int K);
+void drone_row_cache_destroy(drone_row_cache *cache);
+int drone_row_cache_size(const drone_row_cache *cache);
+/* GraphSum_sync_value_nccl / GraphSum_sync_grad_nccl under SEMI_BATCH (cuda_communicate.cu:374-448, :502-557): the
+ * full synchronisation of drone_graphsum_sync_rows_f32 with the contributed rows cached before it (:381-384) and
+ * the agreed rows cached after it (:442-445).  The reference takes this branch at train_step 0 and whenever
+ * train_step % 100 == 5 (values, cuda_module.cu:268) or train_step % 10 == 0 (gradients, cuda_module.cu:364). */
+int drone_graphsum_refresh_rows_cached_f32(Graph *g, drone_row_cache *cache, int kind, float *data, int ld, int K,
+                                           int workerId, int workerNum, Comm *comm, int compress,
+                                           int *mirror2master_recv, int *master2mirror_recv);
+/* GraphSum_sync_value_nccl_cache / GraphSum_sync_grad_nccl_cache (cuda_cache.cu:361-507, :509-626), every other
+ * step.  Per replicated vertex: diff = row - contributed; the replica is active iff max|diff| > max|row| *
+ * error_rate (cuda_cache.cu:106-150, :219-229; the reference starts at 0.1 for values, 0.0 for gradients, and
+ * multiplies the former by 0.9 while the training accuracy falls behind its running mean, cuda_cache.cu:416,
+ * cuda_gcn.cu:366-367 -- that policy stays with the caller).  Active mirrors send diff to their master, which
+ * adds it to the agreed row (source workers in ascending order) and becomes active; every active replica adds
+ * diff to its contributed row; every active master adds its own diff to the agreed row and sends that row to all
+ * its mirrors; finally every replicated vertex's row in data is overwritten with the agreed row, current or
+ * stale.  compress != 0 sends the rows as uint8.  The two outputs (may be NULL) receive the row counts that
+ * arrived per phase (mirror2master_*_total / master2mirror_*_total of the reference).  Blocks like the other
+ * entry points; one call per graph at a time. */
+int drone_graphsum_sync_rows_cached_f32(Graph *g, drone_row_cache *cache, int kind, float error_rate, float *data,
+                                        int ld, int K, int workerId, int workerNum, Comm *comm, int compress,
+                                        int *mirror2master_recv, int *master2mirror_recv);
+
 #ifdef __cplusplus
 }
 #endif

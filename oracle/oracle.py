@@ -498,3 +498,85 @@ def graphsum_sync_rows(parts, data, compress=False):
                 data[dst][p.g2l[gid]] = row
                 recv1[dst] += 1
     return recv0, recv1
+
+
+class RowCacheGroup:
+    """The stale-row ("SEMI_BATCH") synchronisation of cuda_gcn/src/cuda/cuda_cache.cu over all workers at once.
+
+    Every replicated vertex (mirror, or master with at least one mirror: cuda_cache.cu:13-43) keeps two cached
+    rows per kind (0 = values, 1 = gradients): `local`, the partial row this worker last contributed, and `glob`,
+    the row all replicas last agreed on.  refresh() is the full synchronisation with both caches re-seeded around
+    it (cuda_communicate.cu:381-384 before, :442-445 after).  sync() is the incremental one (cuda_cache.cu:361-507
+    for values, :509-626 for gradients):
+      diff = row - local;  active = max|diff| > max|row| * error_rate          (cal_diff_absMax, cal_active)
+      active mirrors send diff to the master, which adds it to glob and becomes active   (apply_sum_diff_*)
+      every active replica: local += diff                                        (update_localCache)
+      every active master: glob += diff, sends glob to all its mirrors, which store it   (set_sync_master2mirror_cache,
+                                                                                          apply_assign_global_*)
+      every replica: row = glob                                                  (load_cache)
+    Additions at a master happen in ascending source-worker order, its own diff last.  Rows on the wire pass through
+    the uint8 compression when compress is set.
+    """
+
+    def __init__(self, parts, K):
+        self.parts, self.K = parts, K
+        self.cached = []
+        for p in parts:
+            c = p.m2w != -1
+            for v in p.master_workers:
+                if len(p.master_workers[v]) > 0:
+                    c[v] = True
+            self.cached.append(c)
+        self.local = [[np.zeros((p.n, K), np.float32) for p in parts] for _ in range(2)]
+        self.glob = [[np.zeros((p.n, K), np.float32) for p in parts] for _ in range(2)]
+
+    def refresh(self, kind, data, compress=False):
+        for w, c in enumerate(self.cached):
+            self.local[kind][w][c] = data[w][c]
+        r = graphsum_sync_rows(self.parts, data, compress=compress)
+        for w, c in enumerate(self.cached):
+            self.glob[kind][w][c] = data[w][c]
+        return r
+
+    def sync(self, kind, data, error_rate, compress=False):
+        parts, W = self.parts, len(self.parts)
+        local, glob = self.local[kind], self.glob[kind]
+        wire = (lambda r: decompress_rows_u8(*compress_rows_u8(r[None, :]))[0]) if compress else (lambda r: r.copy())
+        diff, active = [], []
+        for w, p in enumerate(parts):
+            d = (data[w] - local[w]).astype(np.float32)
+            md = np.abs(d).max(axis=1) if self.K else np.zeros(p.n, np.float32)
+            mv = np.abs(data[w]).max(axis=1)
+            diff.append(d)
+            active.append(self.cached[w] & (md > (mv * np.float32(error_rate)).astype(np.float32)))
+        recv0, recv1 = [0] * W, [0] * W
+        box = [[[] for _ in range(W)] for _ in range(W)]
+        for w, p in enumerate(parts):
+            for v in np.nonzero((p.m2w != -1) & active[w])[0]:
+                box[w][p.m2w[v]].append((p.l2g[v], wire(diff[w][v])))
+        for dst, p in enumerate(parts):
+            for src in range(W):
+                for gid, row in box[src][dst]:
+                    l = p.g2l[gid]
+                    glob[dst][l] = (glob[dst][l] + row).astype(np.float32)
+                    active[dst][l] = True
+                    recv0[dst] += 1
+        for w in range(W):
+            rows = self.cached[w] & active[w]
+            local[w][rows] = (local[w][rows] + diff[w][rows]).astype(np.float32)
+        box = [[[] for _ in range(W)] for _ in range(W)]
+        for w, p in enumerate(parts):
+            for v in sorted(p.master_workers):
+                if not p.master_workers[v] or not active[w][v]:
+                    continue
+                glob[w][v] = (glob[w][v] + diff[w][v]).astype(np.float32)
+                for dst in p.master_workers[v]:
+                    box[w][dst].append((p.l2g[v], wire(glob[w][v])))
+        for dst, p in enumerate(parts):
+            for src in range(W):
+                for gid, row in box[src][dst]:
+                    glob[dst][p.g2l[gid]] = row
+                    recv1[dst] += 1
+        for w, c in enumerate(self.cached):
+            data[w][c] = glob[w][c]
+        return recv0, recv1

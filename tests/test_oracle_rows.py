@@ -64,3 +64,119 @@ def test_row_sync_makes_every_replica_the_sum_of_all_replicas(oracle):
             if gid in seen:
                 np.testing.assert_array_equal(d[l], seen[gid])
             seen[gid] = d[l]
+
+
+# ---- stale-row cache (cuda_cache.cu) ---------------------------------------------------------------------------
+def _two_workers_one_shared_vertex(oracle):
+    """Global vertices 0..2; vertex 1 is shared: worker 0 holds the master, worker 1 a mirror."""
+    a = oracle.Part([0, 1], 3, master_vertex=[1], mirror_number=[1], mirror_workers=[1])
+    b = oracle.Part([1, 2], 3, mirror_vertex=[1], master_worker=[0])
+    return [a, b]
+
+
+def test_row_cache_hand_vectors(oracle):
+    tops = _two_workers_one_shared_vertex(oracle)
+    grp = oracle.RowCacheGroup(tops, 2)
+    d = [np.array([[9, 9], [1, 2]], np.float32), np.array([[10, 20], [7, 7]], np.float32)]
+    assert grp.refresh(0, d) == ([1, 0], [0, 1])
+    np.testing.assert_array_equal(d[0], [[9, 9], [11, 22]])
+    np.testing.assert_array_equal(d[1], [[11, 22], [7, 7]])
+    # only the mirror moves beyond 10 %: its diff (+8, 0) reaches the master, which then also contributes its own
+    # small diff (+0, +0.125) although that alone was below the threshold
+    d = [np.array([[5, 5], [1, 2.125]], np.float32), np.array([[18, 20], [6, 6]], np.float32)]
+    assert grp.sync(0, d, 0.1) == ([1, 0], [0, 1])
+    np.testing.assert_array_equal(d[0], [[5, 5], [19, 22.125]])      # unreplicated rows are never touched
+    np.testing.assert_array_equal(d[1], [[19, 22.125], [6, 6]])
+    np.testing.assert_array_equal(grp.local[0][0][1], [1, 2.125])
+    np.testing.assert_array_equal(grp.local[0][1][0], [18, 20])
+    # only the master moves: the mirror sends nothing, keeps its contribution, and receives the new row
+    d = [np.array([[5, 5], [3, 2.125]], np.float32), np.array([[18.5, 20], [6, 6]], np.float32)]
+    assert grp.sync(0, d, 0.1) == ([0, 0], [0, 1])
+    np.testing.assert_array_equal(d[0][1], [21, 22.125])
+    np.testing.assert_array_equal(d[1][0], [21, 22.125])
+    np.testing.assert_array_equal(grp.local[0][1][0], [18, 20])      # the mirror's skipped change stays pending
+    # nobody moves: no traffic, everybody reads the stale agreed row; the gradient caches are separate state
+    d = [np.array([[5, 5], [3.25, 2.125]], np.float32), np.array([[18.5, 20], [6, 6]], np.float32)]
+    assert grp.sync(0, d, 0.1) == ([0, 0], [0, 0])
+    np.testing.assert_array_equal(d[0][1], [21, 22.125])
+    np.testing.assert_array_equal(d[1][0], [21, 22.125])
+    assert not grp.local[1][0].any() and not grp.glob[1][1].any()
+    # threshold 0: every pending change is flushed and the result is the exact sum again
+    d = [np.array([[5, 5], [3.25, 2.125]], np.float32), np.array([[18.5, 20], [6, 6]], np.float32)]
+    assert grp.sync(0, d, 0.0) == ([1, 0], [0, 1])
+    np.testing.assert_array_equal(d[0][1], [21.75, 22.125])
+    np.testing.assert_array_equal(d[1][0], [21.75, 22.125])
+
+
+def _exact_sum(tops, data, n):
+    want = np.zeros((n, data[0].shape[1]))
+    for t, d in zip(tops, data):
+        np.add.at(want, t.l2g, d.astype(np.float64))
+    return want
+
+
+@pytest.mark.parametrize("compress", [False, True])
+def test_row_cache_threshold_zero_tracks_the_exact_sum(oracle, compress):
+    rng = np.random.default_rng(11)
+    n, W, K = 200, 4, 6
+    u, v = rng.integers(0, n, 1500), rng.integers(0, n, 1500)
+    keep = u != v
+    parts, tops = _parts(oracle, n, u[keep].astype(np.int32), v[keep].astype(np.int32), W, 5)
+    grp = oracle.RowCacheGroup(tops, K)
+    rows = [rng.standard_normal((t.n, K)).astype(np.float32) for t in tops]
+    data = [r.copy() for r in rows]
+    grp.refresh(1, data, compress=False)
+    tol = dict(rtol=1e-5, atol=1e-5)
+    for step in range(4):
+        rows = [(r + 0.1 * rng.standard_normal(r.shape)).astype(np.float32) for r in rows]
+        data = [r.copy() for r in rows]
+        r0, r1 = grp.sync(1, data, 0.0, compress=compress)
+        want = _exact_sum(tops, rows, n)
+        for t, d, c in zip(tops, data, grp.cached):
+            if compress:   # each wire crossing may be off by half a quantisation step of that row
+                assert np.abs(d[c] - want[t.l2g][c]).max() < 0.05 * (step + 1)
+            else:
+                np.testing.assert_allclose(d[c], want[t.l2g][c], **tol)
+            np.testing.assert_array_equal(d[~c], rows[tops.index(t)][~c])
+        assert sum(r0) == sum(int((t.m2w != -1).sum()) for t in tops) and sum(r1) == sum(r0)
+    # unchanged rows: they differ from what was contributed by float rounding of local + (row - local) only, so
+    # with a threshold just above that nothing is sent and the agreed rows come back
+    before = [d.copy() for d in data]
+    data = [r.copy() for r in rows]
+    assert grp.sync(1, data, 1e-5, compress=compress) == ([0] * W, [0] * W)
+    for d, b in zip(data, before):
+        np.testing.assert_array_equal(d, b)
+
+
+def test_row_cache_staleness_is_bounded_by_the_threshold(oracle):
+    rng = np.random.default_rng(12)
+    n, W, K, e = 300, 5, 8, 0.2
+    u, v = rng.integers(0, n, 2500), rng.integers(0, n, 2500)
+    keep = u != v
+    parts, tops = _parts(oracle, n, u[keep].astype(np.int32), v[keep].astype(np.int32), W, 6)
+    grp = oracle.RowCacheGroup(tops, K)
+    rows = [rng.standard_normal((t.n, K)).astype(np.float32) for t in tops]
+    data = [r.copy() for r in rows]
+    full = grp.refresh(0, data)
+    sent = []
+    for step in range(5):
+        rows = [(r * (1 + 0.15 * rng.standard_normal((r.shape[0], 1)))).astype(np.float32) for r in rows]
+        data = [r.copy() for r in rows]
+        r0, r1 = grp.sync(0, data, e)
+        sent.append(sum(r0))
+        want = _exact_sum(tops, rows, n)
+        # a replica that stayed silent is off by less than e * max|row|; slack[g] sums that over the replicas of g
+        slack = np.zeros(n)
+        for t, r, lc in zip(tops, rows, grp.local[0]):
+            np.add.at(slack, t.l2g, np.abs(r - lc).max(axis=1))
+            assert np.all(np.abs(r - lc).max(axis=1)[grp.cached[tops.index(t)]]
+                          <= e * np.abs(r).max(axis=1)[grp.cached[tops.index(t)]] + 1e-6)
+        for t, d, c in zip(tops, data, grp.cached):
+            assert np.all(np.abs(d[c] - want[t.l2g][c]).max(axis=1) <= slack[t.l2g][c] + 1e-4)
+    assert 0 < min(sent) and max(sent) < sum(full[0])          # some rows travel, never all of them
+    # a threshold nobody reaches: silence, and every replica reads the agreed row of the previous step
+    prev = [d.copy() for d in data]
+    data = [(r * 1.5).astype(np.float32) for r in rows]
+    assert grp.sync(0, data, 10.0) == ([0] * W, [0] * W)
+    for d, p, c in zip(data, prev, grp.cached):
+        np.testing.assert_array_equal(d[c], p[c])

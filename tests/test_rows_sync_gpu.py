@@ -112,3 +112,147 @@ def test_clear_mirror_rows(oracle):
     want[m2w != -1, :K] = 0.0
     gcn.clear_mirror_rows(full[:, :K], torch.from_numpy(m2w).cuda())
     np.testing.assert_array_equal(full.cpu().numpy(), want)
+
+
+# ---- stale-row cache (cuda_cache.cu) ---------------------------------------------------------------------------
+@pytest.mark.parametrize("compress", [False, True])
+@pytest.mark.parametrize("W,scale,K,seed", [(2, 8, 16, 1), (3, 11, 41, 2), (4, 10, 128, 3)])
+def test_row_cache_sync_matches_oracle(oracle, compress, W, scale, K, seed):
+    """refresh, then incremental steps with drifting rows at several thresholds (0: everything travels; 0.05 / 0.3:
+    some replicas stay silent; 50: nobody moves), values and gradients interleaved: every worker's rows and the
+    per-phase receive counts equal the oracle's, bit for bit."""
+    import torch
+    from drone_amd import gcn, rmat
+    from drone_amd.pagerank import Loopback, run_workers
+    from drone_amd.traverse import _WorkerCUDA
+    n = 1 << scale
+    s, d = rmat.rmat_edges(scale, 8 << scale, seed=seed)
+    u, v = rmat.clean_directed_np(s, d)
+    parts, _ = vertex_cut(u, v, W, seed)
+    tops = []
+    rng = np.random.default_rng(seed)
+    for p in parts:
+        nl, g2l, l2g, index, dst = oracle.build_graph(n, p["u"], p["v"])
+        tops.append(oracle.Part(l2g, n, p["master_vertex"], p["mirror_number"], p["mirror_workers"],
+                                p["mirror_vertex"], p["master_worker"]))
+    grp = oracle.RowCacheGroup(tops, K)
+    lb = Loopback(W, timeout_ms=60000)
+    ws = [_WorkerCUDA(n, p["u"], p["v"], workerId=i, workerNum=W, routes=p, loopback=lb) for i, p in enumerate(parts)]
+    caches = [gcn.RowCache(ws[i].g, i, W, ws[i].comm, K, compress=compress) for i in range(W)]
+    try:
+        for i in range(W):
+            assert caches[i].size == int(grp.cached[i].sum())
+        rows = [[rng.standard_normal((t.n, K)).astype(np.float32) for t in tops] for _ in range(2)]
+        plan = [(0, None), (1, None), (0, 0.05), (1, 0.0), (0, 0.3), (0, 0.0), (1, 0.3), (0, 50.0), (1, None), (1, 0.05)]
+        moved = []
+        for kind, rate in plan:
+            rows[kind] = [(r * (1 + 0.2 * rng.standard_normal((r.shape[0], 1))) + 0.01 * rng.standard_normal(r.shape))
+                          .astype(np.float32) for r in rows[kind]]
+            host = [r.copy() for r in rows[kind]]
+            dev = [torch.from_numpy(r).cuda() for r in rows[kind]]
+            if rate is None:
+                want = grp.refresh(kind, host, compress=compress)
+                got = run_workers([(lambda i=i: caches[i].refresh(kind, dev[i])) for i in range(W)])
+            else:
+                want = grp.sync(kind, host, rate, compress=compress)
+                got = run_workers([(lambda i=i: caches[i].sync(kind, dev[i], rate)) for i in range(W)])
+                moved.append((rate, sum(want[0])))
+            for i in range(W):
+                assert got[i] == (want[0][i], want[1][i]), (kind, rate, i)
+                np.testing.assert_array_equal(dev[i].cpu().numpy(), host[i], err_msg=f"kind {kind} rate {rate} worker {i}")
+        total = sum(int((t.m2w != -1).sum()) for t in tops)
+        by_rate = dict(moved)
+        assert by_rate[50.0] == 0 and by_rate[0.0] == total and 0 < by_rate[0.3] < total
+    finally:
+        for c in caches:
+            c.close()
+        for w in ws:
+            lib_close(w)
+        lb.close()
+
+
+def test_row_cache_schedule_and_padded_rows(oracle):
+    """The step schedule of CUDAGraphSum (full sync at step 0 and step % 100 == 5 for values, step % 10 == 0 for
+    gradients, threshold decay) on rows with a padded leading dimension."""
+    import torch
+    from drone_amd import gcn, rmat
+    from drone_amd.pagerank import Loopback, run_workers
+    from drone_amd.traverse import _WorkerCUDA
+    W, scale, K, ld, seed = 3, 9, 41, 44, 7
+    n = 1 << scale
+    s, d = rmat.rmat_edges(scale, 8 << scale, seed=seed)
+    u, v = rmat.clean_directed_np(s, d)
+    parts, _ = vertex_cut(u, v, W, seed)
+    tops = []
+    rng = np.random.default_rng(seed)
+    for p in parts:
+        nl, g2l, l2g, index, dst = oracle.build_graph(n, p["u"], p["v"])
+        tops.append(oracle.Part(l2g, n, p["master_vertex"], p["mirror_number"], p["mirror_workers"],
+                                p["mirror_vertex"], p["master_worker"]))
+    grp = oracle.RowCacheGroup(tops, K)
+    lb = Loopback(W, timeout_ms=60000)
+    ws = [_WorkerCUDA(n, p["u"], p["v"], workerId=i, workerNum=W, routes=p, loopback=lb) for i, p in enumerate(parts)]
+    caches = [gcn.RowCache(ws[i].g, i, W, ws[i].comm, K) for i in range(W)]
+    try:
+        rate = np.float32(0.1)
+        rows = [rng.standard_normal((t.n, K)).astype(np.float32) for t in tops]
+        for step in range(13):
+            for c in caches:
+                c.update_threshold = step >= 8
+            for kind in (0, 1):
+                rows = [(r + 0.05 * rng.standard_normal(r.shape)).astype(np.float32) for r in rows]
+                host = [r.copy() for r in rows]
+                full = torch.full((max(t.n for t in tops), ld), 7.0)
+                dev = []
+                for r in rows:
+                    t = full[:r.shape[0]].clone().cuda()
+                    t[:, :K] = torch.from_numpy(r).cuda()
+                    dev.append(t)
+                if kind == 0:
+                    refresh = step == 0 or step % 100 == 5
+                    want = grp.refresh(0, host) if refresh else grp.sync(0, host, rate)
+                    if not refresh and step >= 8:
+                        rate = np.float32(rate * np.float32(0.9))
+                    got = run_workers([(lambda i=i: caches[i].sync_value(dev[i][:, :K])) for i in range(W)])
+                else:
+                    want = grp.refresh(1, host) if step % 10 == 0 else grp.sync(1, host, 0.0)
+                    got = run_workers([(lambda i=i: caches[i].sync_grad(dev[i][:, :K])) for i in range(W)])
+                for i in range(W):
+                    assert got[i] == (want[0][i], want[1][i]), (step, kind, i)
+                    out = dev[i].cpu().numpy()
+                    np.testing.assert_array_equal(out[:, :K], host[i])
+                    assert np.all(out[:, K:] == 7.0)
+        assert caches[0].train_step == 13 and abs(caches[0].error_rate[0] - float(rate)) < 1e-7 and rate < 0.1
+    finally:
+        for c in caches:
+            c.close()
+        for w in ws:
+            lib_close(w)
+        lb.close()
+
+
+def test_row_cache_argument_checks(oracle):
+    import ctypes as C
+    import torch
+    from drone_amd import gcn
+    from drone_amd._lib import lib
+    from drone_amd.traverse import _WorkerCUDA
+    w = _WorkerCUDA(8, np.array([0, 1], np.int32), np.array([1, 2], np.int32))
+    c = gcn.RowCache(w.g, 0, 1, w.comm, 4)
+    x = torch.randn((3, 4), device="cuda")
+    keep = x.clone()
+    assert c.size == 0
+    assert c.refresh(0, x) == (0, 0) and c.sync(1, x, 0.1) == (0, 0)     # one worker: nothing is replicated
+    assert torch.equal(x, keep)
+    L = lib()
+    a = C.c_int(0)
+    args = (x.data_ptr(), 4, 4, 0, 1, C.byref(w.comm), 0, C.byref(a), C.byref(a))
+    assert L.drone_graphsum_sync_rows_cached_f32(w.g, c.h, 2, 0.1, *args) == -1            # kind
+    assert L.drone_graphsum_sync_rows_cached_f32(w.g, c.h, 0, -0.5, *args) == -1           # threshold
+    assert L.drone_graphsum_sync_rows_cached_f32(w.g, c.h, 0, 0.1, x.data_ptr(), 4, 3, 0, 1, C.byref(w.comm), 0,
+                                                 None, None) == -1                          # K of another cache
+    assert L.drone_graphsum_refresh_rows_cached_f32(w.g, None, 0, *args) == -1
+    h = C.c_void_p()
+    assert L.drone_row_cache_create(C.byref(h), w.g, 1, 0) == -1
+    c.close()
+    lib_close(w)
