@@ -291,8 +291,8 @@ def bench_traverse(cpu_baseline=True):
 def bench_exchange():
     """Four subgraphs of a random vertex cut of R-MAT scale 20 (ef 16, seed 2) on one GPU, each worker on its own host
     thread over the in-process loopback transport: PR_PEVal + 5 x PR_IncEVal with the two exchange phases per
-    superstep, and the K-wide row sync of the GCN (K = 128) with and without uint8 compression.  Bytes = ids +
-    values packed once and applied once."""
+    superstep, the K-wide row sync of the GCN (K = 128) with and without uint8 compression, and the stale-row
+    cached sync at three thresholds.  Bytes = ids + values packed once and applied once."""
     import numpy as np
     import torch
     from drone_amd import gcn, rmat
@@ -333,6 +333,26 @@ def bench_exchange():
         wire = rows * 2 * (4 + (K + 8 if compress else 4 * K))
         out["graphsum_sync_K128_" + ("uint8" if compress else "f32")] = {
             "ms": ms, "rows_per_phase": rows, "wire_bytes": wire, "row_GBps": rows * 2 * 4 * K * 2 / (ms * 1e-3) / 1e9}
+    # stale-row cache on the same graphs: rows drift by about 5 % per step (every element scaled by 1 + 0.05 * N(0, 1))
+    caches = [gcn.RowCache(ws[i].g, i, W, ws[i].comm, K) for i in range(W)]
+    base = [torch.rand((w.n, K), device="cuda") + 0.5 for w in ws]
+    work = [b.clone() for b in base]
+    run_workers([(lambda i=i: caches[i].refresh(0, work[i])) for i in range(W)])
+    for rate in (0.0, 0.1, 0.2):
+        ms_all, moved = [], []
+        for _ in range(5):
+            for i in range(W):
+                base[i].mul_(1 + 0.05 * torch.randn_like(base[i]))
+                work[i].copy_(base[i])
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            got = run_workers([(lambda i=i: caches[i].sync(0, work[i], rate)) for i in range(W)])
+            ms_all.append((time.perf_counter() - t) * 1e3)
+            moved.append(sum(g[0] for g in got))
+        out[f"graphsum_cached_sync_K128_rate_{rate}"] = {
+            "ms": float(np.median(ms_all)), "mirror_rows_sent": int(np.median(moved)), "mirror_rows": rows}
+    for c in caches:
+        c.close()
     for w in ws:
         w.close()
     lb.close()
