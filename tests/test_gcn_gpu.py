@@ -353,3 +353,64 @@ def test_spmm_dense_core_matches_oracle(T, oracle):
     b = gcn.spmm(plan, d_rp, d_ci, d_val, dev(T, B))
     assert T.equal(a, b)                       # repeatable bit for bit
     plan.close()
+
+
+def _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, row_sums):
+    """Size-independent checks of C = A * B at a benchmark shape: A * 1 against fp64 row sums, adjointness
+    <A X, Y> = <X, A^T Y> with the separately built transpose, agreement with the vendor's sparse product on a
+    column sample, and a repeatable result."""
+    plan = gcn.SpmmPlan(rp, ci, val, N, max_k=K)
+    planT = gcn.SpmmPlan(rpT, ciT, vT, N, max_k=K)
+    ones = torch.ones((N, 4), device="cuda")
+    got = gcn.spmm(plan, rp, ci, val, ones)
+    assert float(((got[:, 0].double() - row_sums).abs() / row_sums.abs().clamp(min=1e-30)).max()) <= 1e-4
+    g = torch.Generator(device="cuda").manual_seed(K)
+    X = torch.rand((N, K), device="cuda", generator=g) * 2 - 1
+    Y = torch.rand((N, K), device="cuda", generator=g) * 2 - 1
+    AX = gcn.spmm(plan, rp, ci, val, X)
+    ATY = gcn.spmm(planT, rpT, ciT, vT, Y)
+    lhs = float((AX.double() * Y.double()).sum())
+    rhs = float((X.double() * ATY.double()).sum())
+    scale = float((AX.double().abs() * Y.double().abs()).sum())
+    assert abs(lhs - rhs) <= 1e-4 * scale
+    assert torch.equal(gcn.spmm(plan, rp, ci, val, X), AX)          # fixed summation order
+    # vendor sparse product in fp64 on four columns
+    A64 = torch.sparse_csr_tensor(rp.long(), ci.long(), val.double(), size=(N, N))
+    cols = [0, 1, K // 2, K - 1]
+    ref = torch.sparse.mm(A64, X[:, cols].double().contiguous())
+    err = (AX[:, cols].double() - ref).abs().max(dim=0).values / ref.abs().max(dim=0).values
+    assert float(err.max()) <= 1e-4
+    plan.close()
+    planT.close()
+
+
+def test_full_size_properties_config3(T):
+    """Third configuration at full size: R-MAT scale 20, symmetrised with self-loops, normalised adjacency, K = 128."""
+    torch = T
+    from drone_amd import gcn, graphs
+    g = graphs.gcn_graph_torch(20, 16, seed=3)
+    N, rp, ci, deg = g["n"], g["rp"], g["ci"], g["deg"]
+    assert N == 1 << 20 and 30e6 < g["nnz"] < 36e6
+    val = gcn.edge_values(rp, ci, deg, deg)
+    rpT, ciT, vT = gcn.csr_transpose(N, N, rp, ci, val)
+    assert torch.equal(rpT, rp) and torch.equal(ciT, ci) and torch.equal(vT, val)      # symmetric
+    cs = torch.cat([torch.zeros(1, dtype=torch.float64, device="cuda"), torch.cumsum(val.double(), 0)])
+    _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, 128, cs[rp[1:].long()] - cs[rp[:-1].long()])
+
+
+@pytest.mark.parametrize("K", [16, 64])
+def test_full_size_properties_config5(T, K):
+    """Fifth configuration at full size: skewed directed R-MAT scale 22 ef 32, row-normalised; forward and transposed
+    products (K = 256 has the same code path as the 128-wide tiles of the other configurations)."""
+    torch = T
+    from drone_amd import gcn, rmat
+    x = rmat.pagerank_inputs_torch(22, 32, 5, a=0.70, b=0.12, c=0.12)
+    N = x["n"]
+    rp = x["row_ptr"].to(torch.int32)
+    ci = x["col_idx"]
+    assert N == 1 << 22 and 80e6 < x["nnz"] <= 134_217_728          # duplicates of the skewed generator are dropped
+    cnt = (rp[1:] - rp[:-1]).long()
+    val = (1.0 / torch.repeat_interleave(cnt.clamp(min=1).float(), cnt)).contiguous()
+    rpT, ciT, vT = gcn.csr_transpose(N, N, rp, ci, val)
+    assert int(rpT[-1]) == x["nnz"] and int((ciT[1:] < ciT[:-1]).sum()) <= N          # rows ascending inside
+    _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, (cnt > 0).double())
