@@ -2,7 +2,7 @@
 
 python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Headline workload (BASELINE.json configs[1]): PageRank on one subgraph at real shape - R-MAT scale 24, edge
+Headline workload (the second benchmark configuration, configs[1]): PageRank on one subgraph at real shape - R-MAT scale 24, edge
 factor 16, seed 2, in-edge CSR (int64 row_ptr, int32 col_idx), fp64 ranks, damping 0.85.  One "step" is one
 complete 50-iteration PageRank job through drone_pr_run_f64; inputs are resident in HBM before the timed
 region.  value = directed edges in the CSR x 50 x K / seconds / 1e9 (GTEPS).
