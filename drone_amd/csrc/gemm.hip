@@ -26,15 +26,37 @@ constexpr int BM = 128;
 constexpr int BK = 16;
 constexpr int PAD = 4;
 
+// Four consecutive floats that are only known to be 4-byte aligned (leading dimensions such as 602 or 41 are
+// odd multiples of a dword); the hardware takes such a 16-byte load in one instruction.
+struct alignas(4) Float4U {
+    float v[4];
+};
+
 // Loads a (BK x EXT) k-major tile of op(X) into registers: element (k, i) for k in [0,BK), i in [0,EXT).
 // K_CONTIG: memory holds X[i][k] (k contiguous) - lanes walk k fastest; else X[k][i] - lanes walk i fastest.
+// A tile that lies wholly inside the matrix is fetched as 16-byte loads without bounds checks (`full`, uniform
+// over the work-group); edge tiles take dword loads with a check per element.  The two paths distribute the
+// elements over the lanes differently, so store() must be told which one filled the registers.
 template <int EXT, bool K_CONTIG>
 struct TileLoader {
     static constexpr int PER = BK * EXT / 256;
+    static constexpr int VPER = PER / 4;
     float r[PER];
-    __device__ __forceinline__ void load(const float *__restrict__ X, int ld, int i0, int i_end, int k0, int k_end)
+    __device__ __forceinline__ void load(const float *__restrict__ X, int ld, int i0, int i_end, int k0, int k_end, bool full)
     {
         const int t = threadIdx.x;
+        if (full) {
+#pragma unroll
+            for (int p = 0; p < VPER; ++p) {
+                const float *src;
+                if constexpr (K_CONTIG) src = X + (size_t)(i0 + t / (BK / 4) + p * (1024 / BK)) * ld + k0 + 4 * (t % (BK / 4));
+                else src = X + (size_t)(k0 + t / (EXT / 4) + p * (1024 / EXT)) * ld + i0 + 4 * (t % (EXT / 4));
+                const Float4U q = *reinterpret_cast<const Float4U *>(src);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) r[4 * p + j] = q.v[j];
+            }
+            return;
+        }
 #pragma unroll
         for (int p = 0; p < PER; ++p) {
             int k, i;
@@ -46,9 +68,23 @@ struct TileLoader {
             r[p] = v;
         }
     }
-    __device__ __forceinline__ void store(float *s /* [BK][EXT+PAD] */) const
+    __device__ __forceinline__ void store(float *s /* [BK][EXT+PAD] */, bool full) const
     {
         const int t = threadIdx.x;
+        if (full) {
+#pragma unroll
+            for (int p = 0; p < VPER; ++p) {
+                if constexpr (K_CONTIG) {
+                    const int i = t / (BK / 4) + p * (1024 / BK), k = 4 * (t % (BK / 4));
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) s[(k + j) * (EXT + PAD) + i] = r[4 * p + j];
+                } else {
+                    const int k = t / (EXT / 4) + p * (1024 / EXT), i = 4 * (t % (EXT / 4));
+                    *reinterpret_cast<float4 *>(s + k * (EXT + PAD) + i) = make_float4(r[4 * p], r[4 * p + 1], r[4 * p + 2], r[4 * p + 3]);
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int p = 0; p < PER; ++p) {
             int k, i;
@@ -71,8 +107,8 @@ __global__ __launch_bounds__(256) void sgemm_mfma_kernel(int M, int N, int K, fl
     constexpr int WM = 4 / WN;         // wavefronts along m
     constexpr int TM = BM / WM / 32;   // 32x32 accumulators per wavefront along m (2 or 1)
     constexpr int TN = 2;              // and along n (64 columns per wavefront)
-    __shared__ float sA[2][BK * (BM + PAD)];
-    __shared__ float sB[2][BK * (BN + PAD)];
+    __shared__ __attribute__((aligned(16))) float sA[2][BK * (BM + PAD)];
+    __shared__ __attribute__((aligned(16))) float sB[2][BK * (BN + PAD)];
 
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const int kb = blockIdx.z * k_chunk;
@@ -91,36 +127,50 @@ __global__ __launch_bounds__(256) void sgemm_mfma_kernel(int M, int N, int K, fl
 
     TileLoader<BM, !TA> la;
     TileLoader<BN, TB> lb;
-    la.load(A, lda, m0, M, kb, ke);
-    lb.load(B, ldb, n0, N, kb, ke);
-    la.store(sA[0]);
-    lb.store(sB[0]);
+    const bool rows_inside = m0 + BM <= M, cols_inside = n0 + BN <= N;  // the tile's extent in m / n lies inside C
+    bool full = kb + BK <= ke;
+    la.load(A, lda, m0, M, kb, ke, full && rows_inside);
+    lb.load(B, ldb, n0, N, kb, ke, full && cols_inside);
+    la.store(sA[0], full && rows_inside);
+    lb.store(sB[0], full && cols_inside);
     __syncthreads();
 
     int buf = 0;
     for (int k0 = kb; k0 < ke; k0 += BK) {
         const bool more = k0 + BK < ke;
+        full = k0 + 2 * BK <= ke;
         if (more) {
-            la.load(A, lda, m0, M, k0 + BK, ke);
-            lb.load(B, ldb, n0, N, k0 + BK, ke);
+            la.load(A, lda, m0, M, k0 + BK, ke, full && rows_inside);
+            lb.load(B, ldb, n0, N, k0 + BK, ke, full && cols_inside);
         }
         const float *a = sA[buf], *b = sB[buf];
+        // Operands of step kk + 2 are read before the products of step kk are issued (the scheduling barriers keep
+        // the compiler from sinking the reads back to their use), so the LDS latency hides behind 4 MFMAs.
+        float av[2][TM], bv[2][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) av[0][i] = a[lk * (BM + PAD) + wm * (TM * 32) + i * 32 + lr];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bv[0][j] = b[lk * (BN + PAD) + wn * 64 + j * 32 + lr];
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 2) {
-            float av[TM], bv[TN];
+            const int cur = (kk / 2) & 1;
+            if (kk + 2 < BK) {
 #pragma unroll
-            for (int i = 0; i < TM; ++i) av[i] = a[(kk + lk) * (BM + PAD) + wm * (TM * 32) + i * 32 + lr];
+                for (int i = 0; i < TM; ++i) av[cur ^ 1][i] = a[(kk + 2 + lk) * (BM + PAD) + wm * (TM * 32) + i * 32 + lr];
 #pragma unroll
-            for (int j = 0; j < TN; ++j) bv[j] = b[(kk + lk) * (BN + PAD) + wn * 64 + j * 32 + lr];
+                for (int j = 0; j < TN; ++j) bv[cur ^ 1][j] = b[(kk + 2 + lk) * (BN + PAD) + wn * 64 + j * 32 + lr];
+            }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[cur][i], bv[cur][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
         if (more) {
-            la.store(sA[buf ^ 1]);
-            lb.store(sB[buf ^ 1]);
+            la.store(sA[buf ^ 1], full && rows_inside);
+            lb.store(sB[buf ^ 1], full && cols_inside);
         }
         __syncthreads();
         buf ^= 1;
