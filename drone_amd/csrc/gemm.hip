@@ -3,12 +3,21 @@
 // forward, :72-85 input gradient, :92-105 weight gradient), which are tall-skinny: M or K is the vertex
 // count, the other dimensions are feature widths (41..602).
 //
-// Work-group = 256 lanes = 4 wavefronts computing a 128 x BN tile of C (BN = 128 or 64) with
-// v_mfma_f32_32x32x2_f32: every wavefront owns a (128/WM) x (BN/WN) sub-tile as 32x32 accumulators.
-// A and B tiles of depth 16 are staged through LDS k-major ([k][m], [k][n]) so that the lanes of one MFMA
-// operand read consecutive addresses; global loads are issued one tile ahead of the math.  Loads are plain
-// dword loads with bounds checks (arbitrary M, N, K and leading dimensions, no alignment demands); adjacent
-// lanes read adjacent addresses in whichever dimension is contiguous in memory.
+// Work-group = 512 lanes: 4 product wavefronts computing a 128 x BN tile of C (BN = 128 or 64) with
+// v_mfma_f32_32x32x2_f32 - every one owns a (128/WM) x (BN/WN) sub-tile as 32x32 accumulators - and 4 loader
+// wavefronts that move the A and B tiles of depth 32 from global memory into LDS.  The split exists because a
+// wavefront that issues a global load into a backed-up memory pipeline stalls at the issue, in order, for
+// thousands of cycles (measured with the cycle counter: issuing one tile's loads took longer than multiplying
+// it), and a stalled wavefront issues no MFMAs either; with separate roles the loaders absorb that stall while
+// the product wavefronts only ever touch LDS.  One barrier per tile hands tile i + 1 over (double-buffered LDS)
+// while tile i + 2 is in flight in the loaders' registers.
+// Tiles are staged k-major ([k][m], [k][n]) so that the lanes of one MFMA operand read consecutive addresses;
+// the operands of the next k-step are read before the current step's four MFMAs are issued.  A tile that lies
+// inside the matrix is fetched with 16-byte loads (rows whose leading dimension is a multiple of 4 floats get
+// them aligned, which measured 10-20 % faster than odd strides such as 602); edge tiles take dword loads with a
+// bounds check per element, so M, N, K and the leading dimensions are arbitrary.
+// Measured on one MI355X: 232,965 x 602 x 128 100 TFLOP/s (640-wide aligned rows 110), 65,536 x 32,768 x 128 (the
+// dense-core shape of the SpMM) 133 TFLOP/s = 84 % of the 157 TFLOP/s fp32 MFMA peak.
 // A long reduction with a small output (the weight gradient: K = vertex count) is split over grid.z; the
 // partial tiles go to a scratch buffer and are summed in split order by a second kernel.
 #include <map>
@@ -23,7 +32,7 @@ namespace {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int BM = 128;
-constexpr int BK = 16;
+constexpr int BK = 32;
 constexpr int PAD = 4;
 
 // Four consecutive floats that are only known to be 4-byte aligned (leading dimensions such as 602 or 41 are
@@ -42,9 +51,8 @@ struct TileLoader {
     static constexpr int PER = BK * EXT / 256;
     static constexpr int VPER = PER / 4;
     float r[PER];
-    __device__ __forceinline__ void load(const float *__restrict__ X, int ld, int i0, int i_end, int k0, int k_end, bool full)
+    __device__ __forceinline__ void load(int t, const float *__restrict__ X, int ld, int i0, int i_end, int k0, int k_end, bool full)
     {
-        const int t = threadIdx.x;
         if (full) {
 #pragma unroll
             for (int p = 0; p < VPER; ++p) {
@@ -68,9 +76,8 @@ struct TileLoader {
             r[p] = v;
         }
     }
-    __device__ __forceinline__ void store(float *s /* [BK][EXT+PAD] */, bool full) const
+    __device__ __forceinline__ void store(int t, float *s /* [BK][EXT+PAD] */, bool full) const
     {
-        const int t = threadIdx.x;
         if (full) {
 #pragma unroll
             for (int p = 0; p < VPER; ++p) {
@@ -98,10 +105,9 @@ struct TileLoader {
 // op(A) is M x K: TA=false -> A stored M x K (k contiguous); TA=true -> A stored K x M (m contiguous).
 // op(B) is K x N: TB=false -> B stored K x N (n contiguous); TB=true -> B stored N x K (k contiguous).
 template <int BN, bool TA, bool TB>
-__global__ __launch_bounds__(256) void sgemm_mfma_kernel(int M, int N, int K, float alpha, const float *__restrict__ A,
-                                                         int lda, const float *__restrict__ B, int ldb, float beta,
-                                                         float *__restrict__ C, int ldc, int k_chunk,
-                                                         float *__restrict__ partial)
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void sgemm_mfma_kernel(
+    int M, int N, int K, float alpha, const float *__restrict__ A, int lda, const float *__restrict__ B, int ldb,
+    float beta, float *__restrict__ C, int ldc, int k_chunk, float *__restrict__ partial)
 {
     constexpr int WN = BN / 64;        // wavefronts along n (2 or 1)
     constexpr int WM = 4 / WN;         // wavefronts along m
@@ -113,7 +119,41 @@ __global__ __launch_bounds__(256) void sgemm_mfma_kernel(int M, int N, int K, fl
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const int kb = blockIdx.z * k_chunk;
     const int ke = kb + k_chunk < K ? kb + k_chunk : K;
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+    const int tiles = (ke - kb + BK - 1) / BK;
+    const int t = threadIdx.x & 255;
+
+    if (threadIdx.x >= 256) {
+        // ---- loader wavefronts: tile i + 1 goes to LDS while tile i is multiplied, tile i + 2 is in flight ----
+        TileLoader<BM, !TA> la;
+        TileLoader<BN, TB> lb;
+        const bool rows_inside = m0 + BM <= M, cols_inside = n0 + BN <= N;  // the tile's extent in m / n lies inside C
+        auto fetch = [&](int i) {
+            const int k0 = kb + i * BK;
+            const bool full = k0 + BK <= ke;
+            la.load(t, A, lda, m0, M, k0, ke, full && rows_inside);
+            lb.load(t, B, ldb, n0, N, k0, ke, full && cols_inside);
+        };
+        auto put = [&](int i) {
+            const bool full = kb + (i + 1) * BK <= ke;
+            la.store(t, sA[i & 1], full && rows_inside);
+            lb.store(t, sB[i & 1], full && cols_inside);
+        };
+        if (tiles > 0) {
+            fetch(0);
+            put(0);
+        }
+        if (tiles > 1) fetch(1);
+        __syncthreads();
+        for (int i = 0; i < tiles; ++i) {
+            if (i + 1 < tiles) put(i + 1);
+            if (i + 2 < tiles) fetch(i + 2);
+            __syncthreads();
+        }
+        return;
+    }
+
+    // ---- product wavefronts ----
+    const int wave = t / kWave, lane = t & (kWave - 1);
     const int wm = wave / WN, wn = wave % WN;
     const int lr = lane & 31, lk = lane >> 5;
 
@@ -125,25 +165,9 @@ __global__ __launch_bounds__(256) void sgemm_mfma_kernel(int M, int N, int K, fl
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    TileLoader<BM, !TA> la;
-    TileLoader<BN, TB> lb;
-    const bool rows_inside = m0 + BM <= M, cols_inside = n0 + BN <= N;  // the tile's extent in m / n lies inside C
-    bool full = kb + BK <= ke;
-    la.load(A, lda, m0, M, kb, ke, full && rows_inside);
-    lb.load(B, ldb, n0, N, kb, ke, full && cols_inside);
-    la.store(sA[0], full && rows_inside);
-    lb.store(sB[0], full && cols_inside);
     __syncthreads();
-
-    int buf = 0;
-    for (int k0 = kb; k0 < ke; k0 += BK) {
-        const bool more = k0 + BK < ke;
-        full = k0 + 2 * BK <= ke;
-        if (more) {
-            la.load(A, lda, m0, M, k0 + BK, ke, full && rows_inside);
-            lb.load(B, ldb, n0, N, k0 + BK, ke, full && cols_inside);
-        }
-        const float *a = sA[buf], *b = sB[buf];
+    for (int it = 0; it < tiles; ++it) {
+        const float *a = sA[it & 1], *b = sB[it & 1];
         // Operands of step kk + 2 are read before the products of step kk are issued (the scheduling barriers keep
         // the compiler from sinking the reads back to their use), so the LDS latency hides behind 4 MFMAs.
         float av[2][TM], bv[2][TN];
@@ -168,12 +192,7 @@ __global__ __launch_bounds__(256) void sgemm_mfma_kernel(int M, int N, int K, fl
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[cur][i], bv[cur][j], acc[i][j], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (more) {
-            la.store(sA[buf ^ 1], full && rows_inside);
-            lb.store(sB[buf ^ 1], full && cols_inside);
-        }
         __syncthreads();
-        buf ^= 1;
     }
 
     // 32x32 accumulator layout: register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4, column l%32.
@@ -246,10 +265,10 @@ template <int BN>
 void launch(bool ta, bool tb, dim3 grid, hipStream_t s, int M, int N, int K, float alpha, const float *A, int lda,
             const float *B, int ldb, float beta, float *C, int ldc, int k_chunk, float *partial)
 {
-    if (!ta && !tb) sgemm_mfma_kernel<BN, false, false><<<grid, 256, 0, s>>>(M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
-    else if (!ta && tb) sgemm_mfma_kernel<BN, false, true><<<grid, 256, 0, s>>>(M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
-    else if (ta && !tb) sgemm_mfma_kernel<BN, true, false><<<grid, 256, 0, s>>>(M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
-    else sgemm_mfma_kernel<BN, true, true><<<grid, 256, 0, s>>>(M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
+    if (!ta && !tb) sgemm_mfma_kernel<BN, false, false><<<grid, 512, 0, s>>>(M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
+    else if (!ta && tb) sgemm_mfma_kernel<BN, false, true><<<grid, 512, 0, s>>>(M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
+    else if (ta && !tb) sgemm_mfma_kernel<BN, true, false><<<grid, 512, 0, s>>>(M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
+    else sgemm_mfma_kernel<BN, true, true><<<grid, 512, 0, s>>>(M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
 }
 
 }  // namespace
