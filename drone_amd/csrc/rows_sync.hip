@@ -557,7 +557,7 @@ extern "C" int drone_graphsum_sync_rows_cached_f32(Graph *g, drone_row_cache *c,
     DRONE_REQUIRE(error_rate >= 0.0f, "error_rate is negative or not a number");
     if (mirror2master_recv) *mirror2master_recv = 0;
     if (master2mirror_recv) *master2mirror_recv = 0;
-    if (workerNum == 1 || c->size == 0) return DRONE_OK;  // nothing is replicated here
+    if (workerNum == 1) return DRONE_OK;  // nothing is replicated; with peers, a worker without replicas still meets them on the wire
     drone_transport *tr = static_cast<drone_transport *>(comm->comm);
     DRONE_REQUIRE(tr->exchange != nullptr, "the transport has no exchange entry");
     DRONE_HIP_TRY(hipSetDevice(g->GID));

@@ -4,11 +4,12 @@ Test helper only: the reference's partitioner (EBV) is a separate program."""
 import numpy as np
 
 
-def vertex_cut(u, v, W, seed=0):
+def vertex_cut(u, v, W, seed=0, owner=None):
+    """owner: worker of every edge (random when None)."""
     u = np.asarray(u, np.int64)
     v = np.asarray(v, np.int64)
     rng = np.random.default_rng(seed)
-    owner = rng.integers(0, W, len(u))
+    owner = rng.integers(0, W, len(u)) if owner is None else np.asarray(owner)
     edges = [(u[owner == w].astype(np.int32), v[owner == w].astype(np.int32)) for w in range(W)]
     holders = {}
     for w in range(W):

@@ -231,6 +231,56 @@ def test_row_cache_schedule_and_padded_rows(oracle):
         lb.close()
 
 
+@pytest.mark.parametrize("K", [1, 130])
+def test_row_cache_worker_without_replicas_and_odd_widths(oracle, K):
+    """Worker 2 holds a component of its own (no mirrors, no replicated masters: an empty cache) next to two workers
+    that share vertices; widths that are not a multiple of the wavefront."""
+    import torch
+    from drone_amd import gcn
+    from drone_amd.pagerank import Loopback, run_workers
+    from drone_amd.traverse import _WorkerCUDA
+    rng = np.random.default_rng(K)
+    n, W = 400, 3
+    ua, va = rng.integers(0, 300, 2000), rng.integers(0, 300, 2000)
+    ub, vb = rng.integers(300, 400, 300), rng.integers(300, 400, 300)
+    u, v = np.concatenate([ua, ub]).astype(np.int32), np.concatenate([va, vb]).astype(np.int32)
+    owner = np.concatenate([rng.integers(0, 2, len(ua)), np.full(len(ub), 2)])
+    parts, _ = vertex_cut(u, v, W, seed=1, owner=owner)
+    assert len(parts[2]["mirror_vertex"]) == 0 and len(parts[2]["master_vertex"]) == 0
+    tops = []
+    for p in parts:
+        nl, g2l, l2g, index, dst = oracle.build_graph(n, p["u"], p["v"])
+        tops.append(oracle.Part(l2g, n, p["master_vertex"], p["mirror_number"], p["mirror_workers"],
+                                p["mirror_vertex"], p["master_worker"]))
+    grp = oracle.RowCacheGroup(tops, K)
+    lb = Loopback(W, timeout_ms=60000)
+    ws = [_WorkerCUDA(n, p["u"], p["v"], workerId=i, workerNum=W, routes=p, loopback=lb) for i, p in enumerate(parts)]
+    caches = [gcn.RowCache(ws[i].g, i, W, ws[i].comm, K, compress=(K > 1)) for i in range(W)]
+    try:
+        assert caches[2].size == 0 and caches[0].size > 0
+        rows = [rng.standard_normal((t.n, K)).astype(np.float32) for t in tops]
+        for rate in (None, 0.1, 0.0, 0.4):
+            rows = [(r * (1 + 0.2 * rng.standard_normal((r.shape[0], 1)))).astype(np.float32) for r in rows]
+            host = [r.copy() for r in rows]
+            dev = [torch.from_numpy(r).cuda() for r in rows]
+            if rate is None:
+                want = grp.refresh(0, host, compress=(K > 1))
+                got = run_workers([(lambda i=i: caches[i].refresh(0, dev[i])) for i in range(W)])
+            else:
+                want = grp.sync(0, host, rate, compress=(K > 1))
+                got = run_workers([(lambda i=i: caches[i].sync(0, dev[i], rate)) for i in range(W)])
+            for i in range(W):
+                assert got[i] == (want[0][i], want[1][i])
+                np.testing.assert_array_equal(dev[i].cpu().numpy(), host[i])
+            np.testing.assert_array_equal(host[2], rows[2])          # the lone worker's rows never change
+    finally:
+        for c in caches:
+            c.close()
+        for w in ws:
+            lib_close(w)
+        lb.close()
+
+
 def test_row_cache_argument_checks(oracle):
     import ctypes as C
     import torch
