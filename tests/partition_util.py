@@ -35,6 +35,23 @@ def vertex_cut(u, v, W, seed=0, owner=None):
     return parts, master
 
 
+def lone_worker_cut(u, v, nglobal, W, seed=0):
+    """A cut in which the last worker holds a component of its own (no replicas at all): edges inside the upper
+    quarter of the id space go to it, edges inside the lower three quarters are spread over the others, edges
+    between the two are dropped.  Returns (u, v, parts)."""
+    u = np.asarray(u, np.int64)
+    v = np.asarray(v, np.int64)
+    h = nglobal * 3 // 4
+    low, high = (u < h) & (v < h), (u >= h) & (v >= h)
+    keep = low | high
+    rng = np.random.default_rng(seed)
+    owner = np.where(high, W - 1, rng.integers(0, W - 1, len(u)))[keep]
+    u, v = u[keep].astype(np.int32), v[keep].astype(np.int32)
+    parts, _ = vertex_cut(u, v, W, seed, owner=owner)
+    assert len(parts[-1]["mirror_vertex"]) == 0 and len(parts[-1]["master_vertex"]) == 0 and len(parts[-1]["u"]) > 0
+    return u, v, parts
+
+
 def write_partition_files(path, parts, out_degree):
     """G.<i>, Master.<i>, Mirror.<i>, out_degree.txt in the formats DRONE/src/graph/cuda_graph.go:15-164 reads."""
     for i, p in enumerate(parts):

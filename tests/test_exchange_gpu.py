@@ -4,7 +4,7 @@ single-subgraph run of the whole graph."""
 import numpy as np
 import pytest
 
-from partition_util import vertex_cut
+from partition_util import lone_worker_cut, vertex_cut
 
 pytestmark = pytest.mark.gpu
 
@@ -33,13 +33,18 @@ FIELDS = ["VisitedSize", "Mirror2MasterSendSize", "Mirror2MasterRecvSize", "Mast
           "Master2MirrorRecvSize"]
 
 
-@pytest.mark.parametrize("W,scale,seed", [(2, 8, 1), (3, 10, 2), (4, 12, 3), (7, 11, 4)])
-def test_pr_group_matches_oracle_group(oracle, W, scale, seed):
+@pytest.mark.parametrize("W,scale,seed,lone", [(2, 8, 1, False), (3, 10, 2, False), (4, 12, 3, False), (7, 11, 4, False),
+                                               (3, 10, 5, True)])
+def test_pr_group_matches_oracle_group(oracle, W, scale, seed, lone):
+    """lone: the last worker shares no vertex with the others and still has to meet them in every exchange."""
     from drone_amd.pagerank import Loopback, PRWorkerCUDA, run_workers
     nglobal = 1 << scale
     u, v = _graph(scale, 8, seed)
+    if lone:
+        u, v, parts = lone_worker_cut(u, v, nglobal, W, seed)
+    else:
+        parts, _ = vertex_cut(u, v, W, seed)
     outdeg = np.bincount(u, minlength=nglobal).astype(np.int32)
-    parts, _ = vertex_cut(u, v, W, seed)
     grp = _oracle_group(oracle, nglobal, parts, outdeg)
     lb = Loopback(W, timeout_ms=60000)
     ws = [PRWorkerCUDA(nglobal, p["u"], p["v"], outdeg, workerId=i, workerNum=W, routes=p, loopback=lb)

@@ -3,7 +3,7 @@ bit-exact labels and distances, the sign class of g->active, VisitedSize and the
 import numpy as np
 import pytest
 
-from partition_util import vertex_cut
+from partition_util import lone_worker_cut, vertex_cut
 
 pytestmark = pytest.mark.gpu
 
@@ -122,13 +122,17 @@ def _group(oracle, kind, nglobal, parts):
 
 
 @pytest.mark.parametrize("kind", ["cc", "sssp"])
-@pytest.mark.parametrize("W,scale,seed", [(2, 9, 1), (3, 12, 2), (5, 11, 3)])
-def test_group_matches_oracle_group(oracle, kind, W, scale, seed):
+@pytest.mark.parametrize("W,scale,seed,lone", [(2, 9, 1, False), (3, 12, 2, False), (5, 11, 3, False), (3, 10, 4, True)])
+def test_group_matches_oracle_group(oracle, kind, W, scale, seed, lone):
+    """lone: the last worker shares no vertex with the others and still has to meet them in every exchange."""
     from drone_amd.pagerank import Loopback, run_workers
     from drone_amd.traverse import CCWorkerCUDA, SSSPWorkerCUDA
     nglobal = 1 << scale
     u, v = _rmat(scale, 8, seed, symmetric=(kind == "cc"))
-    parts, _ = vertex_cut(u, v, W, seed)
+    if lone:
+        u, v, parts = lone_worker_cut(u, v, nglobal, W, seed)
+    else:
+        parts, _ = vertex_cut(u, v, W, seed)
     grp = _group(oracle, kind, nglobal, parts)
     start = int(u[0])
     lb = Loopback(W, timeout_ms=60000)
