@@ -24,15 +24,17 @@ struct PrF64Epi {
     double alpha, inv_n;
 
     __device__ __forceinline__ double load(int c, int64_t = 0) const { return c_in[c]; }
-    __device__ __forceinline__ void row(int r, double s, double &stat) const
+    // The row's inverse out-degree does not depend on the row sum: a kernel may fetch it long before it calls row().
+    __device__ __forceinline__ double row_operand(int r) const { return __builtin_nontemporal_load(inv + r); }
+    __device__ __forceinline__ void row(int r, double s, double iv, double &stat) const
     {
         const double base = (1.0 - alpha) * inv_n + alpha * dang[0] * inv_n;
         const double rn = base + alpha * s;
-        const double iv = __builtin_nontemporal_load(inv + r);
         c_out[r] = rn * iv;
         if (r_out) r_out[order[r]] = rn;
         if (iv == 0.0) stat += rn;
     }
+    __device__ __forceinline__ void row(int r, double s, double &stat) const { row(r, s, row_operand(r), stat); }
     __device__ __forceinline__ void fix(int r, double carry, double &stat) const
     {
         const double add = alpha * carry;

@@ -81,6 +81,10 @@ __device__ __forceinline__ double block_sum_1024(double v, double *s_red)
 // chunks of 1 K / 4 K / 16 K entries dealt round-robin to the wavefronts: 0.83 / 0.86 / 0.86; the same chunks with
 // every wavefront starting at a different place of the sweep: 0.76 / 0.74 / 0.77.  With slices a CU always runs a
 // mix of wavefronts that hit L1 (popular sources, the first slices) and wavefronts that miss (the cold tail).
+// Cycle counters inside the kernel (same graph): the 267 blocks of ~1 M entries take 66 % of the CU time and retire
+// one entry per clock per CU, the 1009 blocks of 16 K short rows (40 K entries each) the rest; the wavefronts of a
+// block finish within 10 % (dense blocks) to 50 % (short-row blocks) of each other.  More wavefronts per CU do not
+// help: blocks of 8,192 rows with two of them resident per CU measured 0.90 ms (1 M entries) and 0.99 ms (512 K).
 // Indices past the end of a slice are clamped to the block's last entry (gathered, then added as 0.0), which keeps
 // the loop free of divergent branches.
 template <bool kWide, typename Epi>
@@ -144,6 +148,15 @@ __global__ __launch_bounds__(kRbThreads) void pr_rowblock_kernel(const int32_t *
     const int64_t e0 = block_nnz[b], e1 = block_nnz[b + 1];
     const bool wide = block_wide[b] != 0;
     const int32_t *bases = batch_base + block_batch[b];
+    // The epilogue's per-row operand is fetched now and waits in registers: read after the sweep, one row at a
+    // time, it cost a memory latency per row (a quarter of the time of the blocks that hold many short rows).
+    constexpr int kEpiSlots = kRbRows / kRbThreads + 1;
+    double row_op[kEpiSlots];
+#pragma unroll
+    for (int k = 0; k < kEpiSlots; ++k) {
+        const int i = tid + k * kRbThreads;
+        row_op[k] = i < nr ? epi.row_operand(r0 + i) : 0.0;
+    }
     for (int i = tid; i <= nr; i += kRbThreads) s_acc[i] = 0.0;
     __syncthreads();
 
@@ -154,7 +167,11 @@ __global__ __launch_bounds__(kRbThreads) void pr_rowblock_kernel(const int32_t *
     __syncthreads();
 
     double stat = 0.0;
-    for (int i = tid; i < nr; i += kRbThreads) epi.row(r0 + i, s_acc[i], stat);
+#pragma unroll
+    for (int k = 0; k < kEpiSlots; ++k) {
+        const int i = tid + k * kRbThreads;
+        if (i < nr) epi.row(r0 + i, s_acc[i], row_op[k], stat);
+    }
     const double total = block_sum_1024(stat, s_red);
     if (tid == 0) {
         block_stat[b] = total;
