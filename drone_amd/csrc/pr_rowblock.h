@@ -2,7 +2,7 @@
 //
 // Why: an 8-byte gather costs a whole 128-byte line on its way from L2 (or beyond) to the CU, so the gather
 // stream is priced by distinct lines per unit time, not by bytes.  In row order, consecutive gathers hit
-// unrelated lines.  Here the rows are cut into blocks of at most kRbRows rows / kRbItems entries, and inside a
+// unrelated lines.  Here the rows are cut into blocks of at most kRbRows rows / `items` entries, and inside a
 // block the entries are sorted by source id once, at plan time.  A block then sweeps the source vector in
 // ascending order: the popular sources (which hot-first relabelling packs into few lines) are hit by adjacent
 // lanes and back-to-back instructions, so they are served by lane coalescing and L1 instead of L2, and the cold
@@ -11,7 +11,7 @@
 // block's rows with coalesced loads and stores.
 //
 // Blocks are equal shares of the weighted merge of {row ends (weight W)} and {entries (weight 1)}, W =
-// kRbItems / kRbRows, so a block never exceeds its row or entry capacity and empty-row runs and hub rows cost about
+// items / kRbRows, so a block never exceeds its row or entry capacity and empty-row runs and hub rows cost about
 // the same.  A row may straddle blocks: the block in which it ends applies the epilogue to its local part, the
 // parts in earlier blocks are written as carries and folded in by spmv_fixup_kernel (spmv_merge.h), exactly as
 // for the merge-path tiles.  The LDS additions are unordered, so the last bits of a sum can differ between runs
@@ -25,16 +25,17 @@ namespace drone {
 constexpr int kRbThreads = 1024;
 // Shape chosen by measurement on R-MAT scale 24 (ms per iteration, with the slice layout of rb_accumulate): 16,384
 // rows / 1 M entries 0.685; 16,384 / 512 K 0.72; 16,384 / 2 M 0.87 (too few heavy blocks for 256 CUs); 8,192 rows (two
-// blocks per CU) / 1 M 0.85, / 512 K 0.99.  Larger blocks reuse popular lines more often.
+// blocks per CU) / 1 M 0.85, / 512 K 0.99.  Larger blocks reuse popular lines more often, but the blocks that are
+// full of entries must still cover the CUs: the entry capacity is chosen per graph (row_blocks_create).
 constexpr int kRbRows = 16384;       // most rows ending in one block (LDS accumulators: 128 KB)
-constexpr int kRbItems = 1 << 20;    // most entries in one block
-constexpr int kRbWeight = kRbItems / kRbRows;
+constexpr int kRbMaxItems = 1 << 20; // most entries in one block (the plan picks a power of two up to this)
 constexpr int kRbUnroll = 4;
 constexpr int kRbLdsBytes = (kRbRows + 8) * (int)sizeof(double);  // rows ending in a block <= kRbRows + 1, + the open row
 
 struct RowBlocks {
     int64_t n = 0, nnz = 0;
     int num_blocks = 0;
+    int items = 0;                  // entry capacity of a block; a row end weighs items / kRbRows entries
     int32_t *block_row = nullptr;   // device [num_blocks + 1]: first row of the block
     int64_t *block_nnz = nullptr;   // device [num_blocks + 1]: first entry of the block
     int32_t *walk_len = nullptr;    // device [num_blocks]

@@ -7,10 +7,11 @@
 namespace drone {
 namespace {
 
-// Block b starts where the weighted merge path reaches b * kRbItems.  F(i) = W*i + row_ptr[i] is the path
+// Block b starts where the weighted merge path reaches b * kRbItems (the plan's entry capacity, W = its weight).  F(i) = W*i + row_ptr[i] is the path
 // position at which row i begins; inside row i the path first consumes its entries, then the row end (W).
 __global__ void rb_search_kernel(const int64_t *__restrict__ row_ptr, int64_t n, int64_t nnz, int num_blocks,
-                                 int32_t *__restrict__ block_row, int64_t *__restrict__ block_nnz)
+                                 int kRbItems, int kRbWeight, int32_t *__restrict__ block_row,
+                                 int64_t *__restrict__ block_nnz)
 {
     const int b = blockIdx.x * blockDim.x + threadIdx.x;
     if (b > num_blocks) return;
@@ -115,8 +116,18 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
     DRONE_REQUIRE(n > 0 && n < INT32_MAX && nnz >= 0 && nnz < (int64_t)UINT32_MAX, "sizes");
     rb->n = n;
     rb->nnz = nnz;
-    const int64_t total = (int64_t)kRbWeight * n + nnz;
-    rb->num_blocks = (int)ceil_div(total, kRbItems);
+    // Entry capacity of a block: the blocks that are full of entries should about match the number of CUs (one
+    // 1024-lane block is resident per CU, and such a block runs several times longer than a block of short rows),
+    // so the capacity follows the graph: the power of two nearest to nnz / CUs, between 32 K and kRbMaxItems.
+    int device = 0, cus = 256;
+    DRONE_HIP_TRY(hipGetDevice(&device));
+    DRONE_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+    int items = 32768;
+    while (items < kRbMaxItems && (double)items * 1.41421356 < (double)nnz / (cus > 0 ? cus : 256)) items <<= 1;
+    rb->items = items;
+    const int weight = items / kRbRows;
+    const int64_t total = (int64_t)weight * n + nnz;
+    rb->num_blocks = (int)ceil_div(total, items);
     const int nb = rb->num_blocks;
     uint64_t *keys = nullptr, *keys_sorted = nullptr;
     uint16_t *lrow_in = nullptr;
@@ -129,7 +140,7 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
         DRONE_HIP_TRY(hipMalloc(&rb->walk_len, sizeof(int32_t) * (size_t)nb));
         DRONE_HIP_TRY(hipMalloc(&rb->col, sizeof(int32_t) * e));
         DRONE_HIP_TRY(hipMalloc(&rb->lrow, sizeof(uint16_t) * e));
-        rb_search_kernel<<<(int)ceil_div(nb + 1, 256), 256, 0, stream>>>(row_ptr, n, nnz, nb, rb->block_row, rb->block_nnz);
+        rb_search_kernel<<<(int)ceil_div(nb + 1, 256), 256, 0, stream>>>(row_ptr, n, nnz, nb, items, weight, rb->block_row, rb->block_nnz);
         rb_walk_len_kernel<<<(int)ceil_div(nb, 256), 256, 0, stream>>>(row_ptr, nb, rb->block_row, rb->block_nnz, rb->walk_len);
         if (nnz > 0) {
             DRONE_HIP_TRY(hipMalloc(&keys, sizeof(uint64_t) * e));
