@@ -116,7 +116,7 @@ extern "C" int drone_pr_plan_create_ex(drone_pr_plan **out, int64_t n, int64_t n
     hipStream_t s = as_stream(stream);
     const auto build = [&]() -> int {
         DRONE_HIP_TRY(hipGetDevice(&p->device));
-        int rc = relabel_create(&p->rl, n, nnz, row_ptr, col_idx, s);
+        int rc = relabel_create(&p->rl, n, nnz, row_ptr, col_idx, inv_outdeg, s);
         if (rc != DRONE_OK) return rc;
         if (p->deterministic) {
             rc = merge_tiling_create<int64_t>(&p->mt, n, nnz, p->rl.row_ptr, kSpmvBlock * kPrIpt, s);

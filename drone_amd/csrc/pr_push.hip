@@ -353,6 +353,7 @@ extern "C" int drone_pr_run_graph_f64(Graph *g, PRValues *values, double alpha, 
         DRONE_HIP_TRY(hipMalloc(&x->inv64, sizeof(double) * (size_t)x->n));
         DRONE_HIP_TRY(hipMalloc(&x->rank64, sizeof(double) * (size_t)x->n));
         widen_row_ptr_kernel<<<1024, 256>>>(x->in_index, x->row_ptr64, x->n + 1);
+        inverse_out_degree_kernel<<<1024, 256>>>(values->outDegree, x->inv64, x->n);  // the plan orders vertices by it
         int rc = drone_pr_plan_create(&x->plan64, x->n, x->edges, x->row_ptr64, x->in_src, x->inv64, nullptr);
         if (rc != DRONE_OK) return rc;
     }

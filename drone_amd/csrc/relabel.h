@@ -17,9 +17,11 @@ struct Relabel {
     int32_t *col = nullptr;      // device [nnz]: relabelled sources, row order kept
 };
 
-// Builds the relabelled CSR from (row_ptr, col) on `stream`.  All temporaries are freed before return.
+// Builds the relabelled CSR from (row_ptr, col) on `stream`.  inv_outdeg (device [n], may be null): the vertices'
+// inverse out-degrees, 0 for none; when given, the gather counts are read off them instead of being counted.
+// All temporaries are freed before return.
 int relabel_create(Relabel *rl, int64_t n, int64_t nnz, const int64_t *row_ptr, const int32_t *col,
-                   hipStream_t stream);
+                   const double *inv_outdeg, hipStream_t stream);
 void relabel_destroy(Relabel *rl);
 
 // out[i] = in[order[i]]

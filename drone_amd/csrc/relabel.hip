@@ -7,10 +7,25 @@
 namespace drone {
 namespace {
 
+// How often every vertex is gathered: one atomic per entry (263 M entries: 25 ms, bound by the atomics on the
+// popular vertices) ...
 __global__ void count_sources_kernel(const int32_t *__restrict__ col, int64_t nnz, unsigned *__restrict__ count)
 {
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < nnz; e += (int64_t)gridDim.x * blockDim.x)
         atomicAdd(&count[col[e]], 1u);
+}
+
+// ... or, when the caller's inverse out-degrees are at hand, read off them: a vertex is gathered once per
+// out-edge.  The counts only order the vertices, so degrees that do not match the matrix cost speed, not results.
+// (Counting a sample of the entries instead was tried: the order of the mid-degree vertices got noisy and the
+// aggregation kernel ran 20 % slower.)
+__global__ void count_from_inverse_kernel(const double *__restrict__ inv, int64_t n, unsigned *__restrict__ count)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        const double v = inv[i];
+        const double d = v > 0.0 ? 1.0 / v : 0.0;
+        count[i] = d >= 4294967295.0 ? 4294967295u : d >= 0.0 ? (unsigned)(d + 0.5) : 0u;  // NaN -> 0
+    }
 }
 
 __global__ void iota_kernel(int32_t *a, int64_t n)
@@ -29,34 +44,60 @@ __global__ void invert_and_lengths_kernel(const int32_t *__restrict__ order, con
     }
 }
 
-// One wavefront per 64 consecutive new rows: each lane copies its own row when it is short, rows longer
-// than kShort are then copied by the whole wavefront.
-constexpr int kShort = 32;
+// Fills the relabelled CSR by position: a work-group owns kRemapChunk consecutive entries of the new CSR (so a hub
+// row is shared by many work-groups and the stores are coalesced), finds the rows they belong to with two binary
+// searches, keeps those rows' new and old starts in LDS, and every position then finds its row by a search in LDS,
+// reads the old entry from that row's old place and translates it.  All positions are independent, so the two
+// dependent gathers (old entry, then its new id) of many positions overlap.  A chunk that spans more rows than
+// the LDS table holds (a long run of empty rows) searches the row starts in global memory instead.
+constexpr int kRemapChunk = 2048;
+constexpr int kRemapRows = 2048;
+__device__ __forceinline__ int64_t last_row_starting_at_or_before(const int64_t *__restrict__ starts, int64_t lo,
+                                                                  int64_t hi, int64_t p)
+{
+    while (lo < hi) {  // largest r in [lo, hi] with starts[r] <= p
+        const int64_t mid = (lo + hi + 1) >> 1;
+        if (starts[mid] <= p) lo = mid; else hi = mid - 1;
+    }
+    return lo;
+}
+
 __global__ __launch_bounds__(256) void remap_rows_kernel(const int32_t *__restrict__ order,
                                                          const int64_t *__restrict__ row_ptr,
                                                          const int32_t *__restrict__ col,
                                                          const int32_t *__restrict__ new_id,
                                                          const int64_t *__restrict__ new_row_ptr, int64_t n,
-                                                         int32_t *__restrict__ new_col)
+                                                         int64_t nnz, int32_t *__restrict__ new_col)
 {
-    const int lane = threadIdx.x & (kWave - 1);
-    const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
-    const int64_t i = wave * kWave + lane;
-    int64_t src = 0, dst = 0, len = 0;
-    if (i < n) {
-        const int32_t o = order[i];
-        src = row_ptr[o];
-        len = row_ptr[o + 1] - src;
-        dst = new_row_ptr[i];
+    __shared__ int64_t s_dst[kRemapRows + 1];
+    __shared__ int64_t s_src[kRemapRows];
+    __shared__ int64_t s_range[2];
+    const int64_t p0 = (int64_t)blockIdx.x * kRemapChunk;
+    const int64_t p1 = p0 + kRemapChunk < nnz ? p0 + kRemapChunk : nnz;
+    if (threadIdx.x == 0) s_range[0] = last_row_starting_at_or_before(new_row_ptr, 0, n - 1, p0);
+    if (threadIdx.x == kWave) s_range[1] = last_row_starting_at_or_before(new_row_ptr, 0, n - 1, p1 - 1);
+    __syncthreads();
+    const int64_t ra = s_range[0], rb = s_range[1];
+    const int rows = (int)(rb - ra + 1 <= kRemapRows ? rb - ra + 1 : 0);  // 0: the table does not fit
+    for (int r = threadIdx.x; r < rows; r += blockDim.x) {
+        s_dst[r] = new_row_ptr[ra + r];
+        s_src[r] = row_ptr[order[ra + r]];
     }
-    if (len <= kShort)
-        for (int64_t k = 0; k < len; ++k) new_col[dst + k] = new_id[col[src + k]];
-    unsigned long long longs = __ballot(len > kShort);
-    while (longs) {
-        const int l = __ffsll((long long)longs) - 1;
-        longs &= longs - 1;
-        const int64_t s = __shfl(src, l, kWave), d = __shfl(dst, l, kWave), m = __shfl(len, l, kWave);
-        for (int64_t k = lane; k < m; k += kWave) new_col[d + k] = new_id[col[s + k]];
+    __syncthreads();
+    for (int64_t p = p0 + threadIdx.x; p < p1; p += blockDim.x) {
+        int64_t src;
+        if (rows > 0) {
+            int lo = 0, hi = rows - 1;
+            while (lo < hi) {
+                const int mid = (lo + hi + 1) >> 1;
+                if (s_dst[mid] <= p) lo = mid; else hi = mid - 1;
+            }
+            src = s_src[lo] + (p - s_dst[lo]);
+        } else {
+            const int64_t r = last_row_starting_at_or_before(new_row_ptr, ra, rb, p);
+            src = row_ptr[order[r]] + (p - new_row_ptr[r]);
+        }
+        new_col[p] = new_id[col[src]];
     }
 }
 
@@ -79,7 +120,7 @@ __global__ void gather_f64_kernel(const int32_t *__restrict__ order, const doubl
 }  // namespace
 
 int relabel_create(Relabel *rl, int64_t n, int64_t nnz, const int64_t *row_ptr, const int32_t *col,
-                   hipStream_t stream)
+                   const double *inv_outdeg, hipStream_t stream)
 {
     int rc = DRONE_OK;
     unsigned *count = nullptr, *count_sorted = nullptr;
@@ -100,7 +141,8 @@ int relabel_create(Relabel *rl, int64_t n, int64_t nnz, const int64_t *row_ptr, 
     RL_TRY(hipMalloc(&len, sizeof(int64_t) * ((size_t)n + 1)));
     RL_TRY(hipMemsetAsync(count, 0, sizeof(unsigned) * (size_t)n, stream));
     RL_TRY(hipMemsetAsync(len + n, 0, sizeof(int64_t), stream));
-    if (nnz) count_sources_kernel<<<blocks, threads, 0, stream>>>(col, nnz, count);
+    if (inv_outdeg) count_from_inverse_kernel<<<blocks, threads, 0, stream>>>(inv_outdeg, n, count);
+    else if (nnz) count_sources_kernel<<<blocks, threads, 0, stream>>>(col, nnz, count);
     iota_kernel<<<blocks, threads, 0, stream>>>(ids, n);
     // stable descending sort by gather count: order[new] = old
     RL_TRY(rocprim::radix_sort_pairs_desc(nullptr, temp_bytes, count, count_sorted, ids, rl->order, (size_t)n, 0, 32,
@@ -114,8 +156,9 @@ int relabel_create(Relabel *rl, int64_t n, int64_t nnz, const int64_t *row_ptr, 
     invert_and_lengths_kernel<<<blocks, threads, 0, stream>>>(rl->order, row_ptr, n, new_id, len);
     RL_TRY(rocprim::exclusive_scan(temp, temp_bytes, len, rl->row_ptr, (int64_t)0, (size_t)n + 1,
                                    rocprim::plus<int64_t>(), stream));
-    remap_rows_kernel<<<(int)ceil_div(n, 256), 256, 0, stream>>>(rl->order, row_ptr, col, new_id, rl->row_ptr, n,
-                                                               rl->col);
+    if (nnz > 0)
+        remap_rows_kernel<<<(int)ceil_div(nnz, kRemapChunk), 256, 0, stream>>>(rl->order, row_ptr, col, new_id, rl->row_ptr, n,
+                                                                              nnz, rl->col);
     RL_TRY(hipGetLastError());
     RL_TRY(hipStreamSynchronize(stream));
 done:

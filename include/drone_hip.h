@@ -124,7 +124,9 @@ typedef struct drone_pr_plan drone_pr_plan;
 /* Builds, once per CSR: a hot-first relabelled copy of the CSR (vertices sorted by how often they
  * are gathered, so that popular sources share cache lines), its merge-path tiling, and the work
  * vectors - the only allocations of this path.  row_ptr [n+1] and col_idx [nnz] are read during this
- * call only; inv_outdeg [n] is re-read at the start of every run and must outlive the plan.
+ * call only; inv_outdeg [n] is re-read at the start of every run and must outlive the plan.  It is
+ * also read here: a vertex is gathered once per out-edge, so the vertex order is taken from the
+ * out-degrees that inv_outdeg implies (values that do not match the CSR cost speed, never results).
  * Results are returned in the caller's vertex order. */
 int drone_pr_plan_create(drone_pr_plan **plan, int64_t n, int64_t nnz, const int64_t *row_ptr,
                          const int32_t *col_idx, const double *inv_outdeg, drone_stream_t stream);
