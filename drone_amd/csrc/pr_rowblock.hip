@@ -57,55 +57,64 @@ __global__ void rb_walk_len_kernel(const int64_t *__restrict__ row_ptr, int num_
     walk_len[b] = wl;
 }
 
-// One work-group per block: key = (block << 32) | source, value = row relative to the block's first row.
-__global__ __launch_bounds__(256) void rb_keys_kernel(const int64_t *__restrict__ row_ptr, const int32_t *__restrict__ col,
-                                                      const int32_t *__restrict__ block_row,
-                                                      const int64_t *__restrict__ block_nnz,
-                                                      uint64_t *__restrict__ keys, uint16_t *__restrict__ lrow)
+// One work-group per block: key = (block << 32) | source, value = row relative to the block's first row.  The
+// block's row starts (relative to its first entry, so 32 bits) sit in LDS for the per-entry binary search.
+constexpr int kKeysThreads = 1024;
+__global__ __launch_bounds__(kKeysThreads) void rb_keys_kernel(const int64_t *__restrict__ row_ptr,
+                                                               const int32_t *__restrict__ col,
+                                                               const int32_t *__restrict__ block_row,
+                                                               const int64_t *__restrict__ block_nnz,
+                                                               uint64_t *__restrict__ keys, uint16_t *__restrict__ lrow)
 {
+    __shared__ int32_t s_start[kRbRows + 2];  // row r0 + i starts at entry e0 + s_start[i] (clamped to the block)
     const int b = blockIdx.x;
     const int r0 = block_row[b], r1 = block_row[b + 1];
     const int64_t e0 = block_nnz[b], e1 = block_nnz[b + 1];
-    for (int64_t e = e0 + threadIdx.x; e < e1; e += blockDim.x) {
-        int lo = r0, hi = r1;  // largest r in [r0, r1] with row_ptr[r] <= e
+    const int rows = r1 - r0 + 1;  // rows r0 .. r1 may own entries of the block (r1: the row left open)
+    for (int i = threadIdx.x; i < rows; i += kKeysThreads) {
+        const int64_t st = row_ptr[r0 + i] - e0;
+        s_start[i] = st < 0 ? 0 : st > e1 - e0 ? (int32_t)(e1 - e0) : (int32_t)st;
+    }
+    __syncthreads();
+    for (int64_t e = e0 + threadIdx.x; e < e1; e += kKeysThreads) {
+        const int32_t off = (int32_t)(e - e0);
+        int lo = 0, hi = rows - 1;  // largest i with s_start[i] <= off
         while (lo < hi) {
             const int mid = (lo + hi + 1) >> 1;
-            if (row_ptr[mid] <= e) lo = mid; else hi = mid - 1;
+            if (s_start[mid] <= off) lo = mid; else hi = mid - 1;
         }
         keys[e] = ((uint64_t)b << 32) | (uint32_t)col[e];
-        lrow[e] = (uint16_t)(lo - r0);
+        lrow[e] = (uint16_t)lo;
     }
 }
 
-// One thread per 64-entry batch: base = first source of the batch, packed = lrow << 16 | (source - base);
-// a batch that spans more than 65,535 ids flags its block as wide.
-__global__ void rb_pack_kernel(int num_blocks, const int64_t *__restrict__ block_nnz, const int32_t *__restrict__ block_batch,
-                               const int32_t *__restrict__ col, const uint16_t *__restrict__ lrow,
-                               uint32_t *__restrict__ packed, int32_t *__restrict__ batch_base,
-                               int32_t *__restrict__ block_wide)
+// One lane per entry, one wavefront per 64-entry batch of a block's sorted entries: col = the key's source,
+// base = first source of the batch, packed = lrow << 16 | (source - base); a batch that spans more than 65,535 ids
+// flags its block as wide.
+__global__ __launch_bounds__(1024) void rb_pack_kernel(const int64_t *__restrict__ block_nnz,
+                                                       const int32_t *__restrict__ block_batch,
+                                                       const uint64_t *__restrict__ keys_sorted,
+                                                       const uint16_t *__restrict__ lrow, int32_t *__restrict__ col,
+                                                       uint32_t *__restrict__ packed, int32_t *__restrict__ batch_base,
+                                                       int32_t *__restrict__ block_wide)
 {
     const int b = blockIdx.x;
     const int64_t e0 = block_nnz[b], e1 = block_nnz[b + 1];
-    const int batches = block_batch[b + 1] - block_batch[b];
-    for (int j = threadIdx.x; j < batches; j += blockDim.x) {
-        const int64_t s = e0 + (int64_t)j * 64;
-        const int64_t t = s + 64 < e1 ? s + 64 : e1;
-        const int32_t base = col[s];
-        batch_base[block_batch[b] + j] = base;
-        bool overflow = false;
-        for (int64_t e = s; e < t; ++e) {
-            const int32_t off = col[e] - base;  // sources ascend inside a block
-            if (off > 0xFFFF) overflow = true;
+    const int lane = threadIdx.x & (kWave - 1);
+    bool overflow = false;
+    for (int64_t s = e0 + (int64_t)(threadIdx.x - lane); s < e1; s += blockDim.x) {  // s: start of this wavefront's batch
+        const int64_t e = s + lane;
+        const int32_t c = e < e1 ? (int32_t)(keys_sorted[e] & 0xFFFFFFFFull) : 0;
+        const int32_t base = __shfl(c, 0, kWave);  // sources ascend inside a block
+        if (e < e1) {
+            const int32_t off = c - base;
+            overflow |= off > 0xFFFF;
+            col[e] = c;
             packed[e] = ((uint32_t)lrow[e] << 16) | (uint32_t)(off & 0xFFFF);
         }
-        if (overflow) block_wide[b] = 1;
+        if (lane == 0) batch_base[block_batch[b] + (int32_t)((s - e0) >> 6)] = base;
     }
-}
-
-__global__ void rb_unpack_kernel(const uint64_t *__restrict__ keys, int64_t nnz, int32_t *__restrict__ col)
-{
-    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < nnz; e += (int64_t)gridDim.x * blockDim.x)
-        col[e] = (int32_t)(keys[e] & 0xFFFFFFFFull);
+    if (__any(overflow) && lane == 0) block_wide[b] = 1;
 }
 
 }  // namespace
@@ -146,13 +155,12 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
             DRONE_HIP_TRY(hipMalloc(&keys, sizeof(uint64_t) * e));
             DRONE_HIP_TRY(hipMalloc(&keys_sorted, sizeof(uint64_t) * e));
             DRONE_HIP_TRY(hipMalloc(&lrow_in, sizeof(uint16_t) * e));
-            rb_keys_kernel<<<nb, 256, 0, stream>>>(row_ptr, col, rb->block_row, rb->block_nnz, keys, lrow_in);
+            rb_keys_kernel<<<nb, kKeysThreads, 0, stream>>>(row_ptr, col, rb->block_row, rb->block_nnz, keys, lrow_in);
             int bits = 32;
             while (bits < 64 && (1ull << (bits - 32)) < (unsigned long long)nb) ++bits;
             DRONE_HIP_TRY(rocprim::radix_sort_pairs(nullptr, temp_bytes, keys, keys_sorted, lrow_in, rb->lrow, (size_t)nnz, 0, bits, stream));
             DRONE_HIP_TRY(hipMalloc(&temp, temp_bytes ? temp_bytes : 1));
             DRONE_HIP_TRY(rocprim::radix_sort_pairs(temp, temp_bytes, keys, keys_sorted, lrow_in, rb->lrow, (size_t)nnz, 0, bits, stream));
-            rb_unpack_kernel<<<4096, 256, 0, stream>>>(keys_sorted, nnz, rb->col);
         }
         // packed 4-byte entries
         DRONE_HIP_TRY(hipMalloc(&rb->block_batch, sizeof(int32_t) * ((size_t)nb + 1)));
@@ -167,8 +175,8 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
         DRONE_HIP_TRY(hipMalloc(&rb->batch_base, sizeof(int32_t) * (size_t)(h_batch[nb] ? h_batch[nb] : 1)));
         DRONE_HIP_TRY(hipMemcpyAsync(rb->block_batch, h_batch.data(), sizeof(int32_t) * h_batch.size(), hipMemcpyHostToDevice, stream));
         if (nnz > 0)
-            rb_pack_kernel<<<nb, 256, 0, stream>>>(nb, rb->block_nnz, rb->block_batch, rb->col, rb->lrow, rb->packed,
-                                                  rb->batch_base, rb->block_wide);
+            rb_pack_kernel<<<nb, 1024, 0, stream>>>(rb->block_nnz, rb->block_batch, keys_sorted, rb->lrow, rb->col, rb->packed,
+                                                   rb->batch_base, rb->block_wide);
         DRONE_HIP_TRY(hipGetLastError());
         DRONE_HIP_TRY(hipStreamSynchronize(stream));
         return DRONE_OK;
