@@ -201,6 +201,41 @@ def test_build_graph_matches_reference_layout(torch_cuda, oracle, seed):
     w.close()
 
 
+@pytest.mark.parametrize("name", ["multigraph", "one_edge", "no_edges", "descending_ids", "rmat18"])
+def test_build_graph_layout_stress(torch_cuda, oracle, name):
+    """Repeated edges, self-loops, ids that are never used, a single edge, no edge at all, ids first seen in
+    descending order, and a 4 M-edge list: the local ids, both maps and the out-edge CSR equal the host walk."""
+    from drone_amd import rmat
+    from drone_amd.pagerank import PRWorkerCUDA
+    rng = np.random.default_rng(7)
+    if name == "multigraph":
+        gN = 50000
+        u = rng.integers(0, 3000, 400000).astype(np.int32) * 7 % gN
+        v = rng.integers(0, 3000, 400000).astype(np.int32) * 11 % gN
+        u[::17] = v[::17]                                    # self-loops
+    elif name == "one_edge":
+        gN, u, v = 10, np.array([7], np.int32), np.array([7], np.int32)
+    elif name == "no_edges":
+        gN, u, v = 10, np.zeros(0, np.int32), np.zeros(0, np.int32)
+    elif name == "descending_ids":
+        gN = 4096
+        u = np.arange(gN - 1, 0, -1, dtype=np.int32)
+        v = u - 1
+    else:
+        gN = 1 << 18
+        s, d = rmat.rmat_edges(18, 16 << 18, seed=9)
+        u, v = s.astype(np.int32), d.astype(np.int32)        # raw generator output: duplicates and self-loops included
+    w = PRWorkerCUDA(gN, u, v)
+    n, g2l, l2g, index, dst = oracle.build_graph(gN, u, v)
+    got = w.graph_arrays()
+    assert w.n == n
+    np.testing.assert_array_equal(got["Global2Local"], g2l)
+    np.testing.assert_array_equal(got["Local2Global"], l2g)
+    np.testing.assert_array_equal(got["index"], index)
+    np.testing.assert_array_equal(got["dst"], dst)
+    w.close()
+
+
 @pytest.mark.parametrize("seed,scale", [(1, 10), (3, 13)])
 def test_peval_inceval_against_push_oracle(torch_cuda, oracle, seed, scale):
     from drone_amd.pagerank import PRWorkerCUDA
