@@ -107,7 +107,8 @@ extern "C" int drone_pr_plan_create_ex(drone_pr_plan **out, int64_t n, int64_t n
     DRONE_REQUIRE(n > 0 && n < INT32_MAX, "vertex count must be in [1, 2^31-2]");
     DRONE_REQUIRE(nnz >= 0, "nnz");
     DRONE_REQUIRE(row_ptr && inv_outdeg && (col_idx || nnz == 0), "null CSR array");
-    DRONE_REQUIRE((flags & ~DRONE_PR_DETERMINISTIC) == 0, "unknown flag");
+    DRONE_REQUIRE((flags & ~(DRONE_PR_DETERMINISTIC | DRONE_PR_SHARED_BLOCKS | DRONE_PR_WHOLE_BLOCKS)) == 0, "unknown flag");
+    DRONE_REQUIRE(!((flags & DRONE_PR_SHARED_BLOCKS) && (flags & DRONE_PR_WHOLE_BLOCKS)), "contradicting flags");
     drone_pr_plan *p = new drone_pr_plan();
     p->deterministic = (flags & DRONE_PR_DETERMINISTIC) != 0 || nnz >= (int64_t)UINT32_MAX;
     p->n = n;
@@ -123,7 +124,8 @@ extern "C" int drone_pr_plan_create_ex(drone_pr_plan **out, int64_t n, int64_t n
             if (rc != DRONE_OK) return rc;
             p->units = p->mt.num_tiles;
         } else {
-            rc = row_blocks_create(&p->rb, n, nnz, p->rl.row_ptr, p->rl.col, s);
+            rc = row_blocks_create(&p->rb, n, nnz, p->rl.row_ptr, p->rl.col,
+                                   (flags & DRONE_PR_SHARED_BLOCKS) ? 2 : (flags & DRONE_PR_WHOLE_BLOCKS) ? 1 : 0, s);
             if (rc != DRONE_OK) return rc;
             p->units = p->rb.num_blocks;
             // the row-ordered copy is only needed to build the blocks
@@ -261,9 +263,14 @@ extern "C" int drone_pr_run_f64(drone_pr_plan *p, double alpha, int iters, doubl
             spmv_merge_kernel<double, int64_t, kPrIpt, PrF64Epi><<<p->mt.num_tiles, kSpmvBlock, 0, s>>>(
                 p->n, p->nnz, p->mt.tile_row, p->rl.row_ptr, p->rl.col, epi, carry, p->ms.tile_stat);
         } else {
-            pr_rowblock_kernel<PrF64Epi><<<p->rb.num_blocks, kRbThreads, kRbLdsBytes, s>>>(
+            pr_rowblock_kernel<PrF64Epi><<<p->rb.num_units, kRbThreads, kRbLdsBytes, s>>>(
                 p->rb.block_row, p->rb.block_nnz, p->rb.col, p->rb.lrow, p->rb.packed, p->rb.batch_base, p->rb.block_batch,
-                p->rb.block_wide, epi, carry, p->ms.tile_stat);
+                p->rb.block_wide, p->rb.unit_block, p->rb.block_units, p->rb.block_unit0, p->rb.block_partial,
+                p->rb.partial, epi, carry, p->ms.tile_stat);
+            if (p->rb.num_split > 0)
+                pr_rowblock_merge_kernel<PrF64Epi><<<p->rb.num_split, kRbThreads, 0, s>>>(
+                    p->rb.split_block, p->rb.block_row, p->rb.block_units, p->rb.block_partial, p->rb.partial, epi, carry,
+                    p->ms.tile_stat);
         }
         if (prof) DRONE_HIP_TRY(hipEventRecord(p->ev1[p->prof_n++], s));
         spmv_fixup_kernel<double, PrF64Epi><<<fb, kSpmvBlock, 0, s>>>(

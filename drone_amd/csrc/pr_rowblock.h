@@ -30,6 +30,7 @@ constexpr int kRbThreads = 1024;
 constexpr int kRbRows = 16384;       // most rows ending in one block (LDS accumulators: 128 KB)
 constexpr int kRbMaxItems = 1 << 20; // most entries in one block (the plan picks a power of two up to this)
 constexpr int kRbUnroll = 4;
+constexpr int kRbSplit = 4;         // work-groups that share one block of a large matrix
 constexpr int kRbLdsBytes = (kRbRows + 8) * (int)sizeof(double);  // rows ending in a block <= kRbRows + 1, + the open row
 
 struct RowBlocks {
@@ -48,11 +49,25 @@ struct RowBlocks {
     int32_t *batch_base = nullptr;  // device [total batches]
     int32_t *block_batch = nullptr; // device [num_blocks + 1]: first batch of the block
     int32_t *block_wide = nullptr;  // device [num_blocks]
+    // Work units.  A block with many entries is swept by several work-groups, each taking every shares-th slice of
+    // its sorted entries; they leave their row sums in `partial`, and a second kernel adds them up and runs the
+    // epilogue.  Such a block holds kRbSplit times the entries one work-group handles, so the same number of
+    // work-groups finds more entries per source line (R-MAT scale 24: 33.7 M distinct (block, line) pairs with 1 M
+    // entries per block, 14.9 M with 4 M), and every work-group still sweeps hot and cold slices side by side.
+    int num_units = 0;
+    int32_t *unit_block = nullptr;   // device [num_units]
+    int32_t *block_units = nullptr;  // device [num_blocks]: work-groups that share the block (1: the block is not split)
+    int32_t *block_unit0 = nullptr;  // device [num_blocks]: the block's first unit
+    int64_t *block_partial = nullptr;// device [num_blocks]: where the block's shares start in `partial` (in doubles)
+    int num_split = 0;
+    int32_t *split_block = nullptr;  // device [num_split]: the blocks with more than one unit
+    double *partial = nullptr;       // device: per split block, block_units x (rows + 1) row sums
 };
 
 // Builds the blocks for a CSR with device row_ptr / col (already in the plan's internal id space).
+// shared_blocks: 0 = decide by size, 1 = never split a block, 2 = split whenever a block is large enough.
 int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_ptr, const int32_t *col,
-                      hipStream_t stream);
+                      int shared_blocks, hipStream_t stream);
 void row_blocks_destroy(RowBlocks *rb);
 
 __device__ __forceinline__ int64_t ceil_div_dev(int64_t a, int64_t b) { return (a + b - 1) / b; }
@@ -93,17 +108,23 @@ __device__ __forceinline__ double block_sum_1024(double v, double *s_red)
 // Indices past the end of a slice are clamped to the block's last entry (gathered, then added as 0.0), which keeps
 // the loop free of divergent branches.
 template <bool kWide, typename Epi>
-__device__ __forceinline__ void rb_accumulate(int64_t e0, int64_t e1, int tid, const int32_t *__restrict__ col,
-                                              const uint16_t *__restrict__ lrow, const uint32_t *__restrict__ packed,
-                                              const int32_t *__restrict__ bases, const Epi &epi, double *s_acc)
+__device__ __forceinline__ void rb_accumulate(int64_t block_begin, int64_t block_end, int share, int shares, int tid,
+                                              const int32_t *__restrict__ col, const uint16_t *__restrict__ lrow,
+                                              const uint32_t *__restrict__ packed, const int32_t *__restrict__ bases,
+                                              const Epi &epi, double *s_acc)
 {
-    if (e0 >= e1) return;
+    // The block's sorted entries [block_begin, block_end) are cut into 16 * shares slices of whole 64-entry batches;
+    // wavefront w of share k sweeps slice w * shares + k, so every work-group of a split block gets the same mix of
+    // popular (L1-hitting) and cold (missing) slices that an unsplit block has.
     constexpr int kWaves = kRbThreads / kWave;
     const int lane = tid & (kWave - 1), wave = tid / kWave;
-    const int64_t slice = ceil_div_dev(e1 - e0, (int64_t)kWaves * kWave) * kWave;  // a multiple of 64: batches stay whole
-    const int64_t s0 = e0 + wave * slice;
-    const int64_t s1 = s0 + slice < e1 ? s0 + slice : e1;
-    const int64_t last = e1 - 1;
+    const int64_t batches = ceil_div_dev(block_end - block_begin, (int64_t)kWave);
+    const int64_t slices = (int64_t)kWaves * shares, mine = (int64_t)wave * shares + share;
+    const int64_t s0 = block_begin + batches * mine / slices * kWave;
+    int64_t s1 = block_begin + batches * (mine + 1) / slices * kWave;
+    if (s1 > block_end) s1 = block_end;
+    if (s0 >= s1) return;
+    const int64_t last = block_end - 1;
     for (int64_t base = s0; base < s1; base += kWave * kRbUnroll) {
         uint32_t a[kRbUnroll];
         int32_t g[kRbUnroll];
@@ -116,7 +137,7 @@ __device__ __forceinline__ void rb_accumulate(int64_t e0, int64_t e1, int tid, c
                 g[k] = (int32_t)__builtin_nontemporal_load(lrow + e);
             } else {
                 a[k] = __builtin_nontemporal_load(packed + e);
-                g[k] = bases[(e - e0) >> 6];  // same address for all lanes of a wavefront
+                g[k] = bases[(e - block_begin) >> 6];  // same address for all lanes of a wavefront
             }
         }
         int c[kRbUnroll], l[kRbUnroll];
@@ -142,34 +163,55 @@ __global__ __launch_bounds__(kRbThreads) void pr_rowblock_kernel(const int32_t *
                                                                  const uint32_t *__restrict__ packed,
                                                                  const int32_t *__restrict__ batch_base,
                                                                  const int32_t *__restrict__ block_batch,
-                                                                 const int32_t *__restrict__ block_wide, Epi epi,
+                                                                 const int32_t *__restrict__ block_wide,
+                                                                 const int32_t *__restrict__ unit_block,
+                                                                 const int32_t *__restrict__ block_units,
+                                                                 const int32_t *__restrict__ block_unit0,
+                                                                 const int64_t *__restrict__ block_partial,
+                                                                 double *__restrict__ partial, Epi epi,
                                                                  double *__restrict__ block_carry,
                                                                  double *__restrict__ block_stat)
 {
     extern __shared__ double s_acc[];  // [rows ending in the block + 1 (the row left open)]
     __shared__ double s_red[kRbThreads / kWave];
-    const int b = blockIdx.x, tid = threadIdx.x;
+    const int u = blockIdx.x, tid = threadIdx.x;
+    const int b = unit_block[u];
     const int r0 = block_row[b], nr = block_row[b + 1] - r0;
-    const int64_t e0 = block_nnz[b], e1 = block_nnz[b + 1];
+    const int64_t eb = block_nnz[b], ee = block_nnz[b + 1];
+    const int shares = block_units[b];
+    const int share = u - block_unit0[b];
     const bool wide = block_wide[b] != 0;
     const int32_t *bases = batch_base + block_batch[b];
-    // The epilogue's per-row operand is fetched now and waits in registers: read after the sweep, one row at a
-    // time, it cost a memory latency per row (a quarter of the time of the blocks that hold many short rows).
+    // An unsplit block fetches the epilogue's per-row operand now and lets it wait in registers: read after the
+    // sweep, one row at a time, it cost a memory latency per row (a quarter of the time of the blocks that hold
+    // many short rows).  Split blocks hold few rows; the work-group that ends up with the epilogue reads them then.
     constexpr int kEpiSlots = kRbRows / kRbThreads + 1;
     double row_op[kEpiSlots];
+    if (shares == 1) {
 #pragma unroll
-    for (int k = 0; k < kEpiSlots; ++k) {
-        const int i = tid + k * kRbThreads;
-        row_op[k] = i < nr ? epi.row_operand(r0 + i) : 0.0;
+        for (int k = 0; k < kEpiSlots; ++k) {
+            const int i = tid + k * kRbThreads;
+            row_op[k] = i < nr ? epi.row_operand(r0 + i) : 0.0;
+        }
     }
     for (int i = tid; i <= nr; i += kRbThreads) s_acc[i] = 0.0;
     __syncthreads();
 
     if (wide)
-        rb_accumulate<true>(e0, e1, tid, col, lrow, packed, bases, epi, s_acc);
+        rb_accumulate<true>(eb, ee, share, shares, tid, col, lrow, packed, bases, epi, s_acc);
     else
-        rb_accumulate<false>(e0, e1, tid, col, lrow, packed, bases, epi, s_acc);
+        rb_accumulate<false>(eb, ee, share, shares, tid, col, lrow, packed, bases, epi, s_acc);
     __syncthreads();
+
+    if (shares > 1) {
+        // leave the sums in the block's area: pr_rowblock_merge_kernel adds the shares up and runs the epilogue.
+        // (Letting the work-group that arrives last do that inside this kernel needs device-scope fences, and on a
+        // GPU whose XCDs have separate L2s every such fence writes back and invalidates a whole L2: 0.99 ms
+        // instead of 0.68 with two shares per block.)
+        double *mine = partial + block_partial[b] + (int64_t)share * (nr + 1);
+        for (int i = tid; i <= nr; i += kRbThreads) mine[i] = s_acc[i];
+        return;
+    }
 
     double stat = 0.0;
 #pragma unroll
@@ -182,6 +224,31 @@ __global__ __launch_bounds__(kRbThreads) void pr_rowblock_kernel(const int32_t *
         block_stat[b] = total;
         block_carry[b] = s_acc[nr];
     }
+}
+
+// Split blocks: adds the shares of every row and runs the epilogue.  One work-group per split block.
+template <typename Epi>
+__global__ __launch_bounds__(kRbThreads) void pr_rowblock_merge_kernel(const int32_t *__restrict__ split_block,
+                                                                       const int32_t *__restrict__ block_row,
+                                                                       const int32_t *__restrict__ block_units,
+                                                                       const int64_t *__restrict__ block_partial,
+                                                                       const double *__restrict__ partial, Epi epi,
+                                                                       double *__restrict__ block_carry,
+                                                                       double *__restrict__ block_stat)
+{
+    __shared__ double s_red[kRbThreads / kWave];
+    const int b = split_block[blockIdx.x], tid = threadIdx.x;
+    const int r0 = block_row[b], nr = block_row[b + 1] - r0, shares = block_units[b];
+    const double *area = partial + block_partial[b];
+    double stat = 0.0;
+    for (int i = tid; i <= nr; i += kRbThreads) {
+        double sum = 0.0;
+        for (int sh = 0; sh < shares; ++sh) sum += area[(int64_t)sh * (nr + 1) + i];
+        if (i < nr) epi.row(r0 + i, sum, epi.row_operand(r0 + i), stat);
+        else block_carry[b] = sum;  // the row left open at the end of the block
+    }
+    const double total = block_sum_1024(stat, s_red);
+    if (tid == 0) block_stat[b] = total;
 }
 
 }  // namespace drone

@@ -120,7 +120,7 @@ __global__ __launch_bounds__(1024) void rb_pack_kernel(const int64_t *__restrict
 }  // namespace
 
 int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_ptr, const int32_t *col,
-                      hipStream_t stream)
+                      int shared_blocks, hipStream_t stream)
 {
     DRONE_REQUIRE(n > 0 && n < INT32_MAX && nnz >= 0 && nnz < (int64_t)UINT32_MAX, "sizes");
     rb->n = n;
@@ -133,6 +133,12 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
     DRONE_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
     int items = 32768;
     while (items < kRbMaxItems && (double)items * 1.41421356 < (double)nnz / (cus > 0 ? cus : 256)) items <<= 1;
+    const int unit_items = items;          // entries one work-group sweeps
+    // Large matrices get blocks that several work-groups share (measured, ms per iteration at R-MAT scale 20 / 22 /
+    // 24 with 1 / 2 / 4 / 8 / 16 work-groups per block: 0.060 0.063 0.079 0.081 0.087 / 0.175 0.181 0.172 0.216
+    // 0.184 / 0.679 0.649 0.617 0.659 0.670: small ones lose more to the second kernel than they gain).
+    const int split = shared_blocks == 1 ? 1 : (shared_blocks == 2 || nnz >= (int64_t)48 << 20) ? kRbSplit : 1;
+    items *= split;                        // entries one block holds
     rb->items = items;
     const int weight = items / kRbRows;
     const int64_t total = (int64_t)weight * n + nnz;
@@ -177,6 +183,45 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
         if (nnz > 0)
             rb_pack_kernel<<<nb, 1024, 0, stream>>>(rb->block_nnz, rb->block_batch, keys_sorted, rb->lrow, rb->col, rb->packed,
                                                    rb->batch_base, rb->block_wide);
+        // work units: a block is shared by as many work-groups as it holds unit_items entries (at most `split`)
+        std::vector<int32_t> h_row((size_t)nb + 1);
+        DRONE_HIP_TRY(hipMemcpyAsync(h_row.data(), rb->block_row, sizeof(int32_t) * h_row.size(), hipMemcpyDeviceToHost, stream));
+        DRONE_HIP_TRY(hipStreamSynchronize(stream));
+        std::vector<int32_t> h_unit_block, h_units((size_t)nb), h_unit0((size_t)nb);
+        std::vector<int64_t> h_partial((size_t)nb, 0);
+        int64_t partial_doubles = 0;
+        for (int b = 0; b < nb; ++b) {
+            const int64_t entries = h_nnz[b + 1] - h_nnz[b];
+            const int batches = h_batch[b + 1] - h_batch[b];
+            int shares = (int)ceil_div(entries, unit_items);
+            if (shares < 1) shares = 1;
+            if (shares > split) shares = split;
+            if (shares > batches && batches > 0) shares = batches;
+            h_units[b] = shares;
+            h_unit0[b] = (int32_t)h_unit_block.size();
+            for (int sh = 0; sh < shares; ++sh) h_unit_block.push_back(b);
+            if (shares > 1) {
+                h_partial[b] = partial_doubles;
+                partial_doubles += (int64_t)shares * (h_row[b + 1] - h_row[b] + 1);
+            }
+        }
+        rb->num_units = (int)h_unit_block.size();
+        DRONE_HIP_TRY(hipMalloc(&rb->unit_block, sizeof(int32_t) * h_unit_block.size()));
+        DRONE_HIP_TRY(hipMalloc(&rb->block_units, sizeof(int32_t) * (size_t)nb));
+        DRONE_HIP_TRY(hipMalloc(&rb->block_unit0, sizeof(int32_t) * (size_t)nb));
+        DRONE_HIP_TRY(hipMalloc(&rb->block_partial, sizeof(int64_t) * (size_t)nb));
+        DRONE_HIP_TRY(hipMalloc(&rb->partial, sizeof(double) * (size_t)(partial_doubles ? partial_doubles : 1)));
+        DRONE_HIP_TRY(hipMemcpyAsync(rb->unit_block, h_unit_block.data(), sizeof(int32_t) * h_unit_block.size(), hipMemcpyHostToDevice, stream));
+        DRONE_HIP_TRY(hipMemcpyAsync(rb->block_units, h_units.data(), sizeof(int32_t) * (size_t)nb, hipMemcpyHostToDevice, stream));
+        DRONE_HIP_TRY(hipMemcpyAsync(rb->block_unit0, h_unit0.data(), sizeof(int32_t) * (size_t)nb, hipMemcpyHostToDevice, stream));
+        DRONE_HIP_TRY(hipMemcpyAsync(rb->block_partial, h_partial.data(), sizeof(int64_t) * (size_t)nb, hipMemcpyHostToDevice, stream));
+        std::vector<int32_t> h_split;
+        for (int b = 0; b < nb; ++b)
+            if (h_units[b] > 1) h_split.push_back(b);
+        rb->num_split = (int)h_split.size();
+        DRONE_HIP_TRY(hipMalloc(&rb->split_block, sizeof(int32_t) * (h_split.size() ? h_split.size() : 1)));
+        if (!h_split.empty())
+            DRONE_HIP_TRY(hipMemcpyAsync(rb->split_block, h_split.data(), sizeof(int32_t) * h_split.size(), hipMemcpyHostToDevice, stream));
         DRONE_HIP_TRY(hipGetLastError());
         DRONE_HIP_TRY(hipStreamSynchronize(stream));
         return DRONE_OK;
@@ -201,6 +246,12 @@ void row_blocks_destroy(RowBlocks *rb)
     (void)hipFree(rb->batch_base);
     (void)hipFree(rb->block_batch);
     (void)hipFree(rb->block_wide);
+    (void)hipFree(rb->unit_block);
+    (void)hipFree(rb->block_units);
+    (void)hipFree(rb->block_unit0);
+    (void)hipFree(rb->block_partial);
+    (void)hipFree(rb->split_block);
+    (void)hipFree(rb->partial);
     *rb = RowBlocks{};
 }
 

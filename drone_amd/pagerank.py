@@ -175,7 +175,8 @@ class PRWorkerCUDA:
 class PullPlanF64:
     """fp64 pull PageRank over device tensors: row_ptr int64 [n+1], col_idx int32 [nnz], inv_outdeg f64 [n]."""
 
-    def __init__(self, row_ptr, col_idx, inv_outdeg, stream=0, deterministic=False):
+    def __init__(self, row_ptr, col_idx, inv_outdeg, stream=0, deterministic=False, shared_blocks=None):
+        """shared_blocks: None = decided by the matrix size, True / False = DRONE_PR_SHARED_BLOCKS / _WHOLE_BLOCKS."""
         import torch
         assert row_ptr.is_cuda and row_ptr.dtype == torch.int64 and row_ptr.is_contiguous()
         assert col_idx.is_cuda and col_idx.dtype == torch.int32 and col_idx.is_contiguous()
@@ -188,7 +189,9 @@ class PullPlanF64:
         torch.cuda.synchronize()
         h = C.c_void_p()
         check(lib().drone_pr_plan_create_ex(C.byref(h), self.n, self.nnz, row_ptr.data_ptr(), col_idx.data_ptr(),
-                                            inv_outdeg.data_ptr(), 1 if deterministic else 0, stream))
+                                            inv_outdeg.data_ptr(),
+                                            (1 if deterministic else 0) | (0 if shared_blocks is None else 2 if shared_blocks else 4),
+                                            stream))
         self.deterministic = bool(deterministic)
         self.h = h
 

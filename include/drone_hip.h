@@ -135,6 +135,11 @@ int drone_pr_plan_create(drone_pr_plan **plan, int64_t n, int64_t nnz, const int
  * with the reference's float atomics).  DRONE_PR_DETERMINISTIC selects the merge-path kernel, whose
  * results are bitwise reproducible. */
 #define DRONE_PR_DETERMINISTIC 1
+/* Tuning overrides of the default mode.  Row blocks of a large matrix (about 50 M entries and more) are shared by up
+ * to four work-groups, which then find more entries per cache line of the gather source; small matrices keep one
+ * work-group per block.  DRONE_PR_SHARED_BLOCKS forces sharing, DRONE_PR_WHOLE_BLOCKS forbids it. */
+#define DRONE_PR_SHARED_BLOCKS 2
+#define DRONE_PR_WHOLE_BLOCKS 4
 int drone_pr_plan_create_ex(drone_pr_plan **plan, int64_t n, int64_t nnz, const int64_t *row_ptr,
                             const int32_t *col_idx, const double *inv_outdeg, int flags, drone_stream_t stream);
 int drone_pr_plan_destroy(drone_pr_plan *plan);

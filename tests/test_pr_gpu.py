@@ -30,10 +30,16 @@ def in_csr_np(n, src, dst):
     return rp, s.astype(np.int32), inv
 
 
-def run_plan(torch, rp, ci, inv, iters, alpha=ALPHA, deterministic=False):
+def mode_kwargs(mode):
+    """False: the default row-block kernel; "shared": row blocks shared by several work-groups whatever the size;
+    True: the bit-reproducible merge-path kernel."""
+    return dict(deterministic=(mode is True), shared_blocks=(True if mode == "shared" else None))
+
+
+def run_plan(torch, rp, ci, inv, iters, alpha=ALPHA, **plan_kwargs):
     from drone_amd.pagerank import PullPlanF64
     plan = PullPlanF64(torch.from_numpy(rp).cuda(), torch.from_numpy(ci).cuda(), torch.from_numpy(inv).cuda(),
-                       deterministic=deterministic)
+                       **plan_kwargs)
     out = plan.run(alpha, iters).cpu().numpy()
     plan.close()
     return out
@@ -74,7 +80,7 @@ def small_cases():
     return cases
 
 
-MODES = [pytest.param(False, id="rowblock"), pytest.param(True, id="mergepath")]
+MODES = [pytest.param(False, id="rowblock"), pytest.param("shared", id="rowblock-shared"), pytest.param(True, id="mergepath")]
 
 
 @pytest.mark.parametrize("det", MODES)
@@ -83,7 +89,7 @@ MODES = [pytest.param(False, id="rowblock"), pytest.param(True, id="mergepath")]
 def test_pull_f64_edge_cases(torch_cuda, oracle, name, iters, det):
     n, src, dst = small_cases()[name]
     rp, ci, inv = in_csr_np(n, src, dst)
-    got = run_plan(torch_cuda, rp, ci, inv, iters, deterministic=det)
+    got = run_plan(torch_cuda, rp, ci, inv, iters, **mode_kwargs(det))
     ref = oracle.pr_pull_f64(rp, ci, inv, ALPHA, iters)
     assert_rel(got, ref, 1e-9)
     assert abs(got.sum() - 1.0) < 1e-11
@@ -95,7 +101,7 @@ def test_pull_f64_rmat(torch_cuda, oracle, scale, ef, seed, iters, det):
     """(16, 16, seed 1, 20 iterations) is the first benchmark configuration at full size."""
     from drone_amd import rmat
     x = rmat.pagerank_inputs_np(scale, ef, seed)
-    got = run_plan(torch_cuda, x["row_ptr"], x["col_idx"], x["inv_outdeg"], iters, deterministic=det)
+    got = run_plan(torch_cuda, x["row_ptr"], x["col_idx"], x["inv_outdeg"], iters, **mode_kwargs(det))
     ref = oracle.pr_pull_f64(x["row_ptr"], x["col_idx"], x["inv_outdeg"], ALPHA, iters)
     assert_rel(got, ref, 1e-9)
     assert abs(got.sum() - 1.0) < 1e-11
@@ -108,12 +114,12 @@ def test_pull_f64_other_alpha_and_rerun(torch_cuda, oracle, det):
     torch = torch_cuda
     x = rmat.pagerank_inputs_np(12, 16, 9)
     plan = PullPlanF64(torch.from_numpy(x["row_ptr"]).cuda(), torch.from_numpy(x["col_idx"]).cuda(),
-                       torch.from_numpy(x["inv_outdeg"]).cuda(), deterministic=det)
+                       torch.from_numpy(x["inv_outdeg"]).cuda(), **mode_kwargs(det))
     for alpha, iters in ((0.5, 7), (0.99, 3), (0.85, 7)):          # the same plan is reusable
         got = plan.run(alpha, iters).cpu().numpy()
         assert_rel(got, oracle.pr_pull_f64(x["row_ptr"], x["col_idx"], x["inv_outdeg"], alpha, iters), 1e-9)
     a = plan.run(0.85, 7).cpu().numpy()
-    if det:
+    if det is True:
         np.testing.assert_array_equal(a, got)                        # merge-path mode: bitwise run-to-run determinism
     else:
         np.testing.assert_allclose(a, got, rtol=1e-13)               # row-block mode: unordered LDS additions
@@ -130,10 +136,10 @@ def test_pull_f64_torch_streams_and_tensor_devices(torch_cuda):
         rp, ci, inv = (torch.from_numpy(x[k]).cuda() for k in ("row_ptr", "col_idx", "inv_outdeg"))
     s.synchronize()
     for det in (True, False):
-        plan = PullPlanF64(rp, ci, inv, stream=s.cuda_stream, deterministic=det)
+        plan = PullPlanF64(rp, ci, inv, stream=s.cuda_stream, **mode_kwargs(det))
         a = plan.run(0.85, 5)
         s.synchronize()
-        plan0 = PullPlanF64(rp, ci, inv, stream=0, deterministic=det)
+        plan0 = PullPlanF64(rp, ci, inv, stream=0, **mode_kwargs(det))
         b = plan0.run(0.85, 5)
         torch.cuda.synchronize()
         if det:
@@ -154,7 +160,7 @@ def test_pull_f64_full_size_properties(torch_cuda, det):
     torch = torch_cuda
     x = rmat.pagerank_inputs_torch(24, 16, 2)
     n = x["n"]
-    plan = PullPlanF64(x["row_ptr"], x["col_idx"], x["inv_outdeg"], deterministic=det)
+    plan = PullPlanF64(x["row_ptr"], x["col_idx"], x["inv_outdeg"], **mode_kwargs(det))
     r50 = plan.run(ALPHA, 50)
     assert abs(float(r50.sum()) - 1.0) < 1e-10
     assert float(r50.min()) >= (1 - ALPHA) / n * (1 - 1e-12)
