@@ -268,7 +268,7 @@ extern "C" int drone_pr_run_f64(drone_pr_plan *p, double alpha, int iters, doubl
                 p->rb.block_wide, p->rb.unit_block, p->rb.block_units, p->rb.block_unit0, p->rb.block_partial,
                 p->rb.partial, epi, carry, p->ms.tile_stat);
             if (p->rb.num_split > 0)
-                pr_rowblock_merge_kernel<PrF64Epi><<<p->rb.num_split, kRbThreads, 0, s>>>(
+                pr_rowblock_merge_kernel<PrF64Epi><<<dim3((unsigned)p->rb.num_split, (unsigned)(kRbRows / kRbThreads + 1)), kRbThreads, 0, s>>>(
                     p->rb.split_block, p->rb.block_row, p->rb.block_units, p->rb.block_partial, p->rb.partial, epi, carry,
                     p->ms.tile_stat);
         }

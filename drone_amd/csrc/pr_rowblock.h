@@ -210,6 +210,7 @@ __global__ __launch_bounds__(kRbThreads) void pr_rowblock_kernel(const int32_t *
         // instead of 0.68 with two shares per block.)
         double *mine = partial + block_partial[b] + (int64_t)share * (nr + 1);
         for (int i = tid; i <= nr; i += kRbThreads) mine[i] = s_acc[i];
+        if (share == 0 && tid == 0) block_stat[b] = 0.0;  // the merge kernel adds the block's statistic up
         return;
     }
 
@@ -226,7 +227,8 @@ __global__ __launch_bounds__(kRbThreads) void pr_rowblock_kernel(const int32_t *
     }
 }
 
-// Split blocks: adds the shares of every row and runs the epilogue.  One work-group per split block.
+// Split blocks: adds the shares of every row and runs the epilogue.  Work-group (x, y) takes rows y * 1024 ... of the
+// x-th split block; the block's statistic is summed with atomics (share 0 of the block cleared it).
 template <typename Epi>
 __global__ __launch_bounds__(kRbThreads) void pr_rowblock_merge_kernel(const int32_t *__restrict__ split_block,
                                                                        const int32_t *__restrict__ block_row,
@@ -239,16 +241,19 @@ __global__ __launch_bounds__(kRbThreads) void pr_rowblock_merge_kernel(const int
     __shared__ double s_red[kRbThreads / kWave];
     const int b = split_block[blockIdx.x], tid = threadIdx.x;
     const int r0 = block_row[b], nr = block_row[b + 1] - r0, shares = block_units[b];
+    const int i = blockIdx.y * kRbThreads + tid;
+    if (blockIdx.y * kRbThreads > nr) return;
     const double *area = partial + block_partial[b];
     double stat = 0.0;
-    for (int i = tid; i <= nr; i += kRbThreads) {
+    if (i <= nr) {
+        const double op = i < nr ? epi.row_operand(r0 + i) : 0.0;
         double sum = 0.0;
         for (int sh = 0; sh < shares; ++sh) sum += area[(int64_t)sh * (nr + 1) + i];
-        if (i < nr) epi.row(r0 + i, sum, epi.row_operand(r0 + i), stat);
+        if (i < nr) epi.row(r0 + i, sum, op, stat);
         else block_carry[b] = sum;  // the row left open at the end of the block
     }
     const double total = block_sum_1024(stat, s_red);
-    if (tid == 0) block_stat[b] = total;
+    if (tid == 0 && total != 0.0) atomicAdd(&block_stat[b], total);
 }
 
 }  // namespace drone
