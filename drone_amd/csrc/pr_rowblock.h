@@ -103,6 +103,9 @@ __device__ __forceinline__ double block_sum_1024(double v, double *s_red)
 // help: blocks of 8,192 rows with two of them resident per CU measured 0.90 ms (1 M entries) and 0.99 ms (512 K).
 // Summing the short-row blocks in row order instead (a lane per row, four rows in flight, no LDS) took 0.287 ms for
 // the same blocks that add 0.075 ms to this kernel, where they fill the CUs that have run out of dense blocks.
+// In the short-row blocks the wavefronts that finish early wait a third of the block's time at the barrier, but
+// letting every wavefront take the next 256 entries off a counter instead (perfect balance, all wavefronts in the
+// same part of the sweep) measured 0.687 against 0.606 ms.
 // Longer slices for the wavefronts that finish first (6 % / 18 % more entries for the oldest four) measured 0.685
 // against 0.678 with equal slices.
 // Indices past the end of a slice are clamped to the block's last entry (gathered, then added as 0.0), which keeps
