@@ -107,7 +107,8 @@ __device__ __forceinline__ double block_sum_1024(double v, double *s_red)
 // letting every wavefront take the next 256 entries off a counter instead (perfect balance, all wavefronts in the
 // same part of the sweep) measured 0.687 against 0.606 ms.
 // Longer slices for the wavefronts that finish first (6 % / 18 % more entries for the oldest four) measured 0.685
-// against 0.678 with equal slices.
+// against 0.678 with equal slices, and 0.609 against 0.606 when only the short-row blocks got them: the waiting
+// wavefronts cost nothing while the memory system is the bottleneck.
 // Indices past the end of a slice are clamped to the block's last entry (gathered, then added as 0.0), which keeps
 // the loop free of divergent branches.
 template <bool kWide, typename Epi>
