@@ -138,12 +138,11 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
     // 24 with 1 / 2 / 4 / 8 / 16 work-groups per block: 0.060 0.063 0.079 0.081 0.087 / 0.175 0.181 0.172 0.216
     // 0.184 / 0.679 0.649 0.617 0.659 0.670: small ones lose more to the second kernel than they gain).
     const int split = shared_blocks == 1 ? 1 : (shared_blocks == 2 || nnz >= (int64_t)48 << 20) ? kRbSplit : 1;
-    items *= split;                        // entries one block holds
-    rb->items = items;
+    rb->items = items * split;             // entries one block holds at most
     const int weight = items / kRbRows;
     const int64_t total = (int64_t)weight * n + nnz;
-    rb->num_blocks = (int)ceil_div(total, items);
-    const int nb = rb->num_blocks;
+    int nb = (int)ceil_div(total, items);  // blocks of the weighted split; fewer once neighbours are merged
+    rb->num_blocks = nb;
     uint64_t *keys = nullptr, *keys_sorted = nullptr;
     uint16_t *lrow_in = nullptr;
     void *temp = nullptr;
@@ -156,6 +155,34 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
         DRONE_HIP_TRY(hipMalloc(&rb->col, sizeof(int32_t) * e));
         DRONE_HIP_TRY(hipMalloc(&rb->lrow, sizeof(uint16_t) * e));
         rb_search_kernel<<<(int)ceil_div(nb + 1, 256), 256, 0, stream>>>(row_ptr, n, nnz, nb, items, weight, rb->block_row, rb->block_nnz);
+        if (split > 1) {
+            // Shared blocks: the weighted split trades rows against entries, so its blocks reach neither limit.
+            // Neighbours are merged while the result stays within 16,384 rows and split x items entries.
+            std::vector<int32_t> br((size_t)nb + 1);
+            std::vector<int64_t> bn((size_t)nb + 1);
+            DRONE_HIP_TRY(hipMemcpyAsync(br.data(), rb->block_row, sizeof(int32_t) * br.size(), hipMemcpyDeviceToHost, stream));
+            DRONE_HIP_TRY(hipMemcpyAsync(bn.data(), rb->block_nnz, sizeof(int64_t) * bn.size(), hipMemcpyDeviceToHost, stream));
+            DRONE_HIP_TRY(hipStreamSynchronize(stream));
+            int out = 0, first = 0;
+            for (int b = 1; b <= nb; ++b) {
+                // close the block [first, b) when taking block b as well would break a limit
+                const bool last_one = b == nb;
+                if (last_one || br[(size_t)b + 1] - br[(size_t)first] > kRbRows ||
+                    bn[(size_t)b + 1] - bn[(size_t)first] > (int64_t)items * split) {
+                    br[(size_t)out] = br[(size_t)first];
+                    bn[(size_t)out] = bn[(size_t)first];
+                    ++out;
+                    first = b;
+                }
+            }
+            br[(size_t)out] = br[(size_t)nb];
+            bn[(size_t)out] = bn[(size_t)nb];
+            nb = out;
+            rb->num_blocks = nb;
+            DRONE_HIP_TRY(hipMemcpyAsync(rb->block_row, br.data(), sizeof(int32_t) * ((size_t)nb + 1), hipMemcpyHostToDevice, stream));
+            DRONE_HIP_TRY(hipMemcpyAsync(rb->block_nnz, bn.data(), sizeof(int64_t) * ((size_t)nb + 1), hipMemcpyHostToDevice, stream));
+            DRONE_HIP_TRY(hipStreamSynchronize(stream));  // br / bn go out of scope
+        }
         rb_walk_len_kernel<<<(int)ceil_div(nb, 256), 256, 0, stream>>>(row_ptr, nb, rb->block_row, rb->block_nnz, rb->walk_len);
         if (nnz > 0) {
             DRONE_HIP_TRY(hipMalloc(&keys, sizeof(uint64_t) * e));
@@ -193,7 +220,7 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
         for (int b = 0; b < nb; ++b) {
             const int64_t entries = h_nnz[b + 1] - h_nnz[b];
             const int batches = h_batch[b + 1] - h_batch[b];
-            int shares = (int)ceil_div(entries, unit_items);
+            int shares = (int)ceil_div(entries, (int64_t)unit_items);
             if (shares < 1) shares = 1;
             if (shares > split) shares = split;
             if (shares > batches && batches > 0) shares = batches;
