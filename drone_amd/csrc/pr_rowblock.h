@@ -30,7 +30,7 @@ constexpr int kRbThreads = 1024;
 constexpr int kRbRows = 16384;       // most rows ending in one block (LDS accumulators: 128 KB)
 constexpr int kRbMaxItems = 1 << 20; // most entries in one block (the plan picks a power of two up to this)
 constexpr int kRbUnroll = 4;
-constexpr int kRbSplit = 4;         // work-groups that share one block of a large matrix
+constexpr int kRbSplit = 8;         // most work-groups that share one block of a large matrix
 constexpr int kRbLdsBytes = (kRbRows + 8) * (int)sizeof(double);  // rows ending in a block <= kRbRows + 1, + the open row
 
 struct RowBlocks {
@@ -51,7 +51,7 @@ struct RowBlocks {
     int32_t *block_wide = nullptr;  // device [num_blocks]
     // Work units.  A block with many entries is swept by several work-groups, each taking every shares-th slice of
     // its sorted entries; they leave their row sums in `partial`, and a second kernel adds them up and runs the
-    // epilogue.  Such a block holds kRbSplit times the entries one work-group handles, so the same number of
+    // epilogue.  Such a block holds up to kRbSplit times the entries one work-group handles, so the same number of
     // work-groups finds more entries per source line (R-MAT scale 24: 33.7 M distinct (block, line) pairs with 1 M
     // entries per block, 14.9 M with 4 M), and every work-group still sweeps hot and cold slices side by side.
     int num_units = 0;

@@ -134,9 +134,11 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
     int items = 32768;
     while (items < kRbMaxItems && (double)items * 1.41421356 < (double)nnz / (cus > 0 ? cus : 256)) items <<= 1;
     const int unit_items = items;          // entries one work-group sweeps
-    // Large matrices get blocks that several work-groups share (measured, ms per iteration at R-MAT scale 20 / 22 /
-    // 24 with 1 / 2 / 4 / 8 / 16 work-groups per block: 0.060 0.063 0.079 0.081 0.087 / 0.175 0.181 0.172 0.216
-    // 0.184 / 0.679 0.649 0.617 0.659 0.670: small ones lose more to the second kernel than they gain).
+    // Large matrices get blocks that several work-groups share.  Measured, ms per iteration at R-MAT scale 20 / 22 /
+    // 24: with blocks of the weighted split alone and 1 / 2 / 4 / 8 / 16 work-groups per block 0.060 0.063 0.079
+    // 0.081 0.087 / 0.175 0.181 0.172 0.216 0.184 / 0.679 0.649 0.617 0.659 0.670 (small matrices lose more to the
+    // second kernel than they gain); with neighbouring blocks merged up to the limits (below) and up to 3 / 4 / 6 / 8
+    // / 12 / 16 / 32 work-groups per block, scale 24: 0.612 0.588 0.583 0.571 0.573 0.575 0.574.
     const int split = shared_blocks == 1 ? 1 : (shared_blocks == 2 || nnz >= (int64_t)48 << 20) ? kRbSplit : 1;
     rb->items = items * split;             // entries one block holds at most
     const int weight = items / kRbRows;
