@@ -449,7 +449,7 @@ def main():
                      "frac": achieved / HBM_PEAK_GBS,
                      # fabric bytes per launch: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by the 1 GiB copy
                      # kernel; measured for this workload only (profiles/pr_rowblock_pagerank_c2.hbm_traffic.txt)
-                     "traffic": 3.71e9 if (args.scale == 24 and n == 16777216) else None,
+                     "traffic": 3.48e9 if (args.scale == 24 and n == 16777216) else None,
                      "kernel": "pr_rowblock_kernel<PrF64Epi> + pr_rowblock_merge_kernel<PrF64Epi> (one iteration)",
                      "algorithmic_bytes_per_launch": bytes_iter, "mean_launch_ms": prof["mean_ms"],
                      "launches_timed": prof["launches"]},
