@@ -50,7 +50,6 @@ __global__ void set_mirror2worker_kernel(int *m2w, const int *mirror_vertex, con
 // steps: the scan order u[0], v[0], u[1], v[1], ... gives every endpoint a position; a vertex's first position
 // (atomicMin) decides when it is "first seen", an exclusive scan over the first-occurrence flags turns that into the
 // local id, and the two CSRs are stable sorts of the edges by local source / of the out-edge CSR by destination.
-constexpr unsigned kNever = 0xFFFFFFFFu;
 
 __global__ void first_position_kernel(int edges, int nglobal, const int *__restrict__ u, const int *__restrict__ v,
                                       unsigned *__restrict__ first_pos, int *__restrict__ bad_edge)

@@ -2,6 +2,8 @@
 #pragma once
 #include <vector>
 
+#include "pr_rowblock.h"
+#include "relabel.h"
 #include "spmv_merge.h"
 
 struct drone_pr_plan;
@@ -49,6 +51,11 @@ struct GraphExt {
     bool push_ready = false;
     MergeTiling mt;
     MergeScratch ms;
+    // large subgraphs: the same aggregation over source-sorted row blocks (built at the first PR_PEVal)
+    bool rb_tried = false, rb_ready = false;
+    RowBlocks rb;             // over the in-edge CSR with its sources renumbered hot-first
+    MergeScratch ms_rb;
+    int32_t *rb_new_id = nullptr;  // device [n]: local id -> renumbered id (where a vertex's push value is kept)
     // fp64 pull run driven from the Graph
     drone_pr_plan *plan64 = nullptr;
     int64_t *row_ptr64 = nullptr;

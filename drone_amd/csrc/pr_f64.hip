@@ -15,6 +15,8 @@ namespace drone {
 constexpr int kPrIpt = 8;  // items per lane; tile = 2048 merge items, 24.6 KB of LDS
 
 struct PrF64Epi {
+    using Acc = double;         // what an entry contributes and a row accumulates
+    using RowOperand = double;  // what row() needs besides the row sum
     const double *__restrict__ c_in;   // gather source
     const double *__restrict__ inv;    // inverse out-degree, 0 for dangling
     double *__restrict__ c_out;        // next gather source

@@ -19,6 +19,7 @@
 // bit-reproducible results.
 #pragma once
 #include "spmv_merge.h"
+#include <type_traits>
 
 namespace drone {
 
@@ -61,7 +62,7 @@ struct RowBlocks {
     int64_t *block_partial = nullptr;// device [num_blocks]: where the block's shares start in `partial` (in doubles)
     int num_split = 0;
     int32_t *split_block = nullptr;  // device [num_split]: the blocks with more than one unit
-    double *partial = nullptr;       // device: per split block, block_units x (rows + 1) row sums
+    double *partial = nullptr;       // device: per split block, block_units x (rows + 1) row sums (8-byte values)
 };
 
 // Builds the blocks for a CSR with device row_ptr / col (already in the plan's internal id space).
@@ -111,12 +112,40 @@ __device__ __forceinline__ double block_sum_1024(double v, double *s_red)
 // wavefronts cost nothing while the memory system is the bottleneck.
 // Indices past the end of a slice are clamped to the block's last entry (gathered, then added as 0.0), which keeps
 // the loop free of divergent branches.
+// The LDS accumulators are doubles.  A row of the fp64 PageRank is just that sum; a row of the float delta-push
+// entry points is a PushF2 {sum, whether any entry pushed something}, kept as the double sum plus one bit per row
+// in a separate bit mask.  Two float accumulators per row were the obvious layout, but 65 M entries took 0.43 ms per
+// LDS float add and 0.15 ms per LDS double add on this GPU (one float add 0.53 ms, two 0.96 ms, one double 0.25 ms
+// for the whole superstep).
+// `live` is false for the clamped entries past a slice's end, which must add nothing.
+constexpr int kRbSpare = kRbRows + 7;                    // accumulator nobody reads
+constexpr int kRbFlagWords = 4096;  // row i's bit: word i % 4096, bit i / 4096 (neighbouring rows in different words)
+__device__ __forceinline__ void rb_add(double *s_acc, uint32_t *, int l, bool live, double v)
+{
+    atomicAdd(&s_acc[l], live ? v : 0.0);
+}
+__device__ __forceinline__ void rb_add(double *s_acc, uint32_t *s_flag, int l, bool live, PushF2 v)
+{
+    // Both updates are unconditional and a clamped entry goes to the spare accumulator instead of having its value
+    // replaced: with `if (v.c != 0)` around them, or a select on the gathered value, the compiler sinks one entry's
+    // gathers into a branch and waits for each of them on its own.
+    const int slot = live ? l : kRbSpare;
+    atomicAdd(&s_acc[slot], (double)v.s);
+    atomicOr(&s_flag[slot & (kRbFlagWords - 1)], (v.c != 0.0f ? 1u : 0u) << (slot / kRbFlagWords));
+}
+__device__ __forceinline__ void rb_read(const double *s_acc, const uint32_t *, int i, double &out) { out = s_acc[i]; }
+__device__ __forceinline__ void rb_read(const double *s_acc, const uint32_t *s_flag, int i, PushF2 &out)
+{
+    out = PushF2{(float)s_acc[i], (float)((s_flag[i & (kRbFlagWords - 1)] >> (i / kRbFlagWords)) & 1u)};
+}
+
 template <bool kWide, typename Epi>
 __device__ __forceinline__ void rb_accumulate(int64_t block_begin, int64_t block_end, int share, int shares, int tid,
                                               const int32_t *__restrict__ col, const uint16_t *__restrict__ lrow,
                                               const uint32_t *__restrict__ packed, const int32_t *__restrict__ bases,
-                                              const Epi &epi, double *s_acc)
+                                              const Epi &epi, double *s_acc, uint32_t *s_flag)
 {
+    using Acc = typename Epi::Acc;
     // The block's sorted entries [block_begin, block_end) are cut into 16 * shares slices of whole 64-entry batches;
     // wavefront w of share k sweeps slice w * shares + k, so every work-group of a split block gets the same mix of
     // popular (L1-hitting) and cold (missing) slices that an unsplit block has.
@@ -150,12 +179,12 @@ __device__ __forceinline__ void rb_accumulate(int64_t block_begin, int64_t block
             c[k] = kWide ? (int)a[k] : g[k] + (int)(a[k] & 0xFFFFu);
             l[k] = kWide ? g[k] : (int)(a[k] >> 16);
         }
-        double v[kRbUnroll];
+        Acc v[kRbUnroll];
 #pragma unroll
         for (int k = 0; k < kRbUnroll; ++k) v[k] = epi.load(c[k]);
 #pragma unroll
         for (int k = 0; k < kRbUnroll; ++k)
-            atomicAdd(&s_acc[l[k]], base + k * kWave + lane < s1 ? v[k] : 0.0);  // clamped entries add 0
+            rb_add(s_acc, s_flag, l[k], base + k * kWave + lane < s1, v[k]);
     }
 }
 
@@ -172,11 +201,14 @@ __global__ __launch_bounds__(kRbThreads) void pr_rowblock_kernel(const int32_t *
                                                                  const int32_t *__restrict__ block_units,
                                                                  const int32_t *__restrict__ block_unit0,
                                                                  const int64_t *__restrict__ block_partial,
-                                                                 double *__restrict__ partial, Epi epi,
-                                                                 double *__restrict__ block_carry,
+                                                                 typename Epi::Acc *__restrict__ partial, Epi epi,
+                                                                 typename Epi::Acc *__restrict__ block_carry,
                                                                  double *__restrict__ block_stat)
 {
+    using Acc = typename Epi::Acc;
+    constexpr bool kFlagged = !std::is_same<Acc, double>::value;
     extern __shared__ double s_acc[];  // [rows ending in the block + 1 (the row left open)]
+    __shared__ uint32_t s_flag[kFlagged ? kRbFlagWords : 1];
     __shared__ double s_red[kRbThreads / kWave];
     const int u = blockIdx.x, tid = threadIdx.x;
     const int b = unit_block[u];
@@ -190,21 +222,23 @@ __global__ __launch_bounds__(kRbThreads) void pr_rowblock_kernel(const int32_t *
     // sweep, one row at a time, it cost a memory latency per row (a quarter of the time of the blocks that hold
     // many short rows).  Split blocks hold few rows; the work-group that ends up with the epilogue reads them then.
     constexpr int kEpiSlots = kRbRows / kRbThreads + 1;
-    double row_op[kEpiSlots];
+    typename Epi::RowOperand row_op[kEpiSlots];
     if (shares == 1) {
 #pragma unroll
         for (int k = 0; k < kEpiSlots; ++k) {
             const int i = tid + k * kRbThreads;
-            row_op[k] = i < nr ? epi.row_operand(r0 + i) : 0.0;
+            row_op[k] = i < nr ? epi.row_operand(r0 + i) : typename Epi::RowOperand{};
         }
     }
     for (int i = tid; i <= nr; i += kRbThreads) s_acc[i] = 0.0;
+    if (kFlagged)
+        for (int i = tid; i < kRbFlagWords; i += kRbThreads) s_flag[i] = 0u;
     __syncthreads();
 
     if (wide)
-        rb_accumulate<true>(eb, ee, share, shares, tid, col, lrow, packed, bases, epi, s_acc);
+        rb_accumulate<true>(eb, ee, share, shares, tid, col, lrow, packed, bases, epi, s_acc, s_flag);
     else
-        rb_accumulate<false>(eb, ee, share, shares, tid, col, lrow, packed, bases, epi, s_acc);
+        rb_accumulate<false>(eb, ee, share, shares, tid, col, lrow, packed, bases, epi, s_acc, s_flag);
     __syncthreads();
 
     if (shares > 1) {
@@ -212,8 +246,8 @@ __global__ __launch_bounds__(kRbThreads) void pr_rowblock_kernel(const int32_t *
         // (Letting the work-group that arrives last do that inside this kernel needs device-scope fences, and on a
         // GPU whose XCDs have separate L2s every such fence writes back and invalidates a whole L2: 0.99 ms
         // instead of 0.68 with two shares per block.)
-        double *mine = partial + block_partial[b] + (int64_t)share * (nr + 1);
-        for (int i = tid; i <= nr; i += kRbThreads) mine[i] = s_acc[i];
+        Acc *mine = partial + block_partial[b] + (int64_t)share * (nr + 1);
+        for (int i = tid; i <= nr; i += kRbThreads) rb_read(s_acc, s_flag, i, mine[i]);
         if (share == 0 && tid == 0) block_stat[b] = 0.0;  // the merge kernel adds the block's statistic up
         return;
     }
@@ -222,12 +256,16 @@ __global__ __launch_bounds__(kRbThreads) void pr_rowblock_kernel(const int32_t *
 #pragma unroll
     for (int k = 0; k < kEpiSlots; ++k) {
         const int i = tid + k * kRbThreads;
-        if (i < nr) epi.row(r0 + i, s_acc[i], row_op[k], stat);
+        if (i < nr) {
+            Acc sum;
+            rb_read(s_acc, s_flag, i, sum);
+            epi.row(r0 + i, sum, row_op[k], stat);
+        }
     }
     const double total = block_sum_1024(stat, s_red);
     if (tid == 0) {
         block_stat[b] = total;
-        block_carry[b] = s_acc[nr];
+        rb_read(s_acc, s_flag, nr, block_carry[b]);
     }
 }
 
@@ -238,8 +276,9 @@ __global__ __launch_bounds__(kRbThreads) void pr_rowblock_merge_kernel(const int
                                                                        const int32_t *__restrict__ block_row,
                                                                        const int32_t *__restrict__ block_units,
                                                                        const int64_t *__restrict__ block_partial,
-                                                                       const double *__restrict__ partial, Epi epi,
-                                                                       double *__restrict__ block_carry,
+                                                                       const typename Epi::Acc *__restrict__ partial,
+                                                                       Epi epi,
+                                                                       typename Epi::Acc *__restrict__ block_carry,
                                                                        double *__restrict__ block_stat)
 {
     __shared__ double s_red[kRbThreads / kWave];
@@ -247,12 +286,13 @@ __global__ __launch_bounds__(kRbThreads) void pr_rowblock_merge_kernel(const int
     const int r0 = block_row[b], nr = block_row[b + 1] - r0, shares = block_units[b];
     const int i = blockIdx.y * kRbThreads + tid;
     if (blockIdx.y * kRbThreads > nr) return;
-    const double *area = partial + block_partial[b];
+    using Acc = typename Epi::Acc;
+    const Acc *area = partial + block_partial[b];
     double stat = 0.0;
     if (i <= nr) {
-        const double op = i < nr ? epi.row_operand(r0 + i) : 0.0;
-        double sum = 0.0;
-        for (int sh = 0; sh < shares; ++sh) sum += area[(int64_t)sh * (nr + 1) + i];
+        const typename Epi::RowOperand op = i < nr ? epi.row_operand(r0 + i) : typename Epi::RowOperand{};
+        Acc sum = vzero<Acc>();
+        for (int sh = 0; sh < shares; ++sh) sum = sum + area[(int64_t)sh * (nr + 1) + i];
         if (i < nr) epi.row(r0 + i, sum, op, stat);
         else block_carry[b] = sum;  // the row left open at the end of the block
     }

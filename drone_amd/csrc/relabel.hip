@@ -28,6 +28,13 @@ __global__ void count_from_inverse_kernel(const double *__restrict__ inv, int64_
     }
 }
 
+// The gather counts are the row lengths of the transposed CSR when the caller has one.
+__global__ void count_from_offsets_kernel(const int *__restrict__ offsets, int64_t n, unsigned *__restrict__ count)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        count[i] = (unsigned)(offsets[i + 1] - offsets[i]);
+}
+
 __global__ void iota_kernel(int32_t *a, int64_t n)
 {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
@@ -101,6 +108,13 @@ __global__ __launch_bounds__(256) void remap_rows_kernel(const int32_t *__restri
     }
 }
 
+__global__ void remap_cols_kernel(const int32_t *__restrict__ col, const int32_t *__restrict__ new_id, int64_t nnz,
+                                  int32_t *__restrict__ new_col)
+{
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < nnz; e += (int64_t)gridDim.x * blockDim.x)
+        new_col[e] = new_id[col[e]];
+}
+
 __global__ void gather_f64_kernel(const int32_t *__restrict__ order, const double *__restrict__ in, int64_t n,
                                   double *__restrict__ out)
 {
@@ -120,7 +134,7 @@ __global__ void gather_f64_kernel(const int32_t *__restrict__ order, const doubl
 }  // namespace
 
 int relabel_create(Relabel *rl, int64_t n, int64_t nnz, const int64_t *row_ptr, const int32_t *col,
-                   const double *inv_outdeg, hipStream_t stream)
+                   const double *inv_outdeg, hipStream_t stream, bool keep_rows, const int *transposed_offsets)
 {
     int rc = DRONE_OK;
     unsigned *count = nullptr, *count_sorted = nullptr;
@@ -142,6 +156,7 @@ int relabel_create(Relabel *rl, int64_t n, int64_t nnz, const int64_t *row_ptr, 
     RL_TRY(hipMemsetAsync(count, 0, sizeof(unsigned) * (size_t)n, stream));
     RL_TRY(hipMemsetAsync(len + n, 0, sizeof(int64_t), stream));
     if (inv_outdeg) count_from_inverse_kernel<<<blocks, threads, 0, stream>>>(inv_outdeg, n, count);
+    else if (transposed_offsets) count_from_offsets_kernel<<<blocks, threads, 0, stream>>>(transposed_offsets, n, count);
     else if (nnz) count_sources_kernel<<<blocks, threads, 0, stream>>>(col, nnz, count);
     iota_kernel<<<blocks, threads, 0, stream>>>(ids, n);
     // stable descending sort by gather count: order[new] = old
@@ -154,9 +169,14 @@ int relabel_create(Relabel *rl, int64_t n, int64_t nnz, const int64_t *row_ptr, 
     RL_TRY(rocprim::radix_sort_pairs_desc(temp, temp_bytes, count, count_sorted, ids, rl->order, (size_t)n, 0, 32,
                                           stream));
     invert_and_lengths_kernel<<<blocks, threads, 0, stream>>>(rl->order, row_ptr, n, new_id, len);
-    RL_TRY(rocprim::exclusive_scan(temp, temp_bytes, len, rl->row_ptr, (int64_t)0, (size_t)n + 1,
-                                   rocprim::plus<int64_t>(), stream));
-    if (nnz > 0)
+    if (keep_rows) {
+        RL_TRY(hipMemcpyAsync(rl->row_ptr, row_ptr, sizeof(int64_t) * ((size_t)n + 1), hipMemcpyDeviceToDevice, stream));
+        if (nnz > 0) remap_cols_kernel<<<blocks, threads, 0, stream>>>(col, new_id, nnz, rl->col);
+    } else {
+        RL_TRY(rocprim::exclusive_scan(temp, temp_bytes, len, rl->row_ptr, (int64_t)0, (size_t)n + 1,
+                                       rocprim::plus<int64_t>(), stream));
+    }
+    if (nnz > 0 && !keep_rows)
         remap_rows_kernel<<<(int)ceil_div(nnz, kRemapChunk), 256, 0, stream>>>(rl->order, row_ptr, col, new_id, rl->row_ptr, n,
                                                                               nnz, rl->col);
     RL_TRY(hipGetLastError());

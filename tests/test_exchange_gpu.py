@@ -35,7 +35,7 @@ FIELDS = ["VisitedSize", "Mirror2MasterSendSize", "Mirror2MasterRecvSize", "Mast
 
 @pytest.mark.parametrize("W,scale,seed,lone", [(2, 8, 1, False), (3, 10, 2, False), (4, 12, 3, False), (7, 11, 4, False),
                                                (3, 10, 5, True)])
-def test_pr_group_matches_oracle_group(oracle, W, scale, seed, lone):
+def test_pr_group_matches_oracle_group(oracle, push_aggregation, W, scale, seed, lone):
     """lone: the last worker shares no vertex with the others and still has to meet them in every exchange."""
     from drone_amd.pagerank import Loopback, PRWorkerCUDA, run_workers
     nglobal = 1 << scale

@@ -242,10 +242,10 @@ def test_build_graph_layout_stress(torch_cuda, oracle, name):
     w.close()
 
 
-@pytest.mark.parametrize("seed,scale", [(1, 10), (3, 13)])
-def test_peval_inceval_against_push_oracle(torch_cuda, oracle, seed, scale):
+@pytest.mark.parametrize("seed,scale,ef", [(1, 10, 8), (3, 13, 8), (4, 16, 16)])
+def test_peval_inceval_against_push_oracle(torch_cuda, oracle, push_aggregation, seed, scale, ef):
     from drone_amd.pagerank import PRWorkerCUDA
-    u, v, gN = _edges(seed, scale)
+    u, v, gN = _edges(seed, scale, ef)
     outdeg_global = np.bincount(u, minlength=gN).astype(np.int32)
     w = PRWorkerCUDA(gN, u, v, outdeg_global)
     n, g2l, l2g, index, dst = oracle.build_graph(gN, u, v)
@@ -271,7 +271,53 @@ def test_peval_inceval_against_push_oracle(torch_cuda, oracle, seed, scale):
     w.close()
 
 
-def test_push_path_converges_to_pull_ranks(torch_cuda, oracle):
+@pytest.mark.parametrize("shape", ["one_edge", "in_star", "out_star", "path", "multigraph", "two_hubs"])
+def test_peval_inceval_small_shapes(torch_cuda, oracle, push_aggregation, shape):
+    """Rows far longer than a block's entry capacity, single rows, repeated edges: both aggregations against the oracle."""
+    from drone_amd.pagerank import PRWorkerCUDA
+    rng = np.random.default_rng(11)
+    if shape == "one_edge":
+        u, v = np.array([3]), np.array([0])
+    elif shape == "in_star":                      # one row holding every entry
+        u, v = np.arange(1, 70001), np.zeros(70000, dtype=np.int64)
+    elif shape == "out_star":                     # every row gathers the same source
+        u, v = np.zeros(70000, dtype=np.int64), np.arange(1, 70001)
+    elif shape == "path":
+        u, v = np.arange(0, 40000), np.arange(1, 40001)
+    elif shape == "multigraph":
+        u, v = rng.integers(0, 50, 20000), rng.integers(0, 50, 20000)
+    else:                                         # two long rows with short rows in between and after
+        u = np.concatenate([np.arange(2, 40002), rng.integers(2, 3000, 5000), np.arange(2, 40002)])
+        v = np.concatenate([np.zeros(40000, dtype=np.int64), rng.integers(2, 3000, 5000), np.ones(40000, dtype=np.int64)])
+    gN = int(max(u.max(), v.max())) + 1
+    u, v = u.astype(np.int32), v.astype(np.int32)
+    outdeg_global = np.bincount(u, minlength=gN).astype(np.int32)
+    w = PRWorkerCUDA(gN, u, v, outdeg_global)
+    n, g2l, l2g, index, dst = oracle.build_graph(gN, u, v)
+    # The oracle runs the same supersteps in double here: its float restatement adds a row's entries, and the n terms
+    # of the global sums, one after the other, and with 70,000 terms that drifts by 1e-3 (d * 2^-24 of the sum of
+    # magnitudes is the bound for any order, the order of the reference's float atomics included), which these shapes
+    # then amplify from superstep to superstep.  The kernels add rows in trees (merge path) or in double (row blocks)
+    # and the global sums in double, and stay within float rounding of the double run.
+    st = oracle.PushState(index, dst, outdeg_global[l2g], gN, dtype=np.float64)
+    rtol = 5e-5
+    # out_star: from the third superstep on the hub's change is rounding noise around the eps threshold, which
+    # decides whether it pushes at all; the comparison stops before that
+    steps = 2 if shape == "out_star" else 5
+    try:
+        for k in range(steps):
+            res = w.peval() if k == 0 else w.incEval()
+            vis = st.peval() if k == 0 else st.inceval(alpha=0.85, eps=1e-6)
+            s = w.state()
+            assert res.VisitedSize == vis, (shape, k)
+            np.testing.assert_array_equal(s["active"], st.active)
+            np.testing.assert_allclose(s["diff"], st.diff, rtol=rtol, atol=1e-6)   # ranks are of order 1
+            np.testing.assert_allclose(s["pr"], st.pr, rtol=rtol)
+    finally:
+        w.close()
+
+
+def test_push_path_converges_to_pull_ranks(torch_cuda, oracle, push_aggregation):
     """After enough supersteps the float delta-push state sits within the eps bound of the fp64 ranks."""
     from drone_amd.pagerank import PRWorkerCUDA
     u, v, gN = _edges(5, 11)
