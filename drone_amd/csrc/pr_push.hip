@@ -381,6 +381,11 @@ extern "C" Response PR_PEVal(Graph *g, PRValues *values, int workerId, int worke
     return res;
 }
 
+extern "C" int drone_pr_aggregation(const Graph *g)
+{
+    return g && g->ext && static_cast<const GraphExt *>(g->ext)->rb_ready ? 1 : 0;
+}
+
 extern "C" Response PR_IncEVal(Graph *g, PRValues *values, int workerId, int workerNum, Comm *comm)
 {
     clear_error();

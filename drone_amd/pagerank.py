@@ -165,6 +165,10 @@ class PRWorkerCUDA:
                                            out.ctypes.data_as(C.c_void_p)))
         return out
 
+    def aggregation(self):
+        """'row-blocks' or 'merge-path': the kernels PR_PEVal / PR_IncEVal use for this graph (decided at the first peval)."""
+        return "row-blocks" if lib().drone_pr_aggregation(self.g) else "merge-path"
+
     def close(self):
         if self.g:
             lib().drone_pr_values_destroy(self.g, C.byref(self.values))

@@ -113,6 +113,10 @@ void loadOutDegree(Graph *g, PRValues *values, int *globalOutDegree);
 Response PR_PEVal(Graph *g, PRValues *values, int workerId, int workerNum, Comm *comm);
 Response PR_IncEVal(Graph *g, PRValues *values, int workerId, int workerNum, Comm *comm);
 
+/* No counterpart in the reference: which kernels PR_PEVal / PR_IncEVal aggregate this graph with.  0 = merge
+ * path (also before the first PR_PEVal has decided), 1 = source-sorted row blocks. */
+int drone_pr_aggregation(const Graph *g);
+
 /* No counterpart in the reference (it never frees): optional clean-up. */
 void drone_graph_destroy(Graph *g);
 void drone_pr_values_destroy(Graph *g, PRValues *values);

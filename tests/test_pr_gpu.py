@@ -251,6 +251,7 @@ def test_peval_inceval_against_push_oracle(torch_cuda, oracle, push_aggregation,
     n, g2l, l2g, index, dst = oracle.build_graph(gN, u, v)
     st = oracle.PushState(index, dst, outdeg_global[l2g], gN)
     res = w.peval()
+    assert w.aggregation() == push_aggregation
     assert res.VisitedSize == st.peval() and res.LocalVertexSize == n and res.IsEmpty()
     s = w.state()
     np.testing.assert_array_equal(s["outDegree"], outdeg_global[l2g])
@@ -315,6 +316,41 @@ def test_peval_inceval_small_shapes(torch_cuda, oracle, push_aggregation, shape)
             np.testing.assert_allclose(s["pr"], st.pr, rtol=rtol)
     finally:
         w.close()
+
+
+def test_push_full_size_row_blocks_agree_with_merge_path(torch_cuda, monkeypatch):
+    """R-MAT scale 23, edge factor 16 (about 130 M edges, above the size from which the library aggregates over row
+    blocks by itself): six supersteps on the two aggregations, which share no kernel, must agree within float
+    rounding; a handful of vertices whose change sits at the eps threshold may freeze a superstep apart."""
+    from drone_amd import rmat
+    from drone_amd.pagerank import PRWorkerCUDA
+    torch = torch_cuda
+    x = rmat.pagerank_inputs_torch(23, 16, 6)
+    n = x["n"]
+    assert x["nnz"] > 100e6
+    u = x["col_idx"].cpu().numpy()
+    v = torch.repeat_interleave(torch.arange(n, device="cuda", dtype=torch.int32),
+                                torch.diff(x["row_ptr"])).cpu().numpy()
+    outdeg = x["outdeg"].to(torch.int32).cpu().numpy()
+    del x
+    runs = {}
+    for mode in ("merge-path", "row-blocks"):
+        if mode == "merge-path":
+            monkeypatch.setenv("DRONE_PR_ROWBLOCK_MIN_EDGES", str(1 << 40))
+        else:
+            monkeypatch.delenv("DRONE_PR_ROWBLOCK_MIN_EDGES")      # the library's own choice
+        w = PRWorkerCUDA(n, u, v, outdeg)
+        visited = [w.peval().VisitedSize] + [w.incEval().VisitedSize for _ in range(5)]
+        assert w.aggregation() == mode
+        runs[mode] = (visited, w.state())
+        w.close()
+    (vis_a, a), (vis_b, b) = runs["merge-path"], runs["row-blocks"]
+    assert vis_a[0] == vis_b[0] and vis_a[1] == vis_b[1]
+    assert max(abs(p - q) for p, q in zip(vis_a, vis_b)) <= 1e-4 * n
+    np.testing.assert_allclose(b["pr"], a["pr"], rtol=2e-5)
+    np.testing.assert_allclose(b["acc"], a["acc"], rtol=2e-5, atol=1e-6)
+    np.testing.assert_allclose(b["diff"], a["diff"], rtol=1e-4, atol=2e-6)
+    assert np.mean(b["active"] != a["active"]) <= 1e-4
 
 
 def test_push_path_converges_to_pull_ranks(torch_cuda, oracle, push_aggregation):
