@@ -183,11 +183,12 @@ void exchange_push(Graph *g, PRValues *values, int workerId, int workerNum, Comm
 
 // Subgraphs with at least this many edges get source-sorted row blocks for the aggregation.  One superstep at
 // R-MAT scale 20 / 21 / 22 / 23 / 24 (16 ... 263 M edges) takes 0.12 / 0.17 / 0.26 / 0.43 / 0.77 ms with them and
-// 0.12 / 0.20 / 0.39 / 0.78 / 1.65 ms on the merge path, but building them at the first PR_PEVal costs about
-// 23 / 32 / 47 ms at scale 22 / 23 / 24, i.e. 175 / 90 / 55 supersteps' worth of the saving.  The default
-// keeps the merge path (whose sums are also added in a fixed order) until a PageRank run of a hundred supersteps gets
-// the build back; DRONE_PR_ROWBLOCK_MIN_EDGES in the environment moves the limit for jobs that run longer or shorter.
-constexpr int64_t kRowBlockMinEdges = 96ll << 20;
+// 0.12 / 0.20 / 0.39 / 0.78 / 1.65 ms on the merge path; building them at the first PR_PEVal costs 8 / 12 / 22 ms
+// at scale 22 / 23 / 24 (and 15 ms more in a process that has not run these kernels yet), i.e. 65 / 35 / 25
+// supersteps' worth of the saving.  The default keeps the merge path (whose sums are also added in a fixed order)
+// until a PageRank run of fifty to a hundred supersteps gets the build back; DRONE_PR_ROWBLOCK_MIN_EDGES in the
+// environment moves the limit for jobs that run longer or shorter.
+constexpr int64_t kRowBlockMinEdges = 64ll << 20;
 
 int64_t row_block_min_edges()
 {

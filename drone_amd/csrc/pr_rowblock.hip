@@ -57,64 +57,127 @@ __global__ void rb_walk_len_kernel(const int64_t *__restrict__ row_ptr, int num_
     walk_len[b] = wl;
 }
 
-// One work-group per block: key = (block << 32) | source, value = row relative to the block's first row.  The
-// block's row starts (relative to its first entry, so 32 bits) sit in LDS for the per-entry binary search.
-constexpr int kKeysThreads = 1024;
-__global__ __launch_bounds__(kKeysThreads) void rb_keys_kernel(const int64_t *__restrict__ row_ptr,
-                                                               const int32_t *__restrict__ col,
-                                                               const int32_t *__restrict__ block_row,
-                                                               const int64_t *__restrict__ block_nnz,
-                                                               uint64_t *__restrict__ keys, uint16_t *__restrict__ lrow)
+// Sort keys, by position: a work-group owns kKeysChunk consecutive entries (so a block of millions of entries is
+// shared by many work-groups), finds the rows and the block they start in with binary searches, keeps those rows'
+// starts in LDS, and every entry then finds its row by a search in LDS.  key = (block << col_bits) | source, value =
+// row relative to the block's first row.  A chunk that spans more rows than the LDS table holds (a long run of empty
+// rows) searches the row starts in global memory instead.  (One work-group per block took 9.9 ms for 263 M entries.)
+constexpr int kKeysChunk = 4096;
+constexpr int kKeysRows = 4096;
+__device__ __forceinline__ int64_t last_start_at_or_before(const int64_t *__restrict__ starts, int64_t lo, int64_t hi,
+                                                           int64_t p)
 {
-    __shared__ int32_t s_start[kRbRows + 2];  // row r0 + i starts at entry e0 + s_start[i] (clamped to the block)
-    const int b = blockIdx.x;
-    const int r0 = block_row[b], r1 = block_row[b + 1];
-    const int64_t e0 = block_nnz[b], e1 = block_nnz[b + 1];
-    const int rows = r1 - r0 + 1;  // rows r0 .. r1 may own entries of the block (r1: the row left open)
-    for (int i = threadIdx.x; i < rows; i += kKeysThreads) {
-        const int64_t st = row_ptr[r0 + i] - e0;
-        s_start[i] = st < 0 ? 0 : st > e1 - e0 ? (int32_t)(e1 - e0) : (int32_t)st;
+    while (lo < hi) {  // largest i in [lo, hi] with starts[i] <= p
+        const int64_t mid = (lo + hi + 1) >> 1;
+        if (starts[mid] <= p) lo = mid; else hi = mid - 1;
     }
+    return lo;
+}
+
+template <typename Key>
+__global__ __launch_bounds__(256) void rb_keys_kernel(const int64_t *__restrict__ row_ptr,
+                                                      const int32_t *__restrict__ col, int64_t n, int64_t nnz,
+                                                      int num_blocks, const int32_t *__restrict__ block_row,
+                                                      const int64_t *__restrict__ block_nnz, int col_bits,
+                                                      Key *__restrict__ keys, uint16_t *__restrict__ lrow)
+{
+    __shared__ int64_t s_start[kKeysRows];
+    __shared__ int64_t s_range[3];
+    const int64_t p0 = (int64_t)blockIdx.x * kKeysChunk;
+    const int64_t p1 = p0 + kKeysChunk < nnz ? p0 + kKeysChunk : nnz;
+    if (threadIdx.x == 0) s_range[0] = last_start_at_or_before(row_ptr, 0, n - 1, p0);
+    if (threadIdx.x == kWave) s_range[1] = last_start_at_or_before(row_ptr, 0, n - 1, p1 - 1);
+    if (threadIdx.x == 2 * kWave) s_range[2] = last_start_at_or_before(block_nnz, 0, num_blocks - 1, p0);
     __syncthreads();
-    for (int64_t e = e0 + threadIdx.x; e < e1; e += kKeysThreads) {
-        const int32_t off = (int32_t)(e - e0);
-        int lo = 0, hi = rows - 1;  // largest i with s_start[i] <= off
-        while (lo < hi) {
-            const int mid = (lo + hi + 1) >> 1;
-            if (s_start[mid] <= off) lo = mid; else hi = mid - 1;
+    const int64_t ra = s_range[0], rz = s_range[1];
+    const int rows = (int)(rz - ra + 1 <= kKeysRows ? rz - ra + 1 : 0);  // 0: the table does not fit
+    for (int r = threadIdx.x; r < rows; r += blockDim.x) s_start[r] = row_ptr[ra + r];
+    __syncthreads();
+    for (int64_t p = p0 + threadIdx.x; p < p1; p += blockDim.x) {
+        int64_t row;
+        if (rows > 0) {
+            int lo = 0, hi = rows - 1;
+            while (lo < hi) {
+                const int mid = (lo + hi + 1) >> 1;
+                if (s_start[mid] <= p) lo = mid; else hi = mid - 1;
+            }
+            row = ra + lo;
+        } else {
+            row = last_start_at_or_before(row_ptr, ra, rz, p);
         }
-        keys[e] = ((uint64_t)b << 32) | (uint32_t)col[e];
-        lrow[e] = (uint16_t)lo;
+        int b = (int)s_range[2];
+        while (p >= block_nnz[b + 1]) ++b;  // the chunk crosses few block boundaries; empty blocks are stepped over
+        keys[p] = (Key)(((uint64_t)b << col_bits) | (uint32_t)col[p]);
+        lrow[p] = (uint16_t)(row - block_row[b]);
     }
 }
 
-// One lane per entry, one wavefront per 64-entry batch of a block's sorted entries: col = the key's source,
-// base = first source of the batch, packed = lrow << 16 | (source - base); a batch that spans more than 65,535 ids
-// flags its block as wide.
-__global__ __launch_bounds__(1024) void rb_pack_kernel(const int64_t *__restrict__ block_nnz,
-                                                       const int32_t *__restrict__ block_batch,
-                                                       const uint64_t *__restrict__ keys_sorted,
+// One lane per entry, one wavefront per 64-entry batch of a block's sorted entries (the batches of all blocks are
+// numbered through; a wavefront finds its batch's block by a search over the blocks' first batches): col = the key's
+// source, base = first source of the batch, packed = lrow << 16 | (source - base); a batch that spans more than
+// 65,535 ids flags its block as wide.  (One work-group per block took 8.4 ms for 263 M entries.)
+template <typename Key>
+__global__ __launch_bounds__(1024) void rb_pack_kernel(int num_blocks, int total_batches,
+                                                       const int64_t *__restrict__ block_nnz,
+                                                       const int32_t *__restrict__ block_batch, int col_bits,
+                                                       const Key *__restrict__ keys_sorted,
                                                        const uint16_t *__restrict__ lrow, int32_t *__restrict__ col,
                                                        uint32_t *__restrict__ packed, int32_t *__restrict__ batch_base,
                                                        int32_t *__restrict__ block_wide)
 {
-    const int b = blockIdx.x;
-    const int64_t e0 = block_nnz[b], e1 = block_nnz[b + 1];
     const int lane = threadIdx.x & (kWave - 1);
-    bool overflow = false;
-    for (int64_t s = e0 + (int64_t)(threadIdx.x - lane); s < e1; s += blockDim.x) {  // s: start of this wavefront's batch
-        const int64_t e = s + lane;
-        const int32_t c = e < e1 ? (int32_t)(keys_sorted[e] & 0xFFFFFFFFull) : 0;
-        const int32_t base = __shfl(c, 0, kWave);  // sources ascend inside a block
-        if (e < e1) {
-            const int32_t off = c - base;
-            overflow |= off > 0xFFFF;
-            col[e] = c;
-            packed[e] = ((uint32_t)lrow[e] << 16) | (uint32_t)(off & 0xFFFF);
-        }
-        if (lane == 0) batch_base[block_batch[b] + (int32_t)((s - e0) >> 6)] = base;
+    const int batch = (int)(((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave);
+    if (batch >= total_batches) return;  // the same for the whole wavefront
+    int lo = 0, hi = num_blocks - 1;     // largest b with block_batch[b] <= batch; empty blocks own no batch
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (block_batch[mid] <= batch) lo = mid; else hi = mid - 1;
     }
-    if (__any(overflow) && lane == 0) block_wide[b] = 1;
+    const int b = lo;
+    const int64_t e1 = block_nnz[b + 1];
+    const int64_t e = block_nnz[b] + (int64_t)(batch - block_batch[b]) * kWave + lane;
+    const uint32_t col_mask = col_bits >= 32 ? 0xFFFFFFFFu : ((1u << col_bits) - 1u);
+    const int32_t c = e < e1 ? (int32_t)((uint32_t)keys_sorted[e] & col_mask) : 0;
+    const int32_t base = __shfl(c, 0, kWave);  // sources ascend inside a block
+    bool overflow = false;
+    if (e < e1) {
+        const int32_t off = c - base;
+        overflow = off > 0xFFFF;
+        col[e] = c;
+        packed[e] = ((uint32_t)lrow[e] << 16) | (uint32_t)(off & 0xFFFF);
+    }
+    if (lane == 0) batch_base[batch] = base;
+    if (__any(overflow) && lane == 0) block_wide[b] = 1;  // every writer stores the same value
+}
+
+// Sorts the entries by (block, source) and derives the packed entry format.
+template <typename Key>
+int rb_sort_and_pack(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_ptr, const int32_t *col, int nb,
+                     int col_bits, int key_bits, int total_batches, void **scratch, hipStream_t stream)
+{
+    // scratch[0..3]: keys, sorted keys, unsorted local rows, the sort's workspace (freed by the caller)
+    Key *keys = nullptr, *keys_sorted = nullptr;
+    uint16_t *lrow_in = nullptr;
+    void *temp = nullptr;
+    size_t temp_bytes = 0;
+    const size_t e = (size_t)nnz;
+    DRONE_HIP_TRY(hipMalloc(&keys, sizeof(Key) * e));
+    scratch[0] = keys;
+    DRONE_HIP_TRY(hipMalloc(&keys_sorted, sizeof(Key) * e));
+    scratch[1] = keys_sorted;
+    DRONE_HIP_TRY(hipMalloc(&lrow_in, sizeof(uint16_t) * e));
+    scratch[2] = lrow_in;
+    rb_keys_kernel<Key><<<(unsigned)ceil_div(nnz, (int64_t)kKeysChunk), 256, 0, stream>>>(
+        row_ptr, col, n, nnz, nb, rb->block_row, rb->block_nnz, col_bits, keys, lrow_in);
+    DRONE_HIP_TRY(rocprim::radix_sort_pairs(nullptr, temp_bytes, keys, keys_sorted, lrow_in, rb->lrow, e, 0, key_bits, stream));
+    DRONE_HIP_TRY(hipMalloc(&temp, temp_bytes ? temp_bytes : 1));
+    scratch[3] = temp;
+    DRONE_HIP_TRY(rocprim::radix_sort_pairs(temp, temp_bytes, keys, keys_sorted, lrow_in, rb->lrow, e, 0, key_bits, stream));
+    rb_pack_kernel<Key><<<(unsigned)ceil_div((int64_t)total_batches * kWave, (int64_t)1024), 1024, 0, stream>>>(
+        nb, total_batches, rb->block_nnz, rb->block_batch, col_bits, keys_sorted, rb->lrow, rb->col, rb->packed,
+        rb->batch_base, rb->block_wide);
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
 }
 
 }  // namespace
@@ -145,10 +208,7 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
     const int64_t total = (int64_t)weight * n + nnz;
     int nb = (int)ceil_div(total, items);  // blocks of the weighted split; fewer once neighbours are merged
     rb->num_blocks = nb;
-    uint64_t *keys = nullptr, *keys_sorted = nullptr;
-    uint16_t *lrow_in = nullptr;
-    void *temp = nullptr;
-    size_t temp_bytes = 0;
+    void *scratch[4] = {nullptr, nullptr, nullptr, nullptr};  // temporaries of the sort
     auto body = [&]() -> int {
         const size_t e = (size_t)(nnz ? nnz : 1);
         DRONE_HIP_TRY(hipMalloc(&rb->block_row, sizeof(int32_t) * ((size_t)nb + 1)));
@@ -186,18 +246,7 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
             DRONE_HIP_TRY(hipStreamSynchronize(stream));  // br / bn go out of scope
         }
         rb_walk_len_kernel<<<(int)ceil_div(nb, 256), 256, 0, stream>>>(row_ptr, nb, rb->block_row, rb->block_nnz, rb->walk_len);
-        if (nnz > 0) {
-            DRONE_HIP_TRY(hipMalloc(&keys, sizeof(uint64_t) * e));
-            DRONE_HIP_TRY(hipMalloc(&keys_sorted, sizeof(uint64_t) * e));
-            DRONE_HIP_TRY(hipMalloc(&lrow_in, sizeof(uint16_t) * e));
-            rb_keys_kernel<<<nb, kKeysThreads, 0, stream>>>(row_ptr, col, rb->block_row, rb->block_nnz, keys, lrow_in);
-            int bits = 32;
-            while (bits < 64 && (1ull << (bits - 32)) < (unsigned long long)nb) ++bits;
-            DRONE_HIP_TRY(rocprim::radix_sort_pairs(nullptr, temp_bytes, keys, keys_sorted, lrow_in, rb->lrow, (size_t)nnz, 0, bits, stream));
-            DRONE_HIP_TRY(hipMalloc(&temp, temp_bytes ? temp_bytes : 1));
-            DRONE_HIP_TRY(rocprim::radix_sort_pairs(temp, temp_bytes, keys, keys_sorted, lrow_in, rb->lrow, (size_t)nnz, 0, bits, stream));
-        }
-        // packed 4-byte entries
+        // packed 4-byte entries: the blocks' 64-entry batches are numbered through
         DRONE_HIP_TRY(hipMalloc(&rb->block_batch, sizeof(int32_t) * ((size_t)nb + 1)));
         DRONE_HIP_TRY(hipMalloc(&rb->block_wide, sizeof(int32_t) * (size_t)nb));
         DRONE_HIP_TRY(hipMalloc(&rb->packed, sizeof(uint32_t) * e));
@@ -209,9 +258,17 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
         for (int b = 0; b < nb; ++b) h_batch[b + 1] = h_batch[b] + (int32_t)ceil_div(h_nnz[b + 1] - h_nnz[b], 64);
         DRONE_HIP_TRY(hipMalloc(&rb->batch_base, sizeof(int32_t) * (size_t)(h_batch[nb] ? h_batch[nb] : 1)));
         DRONE_HIP_TRY(hipMemcpyAsync(rb->block_batch, h_batch.data(), sizeof(int32_t) * h_batch.size(), hipMemcpyHostToDevice, stream));
-        if (nnz > 0)
-            rb_pack_kernel<<<nb, 1024, 0, stream>>>(rb->block_nnz, rb->block_batch, keys_sorted, rb->lrow, rb->col, rb->packed,
-                                                   rb->batch_base, rb->block_wide);
+        if (nnz > 0) {
+            // key = (block << col_bits) | source: 32-bit keys where they fit (half the sort's traffic)
+            int col_bits = 1, block_bits = 1;
+            while (col_bits < 32 && (1ll << col_bits) < n) ++col_bits;
+            while (block_bits < 31 && (1ll << block_bits) < nb) ++block_bits;
+            const int key_bits = col_bits + block_bits;
+            const int rc = key_bits <= 32
+                               ? rb_sort_and_pack<uint32_t>(rb, n, nnz, row_ptr, col, nb, col_bits, key_bits, h_batch[nb], scratch, stream)
+                               : rb_sort_and_pack<uint64_t>(rb, n, nnz, row_ptr, col, nb, col_bits, key_bits, h_batch[nb], scratch, stream);
+            if (rc != DRONE_OK) return rc;
+        }
         // work units: a block is shared by as many work-groups as it holds unit_items entries (at most `split`)
         std::vector<int32_t> h_row((size_t)nb + 1);
         DRONE_HIP_TRY(hipMemcpyAsync(h_row.data(), rb->block_row, sizeof(int32_t) * h_row.size(), hipMemcpyDeviceToHost, stream));
@@ -256,10 +313,7 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
         return DRONE_OK;
     };
     const int rc = body();
-    (void)hipFree(keys);
-    (void)hipFree(keys_sorted);
-    (void)hipFree(lrow_in);
-    (void)hipFree(temp);
+    for (void *p : scratch) (void)hipFree(p);
     if (rc != DRONE_OK) row_blocks_destroy(rb);
     return rc;
 }

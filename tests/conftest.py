@@ -22,7 +22,7 @@ def oracle():
 @pytest.fixture(params=["merge-path", "row-blocks"])
 def push_aggregation(request, monkeypatch):
     """Which kernels PR_PEVal / PR_IncEVal aggregate with.  The library picks by subgraph size (row blocks from about
-    100 M edges); the environment variable moves the limit, so small test graphs can take the large-graph path."""
+    67 M edges); the environment variable moves the limit, so small test graphs can take the large-graph path."""
     if request.param == "row-blocks":
         monkeypatch.setenv("DRONE_PR_ROWBLOCK_MIN_EDGES", "1")
     else:
