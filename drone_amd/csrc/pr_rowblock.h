@@ -1,4 +1,5 @@
-// Row-block pull aggregation with source-sorted entries and LDS accumulators (fp64 PageRank fast path).
+// Row-block pull aggregation with source-sorted entries and LDS accumulators (fp64 PageRank, and the float
+// delta-push supersteps of large subgraphs).
 //
 // Why: an 8-byte gather costs a whole 128-byte line on its way from L2 (or beyond) to the CU, so the gather
 // stream is priced by distinct lines per unit time, not by bytes.  In row order, consecutive gathers hit
