@@ -288,6 +288,41 @@ def bench_traverse(cpu_baseline=True):
     return out
 
 
+def bench_push(x, supersteps=20):
+    """The reference's own entry points on the benchmark graph as ONE subgraph: build_graph + loadOutDegree, then
+    PR_PEVal and `supersteps` x PR_IncEVal (float delta-push state, alpha 0.85, eps 1e-6).  x: the device CSR of the
+    headline run; its edge list goes through the host, as the Go worker hands it over.  Times are host wall-clock
+    around each call, which is what the worker sees (a call ends with the host reading VisitedSize)."""
+    import numpy as np
+    import torch
+    from drone_amd.pagerank import PRWorkerCUDA
+    n, nnz = x["n"], x["nnz"]
+    u = x["col_idx"].cpu().numpy()
+    v = torch.repeat_interleave(torch.arange(n, device="cuda", dtype=torch.int32), torch.diff(x["row_ptr"])).cpu().numpy()
+    outdeg = x["outdeg"].to(torch.int32).cpu().numpy()
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    w = PRWorkerCUDA(n, u, v, outdeg)
+    build_s = time.perf_counter() - t
+    t = time.perf_counter()
+    first = w.peval()
+    peval_ms = (time.perf_counter() - t) * 1e3
+    ms, visited = [], []
+    for _ in range(supersteps):
+        t = time.perf_counter()
+        r = w.incEval()
+        ms.append((time.perf_counter() - t) * 1e3)
+        visited.append(int(r.VisitedSize))
+    med = float(np.median(ms))
+    out = {"workload": f"PR_PEVal + {supersteps} x PR_IncEVal on the same graph as one subgraph (N={n}, E={nnz}, "
+                       f"{w.n} vertices with edges), float32 delta-push, eps 1e-6",
+           "aggregation": w.aggregation(), "build_graph_s": build_s, "peval_ms_incl_one_off_setup": peval_ms,
+           "inceval_ms_median": med, "inceval_ms_min": float(min(ms)), "GTEPS": nnz / (med * 1e-3) / 1e9,
+           "visited_first_last": [int(first.VisitedSize), visited[-1]]}
+    w.close()
+    return out
+
+
 def bench_exchange():
     """Four subgraphs of a random vertex cut of R-MAT scale 20 (ef 16, seed 2) on one GPU, each worker on its own host
     thread over the in-process loopback transport: PR_PEVal + 5 x PR_IncEVal with the two exchange phases per
@@ -371,7 +406,8 @@ def main():
                     help="launch the 1 GiB stream-copy kernel exactly once (a dispatch of known traffic to scale "
                          "rocprofv3 byte counters by)")
     ap.add_argument("--suite", default="default", choices=["pr", "default", "full", "gcn", "sweep", "traverse", "exchange"],
-                    help="pr: PageRank only; default: + GCN training step (configs[3]); full: + configs[2], [4] and the "
+                    help="pr: PageRank only (fp64 pull plan, then the reference's PR_PEVal / PR_IncEVal on the same "
+                         "graph); default: + GCN training step (configs[3]); full: + configs[2], [4] and the "
                          "SSSP / CC jobs and the replica exchange; gcn, sweep, traverse, exchange: that part alone")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -465,7 +501,14 @@ def main():
         result["cpu_baseline"] = pull
         result["cpu_baseline_drone_go_path"] = go
     plan.close()
-    del x, out, plan
+    del out, plan
+    torch.cuda.empty_cache()
+    result["reference_entry_points"] = bench_push(x)
+    log(f"PR_IncEVal ({result['reference_entry_points']['aggregation']}): "
+        f"{result['reference_entry_points']['inceval_ms_median']:.3f} ms per superstep = "
+        f"{result['reference_entry_points']['GTEPS']:.0f} GTEPS; first PR_PEVal "
+        f"{result['reference_entry_points']['peval_ms_incl_one_off_setup']:.1f} ms")
+    del x
     torch.cuda.empty_cache()
     if args.suite in ("default", "full"):
         result["gcn_step"] = bench_gcn_step(steps=max(3, args.steps), warmup=max(1, args.warmup),
