@@ -314,10 +314,15 @@ def bench_push(x, supersteps=20):
         ms.append((time.perf_counter() - t) * 1e3)
         visited.append(int(r.VisitedSize))
     med = float(np.median(ms))
+    # compulsory traffic of one superstep's aggregation: in-edge sources 4E, in-edge offsets 4(N+1), push vector 4N
+    # read; diff and active 4N each written (int32 / float32 throughout, N = local vertices)
+    algo = 4 * nnz + 4 * (w.n + 1) + 12 * w.n
     out = {"workload": f"PR_PEVal + {supersteps} x PR_IncEVal on the same graph as one subgraph (N={n}, E={nnz}, "
                        f"{w.n} vertices with edges), float32 delta-push, eps 1e-6",
            "aggregation": w.aggregation(), "build_graph_s": build_s, "peval_ms_incl_one_off_setup": peval_ms,
            "inceval_ms_median": med, "inceval_ms_min": float(min(ms)), "GTEPS": nnz / (med * 1e-3) / 1e9,
+           "algorithmic_bytes_per_superstep": algo, "achieved_GBps": algo / (med * 1e-3) / 1e9,
+           "frac_of_hbm_peak": algo / (med * 1e-3) / 1e9 / HBM_PEAK_GBS,
            "visited_first_last": [int(first.VisitedSize), visited[-1]]}
     w.close()
     return out
