@@ -182,9 +182,9 @@ void exchange_push(Graph *g, PRValues *values, int workerId, int workerNum, Comm
 }
 
 // Subgraphs with at least this many edges get source-sorted row blocks for the aggregation.  One superstep at
-// R-MAT scale 20 / 21 / 22 / 23 / 24 (16 ... 263 M edges) takes 0.12 / 0.17 / 0.26 / 0.43 / 0.77 ms with them and
+// R-MAT scale 20 / 21 / 22 / 23 / 24 (16 ... 263 M edges) takes 0.13 / 0.17 / 0.24 / 0.38 / 0.70 ms with them and
 // 0.12 / 0.20 / 0.39 / 0.78 / 1.65 ms on the merge path; building them at the first PR_PEVal costs 8 / 12 / 22 ms
-// at scale 22 / 23 / 24 (and 15 ms more in a process that has not run these kernels yet), i.e. 65 / 35 / 25
+// at scale 22 / 23 / 24 (and 15 ms more in a process that has not run these kernels yet), i.e. 55 / 30 / 23
 // supersteps' worth of the saving.  The default keeps the merge path (whose sums are also added in a fixed order)
 // until a PageRank run of fifty to a hundred supersteps gets the build back; DRONE_PR_ROWBLOCK_MIN_EDGES in the
 // environment moves the limit for jobs that run longer or shorter.
@@ -233,7 +233,7 @@ void ensure_row_blocks(Graph *g, hipStream_t s)
         rc = relabel_create(&rl, x->n, x->edges, row_ptr, x->in_src, nullptr, s, /*keep_rows=*/true, g->index);
     }
     (void)hipFree(row_ptr);
-    if (rc == DRONE_OK) rc = row_blocks_create(&x->rb, x->n, x->edges, rl.row_ptr, rl.col, 2, s);
+    if (rc == DRONE_OK) rc = row_blocks_create(&x->rb, x->n, x->edges, rl.row_ptr, rl.col, 2, s, /*uniform_rows=*/true);
     if (rc == DRONE_OK) {
         if (hipMalloc(&x->rb_new_id, sizeof(int32_t) * (size_t)x->n) != hipSuccess) rc = DRONE_ERR_HIP;
         else invert_order_kernel<<<1024, 256, 0, s>>>(rl.order, x->n, x->rb_new_id);

@@ -68,8 +68,9 @@ struct RowBlocks {
 
 // Builds the blocks for a CSR with device row_ptr / col (already in the plan's internal id space).
 // shared_blocks: 0 = decide by size, 1 = never split a block, 2 = split whenever a block is large enough.
+// uniform_rows: the rows are in no particular order (not sorted by length), so all blocks will look alike.
 int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_ptr, const int32_t *col,
-                      int shared_blocks, hipStream_t stream);
+                      int shared_blocks, hipStream_t stream, bool uniform_rows = false);
 void row_blocks_destroy(RowBlocks *rb);
 
 __device__ __forceinline__ int64_t ceil_div_dev(int64_t a, int64_t b) { return (a + b - 1) / b; }

@@ -183,7 +183,7 @@ int rb_sort_and_pack(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_p
 }  // namespace
 
 int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_ptr, const int32_t *col,
-                      int shared_blocks, hipStream_t stream)
+                      int shared_blocks, hipStream_t stream, bool uniform_rows)
 {
     DRONE_REQUIRE(n > 0 && n < INT32_MAX && nnz >= 0 && nnz < (int64_t)UINT32_MAX, "sizes");
     rb->n = n;
@@ -196,6 +196,11 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
     DRONE_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
     int items = 32768;
     while (items < kRbMaxItems && (double)items * 1.41421356 < (double)nnz / (cus > 0 ? cus : 256)) items <<= 1;
+    // Rows in an order unrelated to their length give blocks that all look alike (about 16,384 rows each, nobody
+    // reaches the entry capacity), and then half the capacity balances the CUs better: one float delta-push
+    // superstep at R-MAT scale 22 / 24 took 0.25 / 0.80 ms with 128 K entries per work-group, 0.26 / 0.73 with 256 K,
+    // 0.34 / 0.70 with 512 K, - / 0.77 with 1 M (the rule above picks 256 K / 1 M).
+    if (uniform_rows && items > 32768) items >>= 1;
     const int unit_items = items;          // entries one work-group sweeps
     // Large matrices get blocks that several work-groups share.  Measured, ms per iteration at R-MAT scale 20 / 22 /
     // 24: with blocks of the weighted split alone and 1 / 2 / 4 / 8 / 16 work-groups per block 0.060 0.063 0.079
