@@ -196,6 +196,12 @@ __global__ __launch_bounds__(kWave * kRowsPerBlock) void spmm_rows_kernel(
 
 // One wavefront per band piece of a long row (work list in band-major order): partial[slot, 0..K) = sum over
 // the piece.  ci / val are the plan's (band,row)-sorted copies.
+// Short pieces are dear: launched band by band on the 229 M-entry graph (K = 128), the bands whose pieces hold 100
+// entries and more cost 25 ps per entry, those with 55-entry pieces 48 ps, those with 20-entry pieces 80 - 100 ps,
+// the cold band 84 ps - a piece is a chain of dependent round trips (bounds, (col, val) pairs, feature rows) however
+// short it is.  Giving a wavefront 2 / 4 / 8 consecutive pieces, their bounds read with one load and the next piece's
+// pairs fetched ahead, made the product slower, 4.48 / 4.71 / 5.16 against 4.43 ms: the extra live values cost
+// occupancy (76 VGPRs, 6 instead of 8 wavefronts per SIMD; capped at 64 VGPRs it spills, 5.17 ms).
 template <int G, int VEC>
 __global__ __launch_bounds__(kWave * kRowsPerBlock) void spmm_pieces_kernel(
     int num_pieces, const int *__restrict__ piece_begin, const int *__restrict__ piece_end,
