@@ -66,6 +66,11 @@ def small_cases():
     keep = src != dst
     pairs = np.unique(np.stack([src[keep], dst[keep]], 1), axis=0)
     cases["ragged"] = (20000, pairs[:, 0], pairs[:, 1])
+    # few entries among very many rows: a chunk of consecutive entries spans more rows than the set-up kernels keep in LDS
+    s_, d_ = rng.integers(0, 200000, 3000), rng.integers(0, 200000, 3000)
+    k_ = s_ != d_
+    pw = np.unique(np.stack([s_[k_], d_[k_]], 1), axis=0)
+    cases["sparse_wide"] = (200000, pw[:, 0], pw[:, 1])
     # exactly one tile of items (n + nnz = 2048) and one more than a tile
     for name, tot in (("one_tile_exact", 2048), ("one_tile_plus_one", 2049)):
         nn = 512
