@@ -274,7 +274,10 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
                                : rb_sort_and_pack<uint64_t>(rb, n, nnz, row_ptr, col, nb, col_bits, key_bits, h_batch[nb], scratch, stream);
             if (rc != DRONE_OK) return rc;
         }
-        // work units: a block is shared by as many work-groups as it holds unit_items entries (at most `split`)
+        // work units: a block is shared by as many work-groups as it holds unit_items entries (at most `split`).
+        // The units are numbered block by block, so the work-groups of one block spread over the XCDs (work-groups go
+        // to the XCDs round-robin); numbering eight blocks share-major, which puts a block's work-groups on one XCD
+        // where they could find each other's source lines in L2, measured 0.590 against 0.572 ms per iteration.
         std::vector<int32_t> h_row((size_t)nb + 1);
         DRONE_HIP_TRY(hipMemcpyAsync(h_row.data(), rb->block_row, sizeof(int32_t) * h_row.size(), hipMemcpyDeviceToHost, stream));
         DRONE_HIP_TRY(hipStreamSynchronize(stream));
