@@ -202,6 +202,8 @@ __global__ __launch_bounds__(kWave * kRowsPerBlock) void spmm_rows_kernel(
 // short it is.  Giving a wavefront 2 / 4 / 8 consecutive pieces, their bounds read with one load and the next piece's
 // pairs fetched ahead, made the product slower, 4.48 / 4.71 / 5.16 against 4.43 ms: the extra live values cost
 // occupancy (76 VGPRs, 6 instead of 8 wavefronts per SIMD; capped at 64 VGPRs it spills, 5.17 ms).
+// One piece per lane group (two or four pieces side by side in a wavefront, nothing folded across groups) lost too:
+// 4.78 / 3.00 ms for K = 128 / 41 against 4.44 / 2.60 - the wavefront runs as long as its longest piece.
 template <int G, int VEC>
 __global__ __launch_bounds__(kWave * kRowsPerBlock) void spmm_pieces_kernel(
     int num_pieces, const int *__restrict__ piece_begin, const int *__restrict__ piece_end,
