@@ -29,7 +29,9 @@
 // of the two kernels' measured costs (about 3 ps per dense cell, 24 ps per gathered entry at K = 128, both
 // proportional to K) and was then set by measurement on the 232,965-vertex / 229 M-entry graph (ms for K = 128 /
 // K = 41: no dense part 6.33 / 3.57; threshold 0.30: 5.39 / 3.02; 0.16: 4.94 / 2.72; 0.12: 4.90 / 2.70; 0.06:
-// 5.17 / 2.81).  Graphs without such a core (every chunk below the threshold) get no dense part.
+// 5.17 / 2.81; again with the later kernels: 0.045: 4.73 / 2.78; 0.06: 4.56 / 2.68; 0.08: 4.42 / 2.58; 0.10: 4.50 /
+// 2.62; 0.12: 4.45 / 2.59; 0.16: 4.58 / 2.67).  Graphs without such a core (every chunk below the threshold) get no
+// dense part.
 #include <algorithm>
 #include <cstring>
 #include <numeric>
