@@ -12,7 +12,7 @@
 // Schedule: rows of at most kSplitRow non-zeros get one wavefront each, in row order.  Longer rows carry
 // most of the non-zeros of power-law graphs and gather from all over B; run row by row their accesses miss
 // L2 (B is hundreds of MB, an XCD's L2 is 4 MB).  They are therefore cut by COLUMN BAND: columns are ranked by
-// how often they occur, a band is the set of columns whose feature rows fill about 2 MB (kBandBytes), the first
+// how often they occur, a band is the set of columns whose feature rows fill about 3 MB (kBandBytes), the first
 // kHotBands bands are kept apart and everything colder shares one last band.  The plan holds a copy of the
 // long rows' entries stably sorted by (band, row) and the resulting pieces (<= kChunk entries each) as a work
 // list in that order.  Work-groups are dispatched in list order, so at any moment the resident wavefronts
@@ -80,8 +80,12 @@ namespace {
 
 constexpr int kSplitRow = 512;          // rows with more non-zeros are cut into band pieces (256: 4.58 / 2.87 ms, 512: 4.45 / 2.60, 1024: 5.03 / 2.76 for K = 128 / 41 on the 229 M-entry graph)
 constexpr int kChunk = 2048;            // most non-zeros in one piece
-constexpr int kHotBands = 24;           // bands kept apart; colder columns share one more band
-constexpr size_t kBandBytes = 2u << 20; // feature rows of one band (half of an XCD's L2)
+constexpr int kHotBands = 20;           // bands kept apart; colder columns share one more band
+constexpr size_t kBandBytes = 3u << 20; // feature rows of one band (three quarters of an XCD's L2)
+// Band size x hot bands, ms for K = 128 / 41 on the 229 M-entry graph: 1 MB x 48: 4.90 / 3.02; 2 MB x 24: 4.44 / 2.59;
+// 2.5 MB x 19: 4.35 / 2.52; 3 MB x 16: 4.32 / 2.48; 3 MB x 20: 4.33 / 2.49; 3 MB x 24: 4.32 / 2.53; 4 MB x 12: 4.45 / 2.46.
+// With 2 MB bands, 10 / 15 / 24 / 32 hot bands: 5.44 / 4.83 / 4.44 / 4.44 ms (K = 128).
+constexpr int kBandMaxCols = 8192;      // narrow feature rows: a band is at most this many columns
 constexpr int kRowsPerBlock = 4;
 constexpr int kDenseChunk = 2048;       // column granularity of the dense rectangles
 constexpr int kDenseMaxCols = 32768;    // widest rectangle
@@ -455,6 +459,7 @@ int build_band_pieces(drone_spmm_plan *p, const std::vector<int> &h_rp, const st
     const int ld = (p->max_k + 3) / 4 * 4;
     int band_cols = (int)(kBandBytes / (sizeof(float) * (size_t)ld));
     if (band_cols < 64) band_cols = 64;
+    if (band_cols > kBandMaxCols) band_cols = kBandMaxCols;
     int num_bands = (int)ceil_div(p->n_cols, band_cols);
     if (num_bands > kHotBands + 1) num_bands = kHotBands + 1;
     if (num_bands < 1) num_bands = 1;
