@@ -79,7 +79,7 @@ namespace drone {
 namespace {
 
 constexpr int kSplitRow = 512;          // rows with more non-zeros are cut into band pieces (256: 4.58 / 2.87 ms, 512: 4.45 / 2.60, 1024: 5.03 / 2.76 for K = 128 / 41 on the 229 M-entry graph)
-constexpr int kChunk = 2048;            // most non-zeros in one piece
+constexpr int kChunk = 1024;            // most non-zeros in one piece (256 ... 4096 all within 2 %: 4.26 / 4.28 / 4.24 / 4.29 / 4.35 ms, K = 128)
 constexpr int kHotBands = 20;           // bands kept apart; colder columns share one more band
 constexpr size_t kBandBytes = 3u << 20; // feature rows of one band (three quarters of an XCD's L2)
 // Band size x hot bands, ms for K = 128 / 41 on the 229 M-entry graph: 1 MB x 48: 4.90 / 3.02; 2 MB x 24: 4.44 / 2.59;
