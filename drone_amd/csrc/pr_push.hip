@@ -183,7 +183,7 @@ void exchange_push(Graph *g, PRValues *values, int workerId, int workerNum, Comm
 
 // Subgraphs with at least this many edges get source-sorted row blocks for the aggregation.  One superstep at
 // R-MAT scale 20 / 21 / 22 / 23 / 24 (16 ... 263 M edges) takes 0.13 / 0.17 / 0.24 / 0.38 / 0.70 ms with them and
-// 0.12 / 0.20 / 0.39 / 0.78 / 1.65 ms on the merge path; building them at the first PR_PEVal costs 8 / 12 / 22 ms
+// 0.12 / 0.20 / 0.39 / 0.78 / 1.65 ms on the merge path; building them at the first PR_PEVal costs 8 / 12 / 18 ms
 // at scale 22 / 23 / 24 (and 15 ms more in a process that has not run these kernels yet), i.e. 55 / 30 / 23
 // supersteps' worth of the saving.  The default keeps the merge path (whose sums are also added in a fixed order)
 // until a PageRank run of fifty to a hundred supersteps gets the build back; DRONE_PR_ROWBLOCK_MIN_EDGES in the

@@ -59,8 +59,9 @@ __global__ void rb_walk_len_kernel(const int64_t *__restrict__ row_ptr, int num_
 
 // Sort keys, by position: a work-group owns kKeysChunk consecutive entries (so a block of millions of entries is
 // shared by many work-groups), finds the rows and the block they start in with binary searches, keeps those rows'
-// starts in LDS, and every entry then finds its row by a search in LDS.  key = (block << col_bits) | source, value =
-// row relative to the block's first row.  A chunk that spans more rows than the LDS table holds (a long run of empty
+// starts in LDS, and every entry then finds its row by a search in LDS.  key = ((block & block_mask) << col_bits) |
+// source (blocks are sorted in groups of block_mask + 1, see rb_sort_and_pack), value = row relative to the block's
+// first row.  A chunk that spans more rows than the LDS table holds (a long run of empty
 // rows) searches the row starts in global memory instead.  (One work-group per block took 9.9 ms for 263 M entries.)
 constexpr int kKeysChunk = 4096;
 constexpr int kKeysRows = 4096;
@@ -79,7 +80,8 @@ __global__ __launch_bounds__(256) void rb_keys_kernel(const int64_t *__restrict_
                                                       const int32_t *__restrict__ col, int64_t n, int64_t nnz,
                                                       int num_blocks, const int32_t *__restrict__ block_row,
                                                       const int64_t *__restrict__ block_nnz, int col_bits,
-                                                      Key *__restrict__ keys, uint16_t *__restrict__ lrow)
+                                                      int block_mask, Key *__restrict__ keys,
+                                                      uint16_t *__restrict__ lrow)
 {
     __shared__ int64_t s_start[kKeysRows];
     __shared__ int64_t s_range[3];
@@ -107,7 +109,7 @@ __global__ __launch_bounds__(256) void rb_keys_kernel(const int64_t *__restrict_
         }
         int b = (int)s_range[2];
         while (p >= block_nnz[b + 1]) ++b;  // the chunk crosses few block boundaries; empty blocks are stepped over
-        keys[p] = (Key)(((uint64_t)b << col_bits) | (uint32_t)col[p]);
+        keys[p] = (Key)(((uint64_t)(b & block_mask) << col_bits) | (uint32_t)col[p]);
         lrow[p] = (uint16_t)(row - block_row[b]);
     }
 }
@@ -150,16 +152,19 @@ __global__ __launch_bounds__(1024) void rb_pack_kernel(int num_blocks, int total
     if (__any(overflow) && lane == 0) block_wide[b] = 1;  // every writer stores the same value
 }
 
-// Sorts the entries by (block, source) and derives the packed entry format.
+// Sorts the entries by (block, source) and derives the packed entry format.  The entries arrive grouped by block
+// already, so consecutive blocks can be sorted as separate ranges: with `group` (a power of two) blocks per range the
+// key needs col_bits + log2(group) bits, which keeps large matrices on 32-bit keys (R-MAT scale 24, 263 M entries:
+// three ranges of 256 blocks and four 8-bit passes over 6-byte pairs instead of five over 10-byte pairs).
 template <typename Key>
 int rb_sort_and_pack(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_ptr, const int32_t *col, int nb,
-                     int col_bits, int key_bits, int total_batches, void **scratch, hipStream_t stream)
+                     int col_bits, int group, const std::vector<int64_t> &h_nnz, int total_batches, void **scratch,
+                     hipStream_t stream)
 {
     // scratch[0..3]: keys, sorted keys, unsorted local rows, the sort's workspace (freed by the caller)
     Key *keys = nullptr, *keys_sorted = nullptr;
     uint16_t *lrow_in = nullptr;
     void *temp = nullptr;
-    size_t temp_bytes = 0;
     const size_t e = (size_t)nnz;
     DRONE_HIP_TRY(hipMalloc(&keys, sizeof(Key) * e));
     scratch[0] = keys;
@@ -168,11 +173,28 @@ int rb_sort_and_pack(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_p
     DRONE_HIP_TRY(hipMalloc(&lrow_in, sizeof(uint16_t) * e));
     scratch[2] = lrow_in;
     rb_keys_kernel<Key><<<(unsigned)ceil_div(nnz, (int64_t)kKeysChunk), 256, 0, stream>>>(
-        row_ptr, col, n, nnz, nb, rb->block_row, rb->block_nnz, col_bits, keys, lrow_in);
-    DRONE_HIP_TRY(rocprim::radix_sort_pairs(nullptr, temp_bytes, keys, keys_sorted, lrow_in, rb->lrow, e, 0, key_bits, stream));
+        row_ptr, col, n, nnz, nb, rb->block_row, rb->block_nnz, col_bits, group - 1, keys, lrow_in);
+    int group_bits = 0;
+    while ((1 << group_bits) < group) ++group_bits;
+    size_t temp_bytes = 0;
+    for (int b0 = 0; b0 < nb; b0 += group) {  // the workspace of the largest range serves all
+        const int b1 = b0 + group < nb ? b0 + group : nb;
+        const size_t count = (size_t)(h_nnz[(size_t)b1] - h_nnz[(size_t)b0]);
+        size_t need = 0;
+        DRONE_HIP_TRY(rocprim::radix_sort_pairs(nullptr, need, keys, keys_sorted, lrow_in, rb->lrow, count, 0,
+                                                col_bits + group_bits, stream));
+        if (need > temp_bytes) temp_bytes = need;
+    }
     DRONE_HIP_TRY(hipMalloc(&temp, temp_bytes ? temp_bytes : 1));
     scratch[3] = temp;
-    DRONE_HIP_TRY(rocprim::radix_sort_pairs(temp, temp_bytes, keys, keys_sorted, lrow_in, rb->lrow, e, 0, key_bits, stream));
+    for (int b0 = 0; b0 < nb; b0 += group) {
+        const int b1 = b0 + group < nb ? b0 + group : nb;
+        const size_t first = (size_t)h_nnz[(size_t)b0], count = (size_t)(h_nnz[(size_t)b1] - h_nnz[(size_t)b0]);
+        if (count == 0) continue;
+        size_t bytes = temp_bytes;
+        DRONE_HIP_TRY(rocprim::radix_sort_pairs(temp, bytes, keys + first, keys_sorted + first, lrow_in + first,
+                                                rb->lrow + first, count, 0, col_bits + group_bits, stream));
+    }
     rb_pack_kernel<Key><<<(unsigned)ceil_div((int64_t)total_batches * kWave, (int64_t)1024), 1024, 0, stream>>>(
         nb, total_batches, rb->block_nnz, rb->block_batch, col_bits, keys_sorted, rb->lrow, rb->col, rb->packed,
         rb->batch_base, rb->block_wide);
@@ -264,14 +286,17 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
         DRONE_HIP_TRY(hipMalloc(&rb->batch_base, sizeof(int32_t) * (size_t)(h_batch[nb] ? h_batch[nb] : 1)));
         DRONE_HIP_TRY(hipMemcpyAsync(rb->block_batch, h_batch.data(), sizeof(int32_t) * h_batch.size(), hipMemcpyHostToDevice, stream));
         if (nnz > 0) {
-            // key = (block << col_bits) | source: 32-bit keys where they fit (half the sort's traffic)
+            // key = (block within its range << col_bits) | source: 32-bit keys while at most 64 ranges do it
             int col_bits = 1, block_bits = 1;
             while (col_bits < 32 && (1ll << col_bits) < n) ++col_bits;
             while (block_bits < 31 && (1ll << block_bits) < nb) ++block_bits;
-            const int key_bits = col_bits + block_bits;
-            const int rc = key_bits <= 32
-                               ? rb_sort_and_pack<uint32_t>(rb, n, nnz, row_ptr, col, nb, col_bits, key_bits, h_batch[nb], scratch, stream)
-                               : rb_sort_and_pack<uint64_t>(rb, n, nnz, row_ptr, col, nb, col_bits, key_bits, h_batch[nb], scratch, stream);
+            int group_bits = block_bits < 32 - col_bits ? block_bits : 32 - col_bits;
+            if (group_bits < 0) group_bits = 0;
+            const bool narrow = col_bits + group_bits <= 32 && ceil_div(nb, 1 << group_bits) <= 64;
+            const int rc = narrow ? rb_sort_and_pack<uint32_t>(rb, n, nnz, row_ptr, col, nb, col_bits, 1 << group_bits,
+                                                               h_nnz, h_batch[nb], scratch, stream)
+                                  : rb_sort_and_pack<uint64_t>(rb, n, nnz, row_ptr, col, nb, col_bits, 1 << block_bits,
+                                                               h_nnz, h_batch[nb], scratch, stream);
             if (rc != DRONE_OK) return rc;
         }
         // work units: a block is shared by as many work-groups as it holds unit_items entries (at most `split`).
