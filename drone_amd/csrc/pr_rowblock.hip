@@ -114,10 +114,12 @@ __global__ __launch_bounds__(256) void rb_keys_kernel(const int64_t *__restrict_
     }
 }
 
-// One lane per entry, one wavefront per 64-entry batch of a block's sorted entries (the batches of all blocks are
-// numbered through; a wavefront finds its batch's block by a search over the blocks' first batches): col = the key's
-// source, base = first source of the batch, packed = lrow << 16 | (source - base); a batch that spans more than
-// 65,535 ids flags its block as wide.  (One work-group per block took 8.4 ms for 263 M entries.)
+// One lane per entry, one wavefront per kPackBatches consecutive 64-entry batches of the blocks' sorted entries (the
+// batches of all blocks are numbered through; a wavefront finds its first batch's block by a search over the blocks'
+// first batches and steps to the next block from there): col = the key's source, base = first source of the batch,
+// packed = lrow << 16 | (source - base); a batch that spans more than 65,535 ids flags its block as wide.  (One
+// work-group per block took 8.4 ms for 263 M entries, a search per batch 2.8 ms.)
+constexpr int kPackBatches = 8;
 template <typename Key>
 __global__ __launch_bounds__(1024) void rb_pack_kernel(int num_blocks, int total_batches,
                                                        const int64_t *__restrict__ block_nnz,
@@ -128,28 +130,32 @@ __global__ __launch_bounds__(1024) void rb_pack_kernel(int num_blocks, int total
                                                        int32_t *__restrict__ block_wide)
 {
     const int lane = threadIdx.x & (kWave - 1);
-    const int batch = (int)(((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave);
-    if (batch >= total_batches) return;  // the same for the whole wavefront
-    int lo = 0, hi = num_blocks - 1;     // largest b with block_batch[b] <= batch; empty blocks own no batch
+    const int64_t first = (((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave) * kPackBatches;
+    if (first >= total_batches) return;  // the same for the whole wavefront
+    const int last = first + kPackBatches < total_batches ? (int)first + kPackBatches : total_batches;
+    int lo = 0, hi = num_blocks - 1;     // largest b with block_batch[b] <= first; empty blocks own no batch
     while (lo < hi) {
         const int mid = (lo + hi + 1) >> 1;
-        if (block_batch[mid] <= batch) lo = mid; else hi = mid - 1;
+        if (block_batch[mid] <= (int)first) lo = mid; else hi = mid - 1;
     }
-    const int b = lo;
-    const int64_t e1 = block_nnz[b + 1];
-    const int64_t e = block_nnz[b] + (int64_t)(batch - block_batch[b]) * kWave + lane;
+    int b = lo;
     const uint32_t col_mask = col_bits >= 32 ? 0xFFFFFFFFu : ((1u << col_bits) - 1u);
-    const int32_t c = e < e1 ? (int32_t)((uint32_t)keys_sorted[e] & col_mask) : 0;
-    const int32_t base = __shfl(c, 0, kWave);  // sources ascend inside a block
-    bool overflow = false;
-    if (e < e1) {
-        const int32_t off = c - base;
-        overflow = off > 0xFFFF;
-        col[e] = c;
-        packed[e] = ((uint32_t)lrow[e] << 16) | (uint32_t)(off & 0xFFFF);
+    for (int batch = (int)first; batch < last; ++batch) {
+        while (batch >= block_batch[b + 1]) ++b;  // block_batch[num_blocks] = total_batches ends the walk
+        const int64_t e1 = block_nnz[b + 1];
+        const int64_t e = block_nnz[b] + (int64_t)(batch - block_batch[b]) * kWave + lane;
+        const int32_t c = e < e1 ? (int32_t)((uint32_t)keys_sorted[e] & col_mask) : 0;
+        const int32_t base = __shfl(c, 0, kWave);  // sources ascend inside a block
+        bool overflow = false;
+        if (e < e1) {
+            const int32_t off = c - base;
+            overflow = off > 0xFFFF;
+            col[e] = c;
+            packed[e] = ((uint32_t)lrow[e] << 16) | (uint32_t)(off & 0xFFFF);
+        }
+        if (lane == 0) batch_base[batch] = base;
+        if (__any(overflow) && lane == 0) block_wide[b] = 1;  // every writer stores the same value
     }
-    if (lane == 0) batch_base[batch] = base;
-    if (__any(overflow) && lane == 0) block_wide[b] = 1;  // every writer stores the same value
 }
 
 // Sorts the entries by (block, source) and derives the packed entry format.  The entries arrive grouped by block
@@ -195,7 +201,7 @@ int rb_sort_and_pack(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_p
         DRONE_HIP_TRY(rocprim::radix_sort_pairs(temp, bytes, keys + first, keys_sorted + first, lrow_in + first,
                                                 rb->lrow + first, count, 0, col_bits + group_bits, stream));
     }
-    rb_pack_kernel<Key><<<(unsigned)ceil_div((int64_t)total_batches * kWave, (int64_t)1024), 1024, 0, stream>>>(
+    rb_pack_kernel<Key><<<(unsigned)ceil_div(ceil_div((int64_t)total_batches, (int64_t)kPackBatches) * kWave, (int64_t)1024), 1024, 0, stream>>>(
         nb, total_batches, rb->block_nnz, rb->block_batch, col_bits, keys_sorted, rb->lrow, rb->col, rb->packed,
         rb->batch_base, rb->block_wide);
     DRONE_HIP_TRY(hipGetLastError());
