@@ -29,6 +29,8 @@ constexpr int kRbThreads = 1024;
 // rows / 1 M entries 0.685; 16,384 / 512 K 0.72; 16,384 / 2 M 0.87 (too few heavy blocks for 256 CUs); 8,192 rows (two
 // blocks per CU) / 1 M 0.85, / 512 K 0.99.  Larger blocks reuse popular lines more often, but the blocks that are
 // full of entries must still cover the CUs: the entry capacity is chosen per graph (row_blocks_create).
+// 18,000 rows (141 KB of accumulators, all that fits beside the float entry points' bit mask) measured 0.574 against
+// 0.573 ms per fp64 iteration and 0.77 against 0.69 ms per float superstep with the current shared blocks.
 constexpr int kRbRows = 16384;       // most rows ending in one block (LDS accumulators: 128 KB)
 constexpr int kRbMaxItems = 1 << 20; // most entries in one block (the plan picks a power of two up to this)
 constexpr int kRbUnroll = 4;
