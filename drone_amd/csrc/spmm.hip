@@ -86,7 +86,7 @@ constexpr size_t kBandBytes = 3u << 20; // feature rows of one band (three quart
 // 2.5 MB x 19: 4.35 / 2.52; 3 MB x 16: 4.32 / 2.48; 3 MB x 20: 4.33 / 2.49; 3 MB x 24: 4.32 / 2.53; 4 MB x 12: 4.45 / 2.46.
 // With 2 MB bands, 10 / 15 / 24 / 32 hot bands: 5.44 / 4.83 / 4.44 / 4.44 ms (K = 128).
 constexpr int kBandMaxCols = 8192;      // narrow feature rows: a band is at most this many columns
-constexpr int kRowsPerBlock = 4;
+constexpr int kRowsPerBlock = 4;        // wavefronts per work-group (2 / 4 / 8: 4.29 / 4.31 / 4.33 ms at K = 128, 2.50 / 2.45 / 2.56 at K = 41)
 constexpr int kDenseChunk = 2048;       // column granularity of the dense rectangles
 constexpr int kDenseMaxCols = 32768;    // widest rectangle
 constexpr int kDenseFirstRows = 4096;   // rows of the first group; every further group doubles the covered rows
