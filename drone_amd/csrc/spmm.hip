@@ -203,6 +203,75 @@ __global__ __launch_bounds__(kWave * kRowsPerBlock) void spmm_rows_kernel(
     }
 }
 
+// Narrow feature rows (K <= 32) leave a wavefront with 8 or 16 lane groups, and a short row cannot feed them: one
+// wavefront per row spends its time on the row's chain of round trips (bounds, pairs, feature rows, store).  Here a
+// wavefront takes R consecutive rows, W = 64 / R lanes each: every row has its own batch of W (col, val) pairs and
+// its own P = W / G lane groups; the loop runs as long as the longest of the R rows.
+template <int G, int VEC, int R>
+__global__ __launch_bounds__(kWave * kRowsPerBlock) void spmm_rows_multi_kernel(
+    int n_rows, const int *__restrict__ rp, const int *__restrict__ ci, const float *__restrict__ val,
+    const float *__restrict__ B, int ldb, float *__restrict__ C, int ldc, int K, float alpha, float beta)
+{
+    constexpr int W = kWave / R, P = W / G, U = G < 8 ? G : 8, S = P * U;
+    static_assert(P >= 1 && W % S == 0, "a step never straddles two batches");
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wl = lane % W, w0 = lane - wl, li = wl % G, sub = wl / G;
+    const int r = (blockIdx.x * kRowsPerBlock + threadIdx.x / kWave) * R + lane / W;
+    int e0 = 0, len = 0;
+    if (r < n_rows) {
+        e0 = rp[r];
+        len = rp[r + 1] - e0;
+        if (len > kSplitRow) len = 0;  // left to the piece kernels
+    }
+    int longest = len;
+#pragma unroll
+    for (int off = W; off < kWave; off <<= 1) {
+        const int other = __shfl_xor(longest, off, kWave);
+        longest = other > longest ? other : longest;
+    }
+    for (int k0 = 0; k0 < K; k0 += G * VEC) {
+        const int kbase = k0 + li * VEC;
+        const bool active = kbase < K;
+        float acc[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
+        for (int base = 0; base < longest; base += W) {
+            const bool mine = base + wl < len;
+            const int c = mine ? ci[e0 + base + wl] : 0;
+            const float a = mine ? val[e0 + base + wl] : 0.0f;
+            const int cnt = len - base;  // entries of this row left in the batch (may be <= 0 or > W)
+            for (int q = 0; q < W; q += S) {
+                int cc[U];
+                float aa[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    cc[u] = __shfl(c, w0 + q + u * P + sub, kWave);
+                    aa[u] = __shfl(a, w0 + q + u * P + sub, kWave);
+                }
+                if (active) {
+                    float b[U][VEC];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) b[u][v] = 0.0f;
+                        if (q + u * P + sub < cnt) load_vec<VEC>(B + (size_t)cc[u] * ldb + kbase, b[u]);
+                    }
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) acc[v] = fmaf(aa[u], b[u][v], acc[v]);
+                }
+            }
+        }
+#pragma unroll
+        for (int off = G; off < W; off <<= 1)
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) acc[v] += __shfl_xor(acc[v], off, kWave);
+        if (sub == 0 && active && r < n_rows && rp[r + 1] - rp[r] <= kSplitRow)
+            store_row<VEC>(C + (size_t)r * ldc, kbase, K, acc, alpha, beta);
+    }
+}
+
 // One wavefront per band piece of a long row (work list in band-major order): partial[slot, 0..K) = sum over
 // the piece.  ci / val are the plan's (band,row)-sorted copies.
 // Short pieces are dear: launched band by band on the 229 M-entry graph (K = 128), the bands whose pieces hold 100
@@ -453,10 +522,18 @@ void launch_spmm(const drone_spmm_plan *plan, const int *rp, const int *ci, cons
             plan->num_pieces, plan->piece_begin, plan->piece_end, plan->piece_slot, plan->ci2, plan->val2, B, ldb,
             plan->partial, plan->max_k, K);
     }
-    const int blocks = (int)ceil_div(plan->n_rows, kRowsPerBlock);
-    if (blocks > 0)
-        spmm_rows_kernel<G, VEC><<<blocks, kWave * kRowsPerBlock, 0, s>>>(plan->n_rows, rp, ci, v, B, ldb, C, ldc, K,
-                                                                         alpha, beta);
+    // rows per wavefront of the short-row kernel.  R-MAT scale 22, 90 M entries, K = 16 (lane groups of 4): 1 / 4 / 8
+    // rows 2.10 / 1.86 / 1.92 ms; two rows for lane groups of 16 lost: K = 64 4.03 against 3.65 ms, K = 41 2.57 against 2.45.
+    constexpr int R = G <= 4 ? 4 : G <= 8 ? 2 : 1;
+    const int blocks = (int)ceil_div(plan->n_rows, kRowsPerBlock * R);
+    if (blocks > 0) {
+        if constexpr (R > 1)
+            spmm_rows_multi_kernel<G, VEC, R><<<blocks, kWave * kRowsPerBlock, 0, s>>>(plan->n_rows, rp, ci, v, B, ldb, C,
+                                                                                      ldc, K, alpha, beta);
+        else
+            spmm_rows_kernel<G, VEC><<<blocks, kWave * kRowsPerBlock, 0, s>>>(plan->n_rows, rp, ci, v, B, ldb, C, ldc, K,
+                                                                             alpha, beta);
+    }
     if (plan->num_long > 0)  // also when every entry of the long rows went to the dense part: C = beta * C there
         spmm_combine_kernel<<<plan->num_long, 128, 0, s>>>(plan->num_long, plan->long_row, plan->first_slot,
                                                           plan->partial, plan->max_k, C, ldc, K, alpha, beta);
