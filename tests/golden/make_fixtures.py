@@ -51,6 +51,35 @@ def main():
         truth=[0, 2, -1, 1, 1, -1],
         keep1=(rng.random((n, hid)) >= 0.5).astype(int).tolist()))
 
+    # 7-vertex DIRECTED graph (in-degree != out-degree, one vertex without in-edges, one without out-edges):
+    # val(u->v) = 1/sqrt(out_deg[u] * in_deg[v]) (cuda_kernel.cu:145-155).  The dense matrix A[u, v] travels with the
+    # fixture so a test can form A^T (forward, cuda_module.cu:245) and A (backward, :335) without any CSR code.
+    rng = np.random.default_rng(4321)
+    n, fin, hid, cls = 7, 4, 5, 3
+    arcs = [(0, 1), (0, 2), (0, 3), (1, 2), (2, 0), (2, 3), (3, 4), (4, 1), (4, 5), (5, 5), (6, 0), (6, 2), (1, 5)]
+    D = np.zeros((n, n), bool)
+    for a, b in arcs:
+        D[a, b] = True
+    out_deg, in_deg = D.sum(1), D.sum(0)
+    assert (out_deg != in_deg).any() and in_deg[6] == 0 and out_deg[5] == 1
+    rp = np.concatenate([[0], np.cumsum(out_deg)]).astype(int)
+    ci = np.concatenate([np.nonzero(D[r])[0] for r in range(n)]).astype(int)
+    u = np.repeat(np.arange(n), out_deg)
+    val = (1.0 / np.sqrt((out_deg[u] * in_deg[ci]).astype(np.float32))).astype(np.float32)
+    dense = np.zeros((n, n), np.float32)
+    dense[u, ci] = val
+    rpT = np.concatenate([[0], np.cumsum(in_deg)]).astype(int)
+    ciT = np.concatenate([np.nonzero(D[:, c])[0] for c in range(n)]).astype(int)
+    valT = np.concatenate([dense[np.nonzero(D[:, c])[0], c] for c in range(n)])
+    dump("gcn_tiny_directed_step.json", dict(
+        rp=rp.tolist(), ci=ci.tolist(), val=val.tolist(), rpT=rpT.tolist(), ciT=ciT.tolist(), valT=valT.tolist(),
+        in_deg=in_deg.tolist(), out_deg=out_deg.tolist(), A_dense=dense.tolist(),
+        X=rng.normal(size=(n, fin)).astype(np.float32).tolist(),
+        W1=rng.uniform(-0.8, 0.8, (fin, hid)).astype(np.float32).tolist(),
+        W2=rng.uniform(-0.8, 0.8, (hid, cls)).astype(np.float32).tolist(),
+        truth=[0, 2, -1, 1, 1, 2, 0],
+        keep1=(rng.random((n, hid)) >= 0.5).astype(int).tolist()))
+
 
 if __name__ == "__main__":
     main()

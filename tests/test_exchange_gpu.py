@@ -98,15 +98,32 @@ def test_pr_group_equals_whole_graph(oracle):
         lb.close()
 
 
-def test_exchange_without_transport_is_refused(oracle):
-    """workerNum > 1 with an empty Comm::comm must not silently skip the exchange."""
-    import ctypes as C
-    from drone_amd import _lib
+def test_single_worker_needs_no_transport(oracle):
+    """One subgraph: no staging is allocated and the empty Comm::comm is never looked at."""
     from drone_amd.pagerank import PRWorkerCUDA
     u, v = _graph(6, 4, 1)
     w = PRWorkerCUDA(64, u, v, workerId=0, workerNum=1)
     try:
         w.peval()
-        assert w.values.sendID is None  # one subgraph: no staging, as before
+        assert w.values.sendID is None
+    finally:
+        w.close()
+
+
+def test_exchange_without_transport_is_refused(oracle):
+    """workerNum > 1 with an empty Comm::comm must not silently skip the exchange.  The reference-compatible entry
+    points can only print and exit, so the refusal is observed through an entry point with a status: the row
+    synchronisation of a worker that was told it has a peer but was given no transport."""
+    import torch
+    from drone_amd import gcn
+    from drone_amd._lib import DroneError
+    from drone_amd.pagerank import PRWorkerCUDA
+    u, v = _graph(6, 4, 1)
+    w = PRWorkerCUDA(64, u, v, workerId=0, workerNum=2)      # no routes, no loopback attached: Comm::comm stays null
+    try:
+        rows = torch.ones((w.n, 8), device="cuda")
+        with pytest.raises(DroneError, match="transport"):
+            gcn.graphsum_sync_rows(w.g, rows, 0, 2, w.comm)
+        assert torch.equal(rows, torch.ones_like(rows))
     finally:
         w.close()

@@ -355,12 +355,14 @@ def test_spmm_dense_core_matches_oracle(T, oracle):
     plan.close()
 
 
-def _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, row_sums):
+def _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, row_sums, dense=None):
     """Size-independent checks of C = A * B at a benchmark shape: A * 1 against fp64 row sums, adjointness
     <A X, Y> = <X, A^T Y> with the separately built transpose, agreement with the vendor's sparse product on a
     column sample, and a repeatable result."""
     plan = gcn.SpmmPlan(rp, ci, val, N, max_k=K)
     planT = gcn.SpmmPlan(rpT, ciT, vT, N, max_k=K)
+    if dense is not None:                      # whether the plans moved part of the matrix to dense rectangles
+        assert (plan.info()["dense_nnz"] > 0) == dense and (planT.info()["dense_nnz"] > 0) == dense
     ones = torch.ones((N, 4), device="cuda")
     got = gcn.spmm(plan, rp, ci, val, ones)
     assert float(((got[:, 0].double() - row_sums).abs() / row_sums.abs().clamp(min=1e-30)).max()) <= 1e-4
@@ -380,6 +382,16 @@ def _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, row_
     ref = torch.sparse.mm(A64, X[:, cols].double().contiguous())
     err = (AX[:, cols].double() - ref).abs().max(dim=0).values / ref.abs().max(dim=0).values
     assert float(err.max()) <= 1e-4
+    mag = torch.sparse.mm(torch.sparse_csr_tensor(rp.long(), ci.long(), val.double().abs(), size=(N, N)),
+                          X[:, cols].double().abs().contiguous())        # every element against its own sum of |a||b|
+    assert float(((AX[:, cols].double() - ref).abs() / mag.clamp(min=1e-30)).max()) <= 1e-4
+    del A64, mag
+    # the transposed product element-wise as well
+    AT64 = torch.sparse_csr_tensor(rpT.long(), ciT.long(), vT.double(), size=(N, N))
+    refT = torch.sparse.mm(AT64, Y[:, cols].double().contiguous())
+    magT = torch.sparse.mm(torch.sparse_csr_tensor(rpT.long(), ciT.long(), vT.double().abs(), size=(N, N)),
+                           Y[:, cols].double().abs().contiguous())
+    assert float(((ATY[:, cols].double() - refT).abs() / magT.clamp(min=1e-30)).max()) <= 1e-4
     plan.close()
     planT.close()
 
@@ -398,10 +410,11 @@ def test_full_size_properties_config3(T):
     _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, 128, cs[rp[1:].long()] - cs[rp[:-1].long()])
 
 
-@pytest.mark.parametrize("K", [16, 64])
+@pytest.mark.parametrize("K", [16, 64, 256])
 def test_full_size_properties_config5(T, K):
     """Fifth configuration at full size: skewed directed R-MAT scale 22 ef 32, row-normalised; forward and transposed
-    products (K = 256 has the same code path as the 128-wide tiles of the other configurations)."""
+    products at every width the configuration names.  K = 256 is the only width at which the plans of this graph hold
+    a dense part."""
     torch = T
     from drone_amd import gcn, rmat
     x = rmat.pagerank_inputs_torch(22, 32, 5, a=0.70, b=0.12, c=0.12)
@@ -413,4 +426,4 @@ def test_full_size_properties_config5(T, K):
     val = (1.0 / torch.repeat_interleave(cnt.clamp(min=1).float(), cnt)).contiguous()
     rpT, ciT, vT = gcn.csr_transpose(N, N, rp, ci, val)
     assert int(rpT[-1]) == x["nnz"] and int((ciT[1:] < ciT[:-1]).sum()) <= N          # rows ascending inside
-    _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, (cnt > 0).double())
+    _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, (cnt > 0).double(), dense=(K == 256))

@@ -1,7 +1,9 @@
 """GPU parity of the 2-layer GCN training step (module layer + C handle API) against the CPU oracle.
-Tolerance: outputs and gradients within 1e-4 of the oracle relative to the tensor's largest magnitude
-(fp32, summation order differs between the wavefront kernels and the oracle's serial loops); arg-max predictions
-identical; masks, counts and the CSR transpose exact."""
+Tolerance: every element of the outputs and gradients within 1e-4 of the oracle, relative to that element's own
+scale - the same computation carried out on absolute values, i.e. the sum of |a||b| over everything that was added
+into it (fp32, summation order differs between the wavefront kernels and the oracle's serial loops) - and, as a
+second bound, within 1e-4 of the tensor's largest magnitude; arg-max predictions identical; masks, counts and the
+CSR transpose exact."""
 import json
 import os
 
@@ -24,16 +26,44 @@ def dev(T, a, dtype=None):
     return T.from_numpy(a).cuda()
 
 
-def close(got, ref, tol=1e-4):
-    scale = max(np.abs(ref).max(), 1e-30)
-    err = np.abs(got.astype(np.float64) - ref.astype(np.float64)).max() / scale
-    assert err <= tol, f"max error {err:.3e} of scale {scale:.3e}"
+def close(got, ref, tol=1e-4, scale=None):
+    """|got - ref| <= tol * max|ref| and, with `scale` (per element, see step_scales), <= tol * scale element-wise."""
+    diff = np.abs(got.astype(np.float64) - ref.astype(np.float64))
+    top = max(np.abs(ref).max(), 1e-30)
+    assert diff.max() <= tol * top, f"max error {diff.max() / top:.3e} of scale {top:.3e}"
+    if scale is not None:
+        rel = diff / np.maximum(scale, 1e-30)
+        assert rel.max() <= tol, f"element {np.unravel_index(rel.argmax(), rel.shape)}: error {rel.max():.3e} of its scale"
+
+
+def step_scales(n, rp, ci, val, rpT, ciT, valT, X, W1, W2, truth, ref, keep=None, p=0.5, grad_scale=1.0):
+    """Per-element magnitude scales of the step's tensors: the step recomputed in fp64 on absolute values (no ReLU
+    mask), which bounds the sum of |a||b| behind every element; the softmax gradient's scale follows its derivative,
+    |dp_j| <= p_j (|dz_j| + sum_k p_k |dz_k|).  Error / scale is what a different summation order can change."""
+    import scipy.sparse as sp
+    from scipy.special import softmax
+    aA = sp.csr_matrix((np.abs(val).astype(np.float64), ci, rp), shape=(n, n))
+    aAT = sp.csr_matrix((np.abs(valT).astype(np.float64), ciT, rpT), shape=(n, n))
+    aX, aW1, aW2 = (np.abs(np.asarray(a, np.float64)) for a in (X, W1, W2))
+    ks = 1.0 if keep is None else keep.astype(np.float64) / (1.0 - p)
+    sH1 = (aAT @ (aX @ aW1)) * ks
+    sZ = aAT @ (sH1 @ aW2)
+    prob = softmax(ref["Z"].astype(np.float64), axis=1)
+    lab = truth >= 0
+    dZ = prob.copy()
+    dZ[np.arange(n)[lab], truth[lab]] -= 1.0
+    sdZ = (np.abs(dZ) + prob * (sZ + (prob * sZ).sum(1, keepdims=True))) * lab[:, None] * grad_scale
+    sdT2 = aA @ sdZ
+    sdH1 = (sdT2 @ aW2.T) * ks
+    sdT1 = aA @ sdH1
+    return dict(Z=sZ, H1=sH1, dW2=sH1.T @ sdT2, dT1=sdT1, dW1=aX.T @ sdT1)
 
 
 def make_model(T, g, X, W1, W2, label, split, **kw):
     from drone_amd.gcn import GcnModel
-    deg = dev(T, g["deg"], np.int32)
-    return GcnModel(dev(T, g["rp"], np.int32), dev(T, g["ci"], np.int32), deg, deg, dev(T, X, np.float32),
+    ind = dev(T, g.get("in_deg", g.get("deg")), np.int32)
+    outd = dev(T, g.get("out_deg", g.get("deg")), np.int32)
+    return GcnModel(dev(T, g["rp"], np.int32), dev(T, g["ci"], np.int32), ind, outd, dev(T, X, np.float32),
                     dev(T, label, np.int32), dev(T, split, np.int32), dev(T, W1, np.float32), dev(T, W2, np.float32), **kw)
 
 
@@ -42,25 +72,35 @@ def oracle_step(oracle, g, X, W1, W2, truth, keep=None, p=0.5):
     return oracle.gcn_forward_backward(g["rp"], g["ci"], g["val"], rpT, ciT, vT, X, W1, W2, truth, keep, p)
 
 
+@pytest.mark.parametrize("fixture", ["gcn_tiny_step.json", "gcn_tiny_directed_step.json"])
 @pytest.mark.parametrize("use_dropout", [False, True])
-def test_tiny_fixture_step(T, oracle, use_dropout):
-    d = {k: np.array(v) for k, v in json.load(open(os.path.join(GOLD, "gcn_tiny_step.json"))).items()}
-    n = 6
-    deg = np.diff(d["rp"]).astype(np.int32)
-    g = dict(n=n, rp=d["rp"], ci=d["ci"], val=d["val"].astype(np.float32), deg=deg)
+def test_tiny_fixture_step(T, oracle, use_dropout, fixture):
+    """The directed fixture (in-degree != out-degree, transpose != itself) pins which orientation the forward
+    (in-edges, cuda_module.cu:245) and the backward (out-edges, :335) aggregate over, and which degree normalises
+    which end of an edge."""
+    d = {k: np.array(v) for k, v in json.load(open(os.path.join(GOLD, fixture))).items()}
+    n = len(d["rp"]) - 1
+    ind = d["in_deg"].astype(np.int32) if "in_deg" in d else np.diff(d["rp"]).astype(np.int32)
+    outd = d["out_deg"].astype(np.int32) if "out_deg" in d else ind
+    g = dict(n=n, rp=d["rp"], ci=d["ci"], val=d["val"].astype(np.float32), in_deg=ind, out_deg=outd)
     truth = d["truth"].astype(np.int32)
     split = np.where(truth >= 0, 1, 2).astype(np.int32)
     label = np.maximum(truth, 0)
     m = make_model(T, g, d["X"], d["W1"], d["W2"], label, split, use_dropout=use_dropout, use_adam=False, lr=0.01, seed=5)
-    np.testing.assert_array_equal(m.tensor("val"), oracle.edge_values(g["rp"], g["ci"], deg, deg))
+    np.testing.assert_array_equal(m.tensor("val"), oracle.edge_values(g["rp"], g["ci"], ind, outd))
+    np.testing.assert_array_equal(m.tensor("val"), g["val"])
+    np.testing.assert_array_equal(m.tensor("rpT"), d["rpT"])
+    np.testing.assert_array_equal(m.tensor("ciT"), d["ciT"])
+    np.testing.assert_array_equal(m.tensor("valT"), d["valT"].astype(np.float32))
     m.set_truth(1)
     np.testing.assert_array_equal(m.tensor("truth"), truth)
     m.forward(True)
     m.backward()
     keep = m.tensor("keep1") if use_dropout else None
     ref = oracle_step(oracle, g, d["X"], d["W1"], d["W2"], truth, keep, 0.5)
-    for name, key in (("Z", "Z"), ("H1", "H1"), ("dW1", "dW1"), ("dW2", "dW2"), ("dT1", "dT1")):
-        close(m.tensor(name), ref[key])
+    sc = step_scales(n, d["rp"], d["ci"], g["val"], d["rpT"], d["ciT"], d["valT"], d["X"], d["W1"], d["W2"], truth, ref, keep)
+    for name in ("Z", "H1", "dW1", "dW2", "dT1"):
+        close(m.tensor(name), ref[name], scale=sc[name])
     loss, acc = m.read_metrics()
     assert loss == pytest.approx(ref["loss"], rel=1e-5)
     m.optimizer_step()
@@ -70,11 +110,31 @@ def test_tiny_fixture_step(T, oracle, use_dropout):
     m.close()
 
 
-@pytest.mark.parametrize("scale,ef,fin,hid,cls,use_dropout", [(10, 8, 50, 16, 7, False), (11, 16, 602, 128, 41, True)])
-def test_rmat_step_against_oracle(T, oracle, scale, ef, fin, hid, cls, use_dropout):
-    """Second case keeps the fourth configuration's widths (602 -> 128 -> 41, dropout 0.5, SGD 0.01, 66 % train)."""
+def directed_graph_np(scale, ef, seed):
+    """Directed R-MAT graph as an out-edge CSR with its own in- and out-degrees (they differ on most vertices) and
+    the reference's edge values."""
+    from drone_amd import rmat
+    n = 1 << scale
+    s, d = rmat.rmat_edges(scale, n * ef, seed=seed)
+    src, dst = rmat.clean_directed_np(s, d)              # sorted by (dst, src)
+    order = np.lexsort((dst, src))
+    src, dst = src[order], dst[order]
+    out_deg = np.bincount(src, minlength=n).astype(np.int32)
+    in_deg = np.bincount(dst, minlength=n).astype(np.int32)
+    rp = np.zeros(n + 1, np.int32)
+    rp[1:] = np.cumsum(out_deg)
+    val = (1.0 / np.sqrt((1.0 * out_deg[src] * in_deg[dst]).astype(np.float32))).astype(np.float32)
+    return dict(n=n, rp=rp, ci=dst.astype(np.int32), val=val, in_deg=in_deg, out_deg=out_deg)
+
+
+@pytest.mark.parametrize("scale,ef,fin,hid,cls,use_dropout,directed",
+                         [(10, 8, 50, 16, 7, False, False), (11, 16, 602, 128, 41, True, False),
+                          (11, 12, 70, 32, 9, True, True)])
+def test_rmat_step_against_oracle(T, oracle, scale, ef, fin, hid, cls, use_dropout, directed):
+    """Second case keeps the fourth configuration's widths (602 -> 128 -> 41, dropout 0.5, SGD 0.01, 66 % train); the
+    third runs on a directed graph (transpose != itself, in-degree != out-degree)."""
     from drone_amd import graphs, rmat
-    g = graphs.gcn_graph_np(scale, ef, seed=4)
+    g = directed_graph_np(scale, ef, seed=4) if directed else graphs.gcn_graph_np(scale, ef, seed=4)
     n = g["n"]
     X = rmat.normal_f32((n, fin), seed=4)
     lim1, lim2 = np.sqrt(6.0 / (fin + hid)), np.sqrt(6.0 / (hid + cls))
@@ -87,6 +147,7 @@ def test_rmat_step_against_oracle(T, oracle, scale, ef, fin, hid, cls, use_dropo
     # set-up products: edge values and the transposed CSR are exact
     np.testing.assert_array_equal(m.tensor("val"), g["val"])
     rpT, ciT, vT = oracle.csr_transpose(n, n, g["rp"], g["ci"], g["val"])
+    assert directed == (not np.array_equal(rpT, g["rp"]))
     np.testing.assert_array_equal(m.tensor("rpT"), rpT)
     np.testing.assert_array_equal(m.tensor("ciT"), ciT)
     np.testing.assert_array_equal(m.tensor("valT"), vT)
@@ -97,11 +158,9 @@ def test_rmat_step_against_oracle(T, oracle, scale, ef, fin, hid, cls, use_dropo
     if use_dropout:
         assert abs(keep.mean() - 0.5) < 0.02
     ref = oracle.gcn_forward_backward(g["rp"], g["ci"], g["val"], rpT, ciT, vT, X, W1, W2, truth, keep, 0.5)
-    close(m.tensor("Z"), ref["Z"])
-    close(m.tensor("H1"), ref["H1"])
-    close(m.tensor("dW1"), ref["dW1"])
-    close(m.tensor("dW2"), ref["dW2"])
-    close(m.tensor("dT1"), ref["dT1"])
+    sc = step_scales(n, g["rp"], g["ci"], g["val"], rpT, ciT, vT, X, W1, W2, truth, ref, keep)
+    for name in ("Z", "H1", "dW1", "dW2", "dT1"):
+        close(m.tensor(name), ref[name], scale=sc[name])
     assert loss == pytest.approx(ref["loss"], rel=1e-4)
     assert acc == pytest.approx(oracle.accuracy(ref["Z"], truth), abs=2.0 / n)
     # identical arg-max predictions
@@ -162,6 +221,7 @@ def test_training_reduces_loss_with_adam_and_eval_is_pure(T, oracle):
 def test_full_size_properties_config4(T):
     """Fourth configuration at full size (232,965 vertices, ~229 M entries, 602 -> 128 -> 41): properties that
     need no CPU oracle - A_hat * 1 against fp64 row sums, forward/backward adjointness <A^T X, Y> = <X, A Y>,
+    every element of four columns of the K = 41 and K = 128 products against the vendor's fp64 sparse product,
     the big GEMMs against torch.matmul in fp32/fp64, and a bitwise repeatable, finite training step."""
     torch = T
     from drone_amd import gcn, graphs, rmat
@@ -173,6 +233,8 @@ def test_full_size_properties_config4(T):
     rpT, ciT, vT = gcn.csr_transpose(N, N, rp, ci, val)
     assert torch.equal(rpT, rp) and torch.equal(ciT, ci) and torch.equal(vT, val)      # symmetric graph
     plan = gcn.SpmmPlan(rp, ci, val, N, max_k=HID)
+    assert plan.info()["dense_nnz"] > 50_000_000           # the products below go through the dense core
+    A64 = torch.sparse_csr_tensor(rp.long(), ci.long(), val.double(), size=(N, N))
     # A * ones == row sums (fp64 prefix sums as the reference value)
     ones = torch.ones((N, 4), device="cuda")
     got = gcn.spmm(plan, rp, ci, val, ones)
@@ -195,6 +257,13 @@ def test_full_size_properties_config4(T):
         again = torch.empty((N, ld), device="cuda")[:, :K]       # same leading dimension -> same lane layout
         gcn.spmm(plan, rp, ci, val, X, K=K, out=again)
         assert torch.equal(again, AX)                          # fixed summation order
+        # element-wise: the vendor's sparse product in fp64 on four columns, every element against its own sum of
+        # |a||b| (the values are positive, so that is A * |X|)
+        cols = [0, 1, K // 2, K - 1]
+        ref = torch.sparse.mm(A64, X[:, cols].double().contiguous())
+        mag = torch.sparse.mm(A64, X[:, cols].double().abs().contiguous())
+        assert float(((AX[:, cols].double() - ref).abs() / mag.clamp(min=1e-30)).max()) <= 1e-4
+    del A64
     plan.close()
     # the step's GEMM shapes against torch (fp64 reference on a row sample, fp32 on the whole)
     Xf = torch.from_numpy(rmat.normal_f32((N, FIN), seed=4)).cuda()

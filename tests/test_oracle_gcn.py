@@ -192,15 +192,14 @@ def test_adam_and_sgd_textbook(oracle):
         np.testing.assert_allclose(w, W, rtol=2e-5, atol=1e-6)
 
 
-def _tiny_gcn_inputs():
-    k = load("gcn_tiny_step.json")
+def _tiny_gcn_inputs(name="gcn_tiny_step.json"):
+    k = load(name)
     return {a: np.array(b) for a, b in k.items()}
 
 
-def _np_loss(rpT, ciT, vT, X, W1, W2, truth, keep, p):
-    """Own fp64 forward of the 2-layer net; returns the SUM loss over labelled rows."""
-    n = X.shape[0]
-    At = sp.csr_matrix((vT.astype(np.float64), ciT, rpT), shape=(n, n))
+def _np_loss(At, X, W1, W2, truth, keep, p):
+    """Own fp64 forward of the 2-layer net, At = the matrix the forward aggregation multiplies by (A transposed:
+    out[v] = sum over edges u->v); returns the SUM loss over labelled rows."""
     H = At @ (X @ W1)
     H = np.maximum(H, 0)
     if keep is not None:
@@ -211,16 +210,40 @@ def _np_loss(rpT, ciT, vT, X, W1, W2, truth, keep, p):
     return -ls[lab, truth[lab]].sum(), Z
 
 
+def test_directed_fixture_edge_values_and_transpose(oracle):
+    """The directed fixture's arrays were written from a dense matrix; the oracle's edge values (out-degree of the
+    source, in-degree of the target: swapping the two changes them on this graph) and its transpose must agree."""
+    d = _tiny_gcn_inputs("gcn_tiny_directed_step.json")
+    n = len(d["rp"]) - 1
+    val = oracle.edge_values(d["rp"], d["ci"], d["in_deg"], d["out_deg"])
+    np.testing.assert_array_equal(val, d["val"].astype(np.float32))
+    assert not np.array_equal(oracle.edge_values(d["rp"], d["ci"], d["out_deg"], d["in_deg"]), val)
+    rpT, ciT, vT = oracle.csr_transpose(n, n, d["rp"], d["ci"], d["val"].astype(np.float32))
+    assert rpT.tolist() == d["rpT"].tolist() and ciT.tolist() == d["ciT"].tolist()
+    np.testing.assert_array_equal(vT, d["valT"].astype(np.float32))
+    dense = sp.csr_matrix((d["val"], d["ci"], d["rp"]), shape=(n, n)).toarray()
+    np.testing.assert_array_equal(dense.astype(np.float32), d["A_dense"].astype(np.float32))
+    assert not np.array_equal(dense, dense.T)
+
+
+@pytest.mark.parametrize("fixture", ["gcn_tiny_step.json", "gcn_tiny_directed_step.json"])
 @pytest.mark.parametrize("use_dropout", [False, True])
-def test_gcn_step_finite_difference(oracle, use_dropout):
-    d = _tiny_gcn_inputs()
+def test_gcn_step_finite_difference(oracle, use_dropout, fixture):
+    """Forward = multiplication by A^T (cuda_module.cu:245 uses matAT), backward = by A (:335): on the directed
+    fixture the forward is formed from the dense matrix's transpose, so an oracle that aggregated over out-edges
+    fails the Z comparison, and one whose backward is not the adjoint of its forward fails the gradient check."""
+    d = _tiny_gcn_inputs(fixture)
+    n = len(d["rp"]) - 1
     keep = d["keep1"].astype(np.uint8) if use_dropout else None
     res = oracle.gcn_forward_backward(d["rp"], d["ci"], d["val"], d["rpT"], d["ciT"], d["valT"], d["X"],
                                       d["W1"], d["W2"], d["truth"], keep, 0.5)
     X, W1, W2 = d["X"].astype(np.float64), d["W1"].astype(np.float64), d["W2"].astype(np.float64)
     truth = d["truth"].astype(np.int64)
-    args = (d["rpT"], d["ciT"], d["valT"].astype(np.float32))
-    loss_sum, Z = _np_loss(*args, X, W1, W2, truth, keep, 0.5)
+    if "A_dense" in d:
+        At = d["A_dense"].astype(np.float32).astype(np.float64).T
+    else:
+        At = sp.csr_matrix((d["valT"].astype(np.float32).astype(np.float64), d["ciT"], d["rpT"]), shape=(n, n)).toarray()
+    loss_sum, Z = _np_loss(At, X, W1, W2, truth, keep, 0.5)
     np.testing.assert_allclose(res["Z"], Z, rtol=1e-4, atol=1e-6)
     np.testing.assert_allclose(res["loss"], loss_sum / (truth >= 0).sum(), rtol=1e-5)
     h = 1e-6
@@ -232,5 +255,5 @@ def test_gcn_step_finite_difference(oracle, use_dropout):
             Wm[idx] -= h
             a = (Wp, W2) if name == "W1" else (W1, Wp)
             b = (Wm, W2) if name == "W1" else (W1, Wm)
-            fd[idx] = (_np_loss(*args, X, *a, truth, keep, 0.5)[0] - _np_loss(*args, X, *b, truth, keep, 0.5)[0]) / (2 * h)
+            fd[idx] = (_np_loss(At, X, *a, truth, keep, 0.5)[0] - _np_loss(At, X, *b, truth, keep, 0.5)[0]) / (2 * h)
         np.testing.assert_allclose(got, fd, rtol=2e-3, atol=2e-4)
