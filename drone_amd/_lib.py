@@ -110,6 +110,8 @@ SIGNATURES = {
     "drone_spmm_bytes": (_I64, [_I, _I64, _I]),
     "drone_sgemm_rm_f32": (_I, [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P]),
     "drone_sgemm_flops": (_I64, [_I, _I, _I]),
+    "drone_sgemm_rm_f32_noalloc": (_I, [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P]),
+    "drone_sgemm_noalloc_scratch_bytes": (_I64, []),
     "drone_relu_forward_f32": (_I, [_P, _P, _I64, _I, _P]),
     "drone_relu_backward_f32": (_I, [_P, _P, _I64, _P]),
     "drone_dropout_mask": (_I, [_P, _I64, _U64, _U64, _F, _P]),

@@ -276,8 +276,36 @@ void launch(bool ta, bool tb, dim3 grid, hipStream_t s, int M, int N, int K, flo
 
 using namespace drone;
 
-extern "C" int drone_sgemm_rm_f32(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,
-                                  const float *B, int ldb, float beta, float *C, int ldc, drone_stream_t stream)
+// Split-K partials of the entry point that may not allocate: one fixed array per GPU, held by the library's code
+// object until the process ends.  In host code this name is only a handle for hipGetSymbolAddress; the address a
+// kernel can use is looked up once per device (static_scratch) and passed on as an ordinary pointer.
+constexpr size_t kStaticScratchFloats = (size_t)8 << 20;  // 32 MiB
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_static_mutex;
+float *g_static_scratch[kMaxDevices] = {};
+
+// Device address of this GPU's copy of `scratch` (every device holds its own copy at its own address).
+int static_scratch(float **out)
+{
+    int dev = 0;
+    DRONE_HIP_TRY(hipGetDevice(&dev));
+    DRONE_REQUIRE(dev >= 0 && dev < kMaxDevices, "device ordinal out of range");
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (!g_static_scratch[dev]) {
+        void *p = nullptr;
+        DRONE_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        DRONE_REQUIRE(p != nullptr, "no device address for the static scratch array");
+        g_static_scratch[dev] = static_cast<float *>(p);
+    }
+    *out = g_static_scratch[dev];
+    return DRONE_OK;
+}
+
+int sgemm_entry(bool may_allocate, int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,
+                const float *B, int ldb, float beta, float *C, int ldc, drone_stream_t stream)
 {
     clear_error();
     DRONE_REQUIRE(M >= 0 && N >= 0 && K >= 0, "negative dimension");
@@ -306,8 +334,22 @@ extern "C" int drone_sgemm_rm_f32(int transA, int transB, int M, int N, int K, f
     splits = (int)ceil_div(K > 0 ? K : 1, k_chunk);
     float *partial = nullptr;
     if (splits > 1) {
-        int rc = workspace(sizeof(float) * (size_t)splits * M * N, s, &partial);
-        if (rc != DRONE_OK) return rc;
+        // every (tile, split) work-group stores its whole tile, so the partials need no clearing
+        const size_t floats = (size_t)splits * M * N;
+        if (may_allocate) {
+            int rc = workspace(sizeof(float) * floats, s, &partial);
+            if (rc != DRONE_OK) return rc;
+        } else {
+            if (floats > kStaticScratchFloats) {
+                set_error(DRONE_ERR_INVALID,
+                          "drone_sgemm_rm_f32_noalloc: %d x %d x %d splits the reduction %d ways and needs %zu bytes of "
+                          "partial sums, the fixed scratch holds %zu; use drone_sgemm_rm_f32",
+                          M, N, K, splits, floats * sizeof(float), kStaticScratchFloats * sizeof(float));
+                return DRONE_ERR_INVALID;
+            }
+            int rc = static_scratch(&partial);
+            if (rc != DRONE_OK) return rc;
+        }
     }
     dim3 grid((unsigned)ceil_div(N, bn), (unsigned)ceil_div(M, BM), (unsigned)splits);
     DRONE_REQUIRE(grid.y <= 65535u * 32u, "M too large for the launch grid");
@@ -321,5 +363,21 @@ extern "C" int drone_sgemm_rm_f32(int transA, int transB, int M, int N, int K, f
     DRONE_HIP_TRY(hipGetLastError());
     return DRONE_OK;
 }
+}  // namespace
+
+extern "C" int drone_sgemm_rm_f32(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,
+                                  const float *B, int ldb, float beta, float *C, int ldc, drone_stream_t stream)
+{
+    return sgemm_entry(true, transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream);
+}
+
+extern "C" int drone_sgemm_rm_f32_noalloc(int transA, int transB, int M, int N, int K, float alpha, const float *A,
+                                          int lda, const float *B, int ldb, float beta, float *C, int ldc,
+                                          drone_stream_t stream)
+{
+    return sgemm_entry(false, transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream);
+}
+
+extern "C" int64_t drone_sgemm_noalloc_scratch_bytes(void) { return (int64_t)(kStaticScratchFloats * sizeof(float)); }
 
 extern "C" int64_t drone_sgemm_flops(int M, int N, int K) { return 2ll * M * N * K; }

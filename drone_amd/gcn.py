@@ -76,8 +76,9 @@ def spmm(plan, rp, ci, val, B, K=None, out=None, alpha=1.0, beta=0.0, stream=0):
     return out
 
 
-def sgemm(transA, transB, A, B, out=None, alpha=1.0, beta=0.0, M=None, N=None, K=None, stream=0):
-    """Row-major out(MxN) = alpha * op(A) @ op(B) + beta * out, dimensions default to the tensors' shapes."""
+def sgemm(transA, transB, A, B, out=None, alpha=1.0, beta=0.0, M=None, N=None, K=None, stream=0, noalloc=False):
+    """Row-major out(MxN) = alpha * op(A) @ op(B) + beta * out, dimensions default to the tensors' shapes.
+    noalloc: through drone_sgemm_rm_f32_noalloc (`out` must be given: the wrapper may not allocate either)."""
     import torch
     M = (A.shape[1] if transA else A.shape[0]) if M is None else M
     K = (A.shape[0] if transA else A.shape[1]) if K is None else K
@@ -85,8 +86,9 @@ def sgemm(transA, transB, A, B, out=None, alpha=1.0, beta=0.0, M=None, N=None, K
     if out is None:
         out = torch.empty((M, N), dtype=torch.float32, device=A.device)
     assert A.stride(1) == 1 and B.stride(1) == 1 and out.stride(1) == 1
-    check(lib().drone_sgemm_rm_f32(int(transA), int(transB), M, N, K, alpha, _ptr(A), A.stride(0), _ptr(B),
-                                   B.stride(0), beta, _ptr(out), out.stride(0), stream))
+    fn = lib().drone_sgemm_rm_f32_noalloc if noalloc else lib().drone_sgemm_rm_f32
+    check(fn(int(transA), int(transB), M, N, K, alpha, _ptr(A), A.stride(0), _ptr(B), B.stride(0), beta, _ptr(out),
+             out.stride(0), stream))
     return out
 
 

@@ -217,6 +217,17 @@ int64_t drone_spmm_bytes(int n_rows, int64_t nnz, int K);
 int drone_sgemm_rm_f32(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,
                        const float *B, int ldb, float beta, float *C, int ldc, drone_stream_t stream);
 int64_t drone_sgemm_flops(int M, int N, int K);
+/* No counterpart in the reference.  For callers that cannot allocate device memory at the time of the call (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the same product as
+ * drone_sgemm_rm_f32, bit for bit, with the partial sums of a split reduction kept in a fixed 32 MiB array that the
+ * library's code object holds on every GPU it runs on until the process ends, instead of the grow-only scratch.
+ * Calls no hipMalloc / hipFree.  The array is sized for the worst case of the split rule (at most 512 work-groups
+ * of 128 x 128 outputs); a product whose partial sums (splits * M * N floats) would exceed
+ * drone_sgemm_noalloc_scratch_bytes() is refused with DRONE_ERR_INVALID and leaves C untouched.  All calls on one GPU share the array: calls that overlap on one GPU (different streams or
+ * threads) race; order them on one stream or with events. */
+int drone_sgemm_rm_f32_noalloc(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,
+                               const float *B, int ldb, float beta, float *C, int ldc, drone_stream_t stream);
+int64_t drone_sgemm_noalloc_scratch_bytes(void);
 /* cuda_module.cu:50-62 clear_mirror_grad, launched between the two GEMMs of CUDAMatmul::backward (:89-90): rows
  * of grad [rows][ld] (K used columns) whose vertex is a mirror (mirror2worker[row] != -1) are set to zero, so a
  * replicated vertex contributes to the weight gradient on its master's worker only. */
