@@ -70,7 +70,8 @@ class SSSPValues(C.Structure):
 class GcnConfig(C.Structure):
     _fields_ = [("n", C.c_int), ("input_dim", C.c_int), ("hidden_dim", C.c_int), ("output_dim", C.c_int),
                 ("dropout", C.c_float), ("learning_rate", C.c_float), ("weight_decay", C.c_float),
-                ("use_dropout", C.c_int), ("use_adam", C.c_int), ("mean_gradient", C.c_int), ("seed", C.c_uint64)]
+                ("use_dropout", C.c_int), ("use_adam", C.c_int), ("mean_gradient", C.c_int), ("seed", C.c_uint64),
+                ("fold_input_aggregation", C.c_int)]
 
 
 _lib = None
@@ -117,11 +118,14 @@ SIGNATURES = {
     "drone_dropout_mask": (_I, [_P, _I64, _U64, _U64, _F, _P]),
     "drone_dropout_apply_f32": (_I, [_P, _P, _I64, _F, _P]),
     "drone_cross_entropy_f32": (_I, [_I, _I, _P, _I, _P, _P, _I, _F, _P, _P, _P]),
-    "drone_accuracy_f32": (_I, [_I, _I, _P, _I, _P, _P, _P, _P]),
+    "drone_accuracy_f32": (_I, [_I, _I, _P, _I, _P, _P, _P, _P, _P]),
+    "drone_sum_squares_f32": (_I, [_P, _I64, _P, _P]),
     "drone_sgd_step_f32": (_I, [_P, _P, _I64, _F, _P]),
     "drone_adam_step_f32": (_I, [_P, _P, _P, _P, _I64, _I, _F, _F, _F, _F, _F, _I, _P]),
     "drone_fill_f32": (_I, [_P, _I64, _F, _P]),
     "drone_gcn_create": (_I, [C.POINTER(_P), C.POINTER(GcnConfig), _I64, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P]),
+    "drone_gcn_create_worker": (_I, [C.POINTER(_P), C.POINTER(GcnConfig), C.POINTER(Graph), C.POINTER(Comm), _I, _I, _I, _I,
+                                     _P, _P, _P, _I, _P, _P, _P, _P]),
     "drone_gcn_destroy": (_I, [_P]),
     "drone_gcn_set_truth": (_I, [_P, _I]),
     "drone_gcn_forward": (_I, [_P, _I]),
@@ -129,6 +133,8 @@ SIGNATURES = {
     "drone_gcn_optimizer_step": (_I, [_P]),
     "drone_gcn_train_step_async": (_I, [_P]),
     "drone_gcn_read_metrics": (_I, [_P, C.POINTER(_F), C.POINTER(_F)]),
+    "drone_gcn_read_losses": (_I, [_P, C.POINTER(_F), C.POINTER(_F)]),
+    "drone_gcn_rows_received": (_I, [_P, _I, C.POINTER(C.c_longlong)]),
     "drone_gcn_train_epoch": (_I, [_P, C.POINTER(_F), C.POINTER(_F)]),
     "drone_gcn_eval": (_I, [_P, _I, C.POINTER(_F), C.POINTER(_F)]),
     "drone_gcn_tensor": (_I, [_P, C.c_char_p, C.POINTER(_P), C.POINTER(_I), C.POINTER(_I), C.POINTER(_I)]),

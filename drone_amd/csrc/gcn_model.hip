@@ -43,17 +43,18 @@ struct drone_gcn {
     drone_gcn_mod::GCN *model;
 };
 
-extern "C" int drone_gcn_create(struct drone_gcn **out, const drone_gcn_config *cfg, int64_t nnz, const int *rp,
-                                const int *ci, const int *in_degree, const int *out_degree, float *X, int ldx,
-                                const int *label, const int *split, const float *W1, const float *W2,
-                                drone_stream_t stream)
+namespace {
+int make_model(struct drone_gcn **out, const drone_gcn_config *cfg, int64_t nnz, const int *rp, const int *ci,
+               const int *in_degree, const int *out_degree, float *X, int ldx, const int *label, const int *split,
+               const float *W1, const float *W2, drone_stream_t stream, const drone_gcn_mod::Replicas *rep)
 {
-    clear_error();
     DRONE_REQUIRE(out && cfg, "null handle / config");
     DRONE_REQUIRE(cfg->n > 0 && cfg->input_dim > 0 && cfg->hidden_dim > 0 && cfg->output_dim > 0, "dimensions");
     DRONE_REQUIRE(nnz >= 0 && nnz < INT32_MAX && rp && (ci || nnz == 0) && in_degree && out_degree, "graph arrays");
     DRONE_REQUIRE(X && ldx >= cfg->input_dim && label && split && W1 && W2, "feature / label / weight arrays");
     DRONE_REQUIRE(cfg->dropout >= 0.0f && cfg->dropout < 1.0f, "dropout probability");
+    DRONE_REQUIRE(!(cfg->fold_input_aggregation && rep && rep->workerNum > 1),
+                  "fold_input_aggregation needs a single subgraph");
     drone_gcn_mod::GCNParams p;
     p.localVertexSize = cfg->n;
     p.input_dim = cfg->input_dim;
@@ -66,10 +67,44 @@ extern "C" int drone_gcn_create(struct drone_gcn **out, const drone_gcn_config *
     p.use_adam = cfg->use_adam != 0;
     p.mean_gradient = cfg->mean_gradient != 0;
     p.seed = cfg->seed;
+    p.fold_input_aggregation = cfg->fold_input_aggregation != 0;
     struct drone_gcn *h = new drone_gcn();
-    h->model = new drone_gcn_mod::GCN(p, nnz, rp, ci, in_degree, out_degree, X, ldx, label, split, W1, W2, stream);
+    h->model = new drone_gcn_mod::GCN(p, nnz, rp, ci, in_degree, out_degree, X, ldx, label, split, W1, W2, stream, rep);
     *out = h;
     return DRONE_OK;
+}
+}  // namespace
+
+extern "C" int drone_gcn_create(struct drone_gcn **out, const drone_gcn_config *cfg, int64_t nnz, const int *rp,
+                                const int *ci, const int *in_degree, const int *out_degree, float *X, int ldx,
+                                const int *label, const int *split, const float *W1, const float *W2,
+                                drone_stream_t stream)
+{
+    clear_error();
+    return make_model(out, cfg, nnz, rp, ci, in_degree, out_degree, X, ldx, label, split, W1, W2, stream, nullptr);
+}
+
+extern "C" int drone_gcn_create_worker(struct drone_gcn **out, const drone_gcn_config *cfg, Graph *g, Comm *comm,
+                                       int workerId, int workerNum, int semi_batch, int compress, const int *in_degree,
+                                       const int *out_degree, float *X, int ldx, const int *label, const int *split,
+                                       const float *W1, const float *W2)
+{
+    clear_error();
+    DRONE_REQUIRE(g && g->ext && comm && cfg, "null graph / communicator / config");
+    DRONE_REQUIRE(workerNum >= 1 && workerId >= 0 && workerId < workerNum, "worker id / count");
+    DRONE_REQUIRE(cfg->n == *g->localVertexSize, "cfg->n is not the subgraph's local vertex count");
+    DRONE_REQUIRE(workerNum == 1 || comm->comm, "workerNum > 1 needs a transport in Comm::comm (see drone_loopback_attach)");
+    DRONE_HIP_TRY(hipSetDevice(g->GID));
+    drone_gcn_mod::Replicas rep;
+    rep.graph = g;
+    rep.comm = comm;
+    rep.workerId = workerId;
+    rep.workerNum = workerNum;
+    rep.semi_batch = semi_batch != 0;
+    rep.compress = compress != 0;
+    // the model works on the communicator's stream, so its kernels and the row synchronisation are ordered
+    return make_model(out, cfg, (int64_t)*g->edgeSize, g->index, g->dst, in_degree, out_degree, X, ldx, label, split, W1,
+                      W2, comm->s, &rep);
 }
 
 extern "C" int drone_gcn_destroy(struct drone_gcn *h)
@@ -130,6 +165,26 @@ extern "C" int drone_gcn_read_metrics(struct drone_gcn *h, float *loss, float *a
     return DRONE_OK;
 }
 
+extern "C" int drone_gcn_read_losses(struct drone_gcn *h, float *cross_entropy, float *l2_penalty)
+{
+    clear_error();
+    DRONE_REQUIRE(h != nullptr, "handle");
+    float ce = 0.0f;
+    const auto r = h->model->read_metrics(&ce);
+    if (cross_entropy) *cross_entropy = ce;
+    if (l2_penalty) *l2_penalty = r.first - ce;
+    return DRONE_OK;
+}
+
+extern "C" int drone_gcn_rows_received(struct drone_gcn *h, int layer, long long *out4)
+{
+    clear_error();
+    DRONE_REQUIRE(h && out4 && (layer == 0 || layer == 1), "handle / layer");
+    const drone_gcn_mod::GraphSum *gs = layer == 0 ? h->model->graphsum1 : h->model->graphsum2;
+    for (int i = 0; i < 4; ++i) out4[i] = gs ? gs->received[i / 2][i % 2] : 0;
+    return DRONE_OK;
+}
+
 extern "C" int drone_gcn_train_epoch(struct drone_gcn *h, float *loss, float *accuracy)
 {
     clear_error();
@@ -161,10 +216,10 @@ extern "C" int drone_gcn_tensor(struct drone_gcn *h, const char *name, void **pt
         {"W1", m->layer1_weight, false},  {"dW1", m->layer1_weight, true},  {"H1", m->layer1_var2, false},
         {"dH1", m->layer1_var2, true},    {"T2", m->layer2_var1, false},    {"dT2", m->layer2_var1, true},
         {"W2", m->layer2_weight, false},  {"dW2", m->layer2_weight, true},  {"Z", m->output, false},
-        {"dZ", m->output, true},
+        {"dZ", m->output, true},          {"AX", m->aggregated_input, false},
     };
     for (const Entry &e : table)
-        if (strcmp(e.name, name) == 0) {
+        if (strcmp(e.name, name) == 0 && e.v != nullptr) {
             *ptr = e.grad ? e.v->grad : e.v->data;
             if (rows) *rows = e.v->rows;
             if (cols) *cols = e.v->cols;

@@ -75,7 +75,7 @@ __global__ __launch_bounds__(kThreads) void cross_entropy_kernel(int n, int clas
     for (int row = blockIdx.x * (kThreads / kWave) + wave; row < n; row += gridDim.x * (kThreads / kWave)) {
         const float *z = logits + (size_t)row * ld;
         const int t = truth[row];
-        if (t < 0) {
+        if (t < 0 || t >= classes) {  // unlabelled (a label outside the classes counts as none)
             if (grad) for (int j = lane; j < classes; j += kWave) grad[(size_t)row * ldg + j] = 0.0f;
             continue;
         }
@@ -133,11 +133,12 @@ __global__ __launch_bounds__(kThreads) void cross_entropy_finish_kernel(int bloc
     }
 }
 
-// cuda_gcn.cu:226-246: a labelled row is wrong iff some logit is strictly greater than the true-class logit.
+// cuda_gcn.cu:226-246: a labelled row is wrong iff some logit is strictly greater than the true-class logit; rows of
+// mirrors (skip[row] != -1, the reference's Mirror2WorkerHost) are left out of the counts (:234).
 // pred[row] = arg-max with ties to the lowest index (optional).  counts[0] += correct, counts[1] += labelled.
 __global__ __launch_bounds__(kThreads) void accuracy_kernel(int n, int classes, const float *__restrict__ logits, int ld,
-                                                            const int *__restrict__ truth, int *__restrict__ pred,
-                                                            int *__restrict__ counts)
+                                                            const int *__restrict__ truth, const int *__restrict__ skip,
+                                                            int *__restrict__ pred, int *__restrict__ counts)
 {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     int correct = 0, total = 0;
@@ -158,7 +159,7 @@ __global__ __launch_bounds__(kThreads) void accuracy_kernel(int n, int classes, 
         if (lane == 0) {
             if (pred) pred[row] = arg;
             const int t = truth ? truth[row] : -1;
-            if (t >= 0) {
+            if (t >= 0 && t < classes && !(skip && skip[row] != -1)) {
                 total++;
                 if (!(best > z[t])) correct++;
             }
@@ -176,6 +177,22 @@ __global__ __launch_bounds__(kThreads) void accuracy_kernel(int n, int classes, 
             atomicAdd(&counts[1], t);
         }
     }
+}
+
+// out[0] = sum of x[i]^2, accumulated in double by one work-group in a fixed order (weights are small)
+__global__ __launch_bounds__(kThreads) void sum_squares_kernel(const float *__restrict__ x, int64_t n,
+                                                               float *__restrict__ out)
+{
+    __shared__ double s_part[kThreads];
+    double t = 0.0;
+    for (int64_t i = threadIdx.x; i < n; i += kThreads) t += (double)x[i] * (double)x[i];
+    s_part[threadIdx.x] = t;
+    __syncthreads();
+    for (int m = kThreads / 2; m > 0; m >>= 1) {
+        if (threadIdx.x < m) s_part[threadIdx.x] += s_part[threadIdx.x + m];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[0] = (float)s_part[0];
 }
 
 __global__ void sgd_kernel(float *__restrict__ w, const float *__restrict__ g, int64_t n, float lr)
@@ -284,15 +301,24 @@ extern "C" int drone_cross_entropy_f32(int n, int classes, const float *logits, 
     return DRONE_OK;
 }
 
-extern "C" int drone_accuracy_f32(int n, int classes, const float *logits, int ld, const int *truth, int *pred,
-                                  int *counts, drone_stream_t stream)
+extern "C" int drone_sum_squares_f32(const float *x, int64_t n, float *out, drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(n >= 0 && (n == 0 || x) && out, "null operand");
+    sum_squares_kernel<<<1, kThreads, 0, as_stream(stream)>>>(x, n, out);
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
+extern "C" int drone_accuracy_f32(int n, int classes, const float *logits, int ld, const int *truth, const int *skip,
+                                  int *pred, int *counts, drone_stream_t stream)
 {
     clear_error();
     DRONE_REQUIRE(n > 0 && classes > 0 && logits && ld >= classes, "operands");
     hipStream_t s = as_stream(stream);
     int blocks = (int)ceil_div(n, kThreads / kWave);
     if (blocks > 1024) blocks = 1024;
-    accuracy_kernel<<<blocks, kThreads, 0, s>>>(n, classes, logits, ld, truth, pred, counts);
+    accuracy_kernel<<<blocks, kThreads, 0, s>>>(n, classes, logits, ld, truth, skip, pred, counts);
     DRONE_HIP_TRY(hipGetLastError());
     return DRONE_OK;
 }

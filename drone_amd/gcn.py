@@ -120,15 +120,24 @@ def cross_entropy(logits, truth, classes=None, grad=None, grad_scale=1.0, stream
     return loss, count
 
 
-def accuracy(logits, truth, classes=None, want_pred=False, stream=0):
+def accuracy(logits, truth, classes=None, want_pred=False, stream=0, skip=None):
+    """skip: int32 [n] on the device (Mirror2Worker): rows whose entry is not -1 are left out of the counts."""
     import torch
     n = logits.shape[0]
     classes = logits.shape[1] if classes is None else classes
     counts = torch.zeros(2, dtype=torch.int32, device=logits.device)
     pred = torch.empty(n, dtype=torch.int32, device=logits.device) if want_pred else None
-    check(lib().drone_accuracy_f32(n, classes, _ptr(logits), logits.stride(0), _ptr(truth), _ptr(pred), _ptr(counts),
-                                   stream))
+    check(lib().drone_accuracy_f32(n, classes, _ptr(logits), logits.stride(0), _ptr(truth), _ptr(skip), _ptr(pred),
+                                   _ptr(counts), stream))
     return counts, pred
+
+
+def sum_squares(x, stream=0):
+    """drone_sum_squares_f32: device scalar = sum of x^2 (the L2 penalty's reduction, cuda_gcn.cu:254-260)."""
+    import torch
+    out = torch.empty(1, dtype=torch.float32, device=x.device)
+    check(lib().drone_sum_squares_f32(_ptr(x), x.numel(), _ptr(out), stream))
+    return out
 
 
 def sgd_step(w, g, lr, stream=0):
@@ -146,19 +155,31 @@ class GcnModel:
     label/split: int32 (split 1 = train), W1/W2: float32 initial weights."""
 
     def __init__(self, rp, ci, in_deg, out_deg, X, label, split, W1, W2, dropout=0.5, lr=0.01, weight_decay=5e-4,
-                 use_dropout=False, use_adam=True, mean_gradient=False, seed=1234, stream=0):
+                 use_dropout=False, use_adam=True, mean_gradient=False, seed=1234, stream=0, fold_input_aggregation=False,
+                 worker=None):
+        """worker: None for a whole graph, or dict(g=Graph pointer, comm=Comm, workerId=, workerNum=, semi_batch=False,
+        compress=False) for one subgraph of a vertex cut (drone_gcn_create_worker); rp / ci are then ignored (the
+        adjacency is the subgraph's own out-edge CSR) and in_deg / out_deg are the GLOBAL degrees per local vertex."""
         from ._lib import GcnConfig
         n, input_dim = X.shape
         hidden, classes = W1.shape[1], W2.shape[1]
         assert W1.shape[0] == input_dim and W2.shape[0] == hidden and W1.is_contiguous() and W2.is_contiguous()
         assert X.stride(1) == 1
-        cfg = GcnConfig(n, input_dim, hidden, classes, dropout, lr, weight_decay, int(use_dropout), int(use_adam), int(mean_gradient), seed)
-        self._keep = (rp, ci, in_deg, out_deg, X, label, split)
+        cfg = GcnConfig(n, input_dim, hidden, classes, dropout, lr, weight_decay, int(use_dropout), int(use_adam),
+                        int(mean_gradient), seed, int(fold_input_aggregation))
+        self._keep = (rp, ci, in_deg, out_deg, X, label, split, worker)
         self.n, self.input_dim, self.hidden, self.classes = n, input_dim, hidden, classes
-        self.nnz = ci.numel()
         h = C.c_void_p()
-        check(lib().drone_gcn_create(C.byref(h), C.byref(cfg), self.nnz, _ptr(rp), _ptr(ci), _ptr(in_deg), _ptr(out_deg),
-                                     _ptr(X), X.stride(0), _ptr(label), _ptr(split), _ptr(W1), _ptr(W2), stream))
+        if worker is None:
+            self.nnz = ci.numel()
+            check(lib().drone_gcn_create(C.byref(h), C.byref(cfg), self.nnz, _ptr(rp), _ptr(ci), _ptr(in_deg), _ptr(out_deg),
+                                         _ptr(X), X.stride(0), _ptr(label), _ptr(split), _ptr(W1), _ptr(W2), stream))
+        else:
+            check(lib().drone_gcn_create_worker(C.byref(h), C.byref(cfg), worker["g"], C.byref(worker["comm"]),
+                                                int(worker["workerId"]), int(worker["workerNum"]),
+                                                int(worker.get("semi_batch", False)), int(worker.get("compress", False)),
+                                                _ptr(in_deg), _ptr(out_deg), _ptr(X), X.stride(0), _ptr(label), _ptr(split),
+                                                _ptr(W1), _ptr(W2)))
         self.h = h
 
     def set_truth(self, split):
@@ -180,6 +201,17 @@ class GcnModel:
         loss, acc = C.c_float(0), C.c_float(0)
         check(lib().drone_gcn_read_metrics(self.h, C.byref(loss), C.byref(acc)))
         return loss.value, acc.value
+
+    def read_losses(self):
+        """(mean cross-entropy, L2 penalty) of the last forward pass; read_metrics() reports their sum."""
+        ce, l2 = C.c_float(0), C.c_float(0)
+        check(lib().drone_gcn_read_losses(self.h, C.byref(ce), C.byref(l2)))
+        return ce.value, l2.value
+
+    def rows_received(self, layer):
+        out = (C.c_longlong * 4)()
+        check(lib().drone_gcn_rows_received(self.h, int(layer), out))
+        return list(out)
 
     def train_epoch(self):
         loss, acc = C.c_float(0), C.c_float(0)

@@ -53,6 +53,11 @@ class _WorkerCUDA:
     def local2global(self):
         return copy_to_host(self.g.contents.Local2Global, self.n, np.int32)
 
+    def close(self):
+        if self.g:
+            lib().drone_graph_destroy(self.g)
+            self.g = None
+
     def set_edge_len(self, edge_len):
         """Overwrites g->edgeLen (out-edge CSR order), which build_graph fills with 1.0."""
         g = self.g.contents

@@ -3,8 +3,10 @@
 // the C ABI of drone_hip.h.  A maintainer of cuda_gcn can swap CUDAMatmul / CUDAGraphSum / CUDAReLU /
 // CUDADropout / CUDACrossEntropyLoss / CUDAAdam for these classes: constructor arguments keep the
 // reference's meaning (m, n, p; in/out variables; dim), forward(bool)/backward() keep its contract.
-// Differences, all forced by the single-subgraph scope: no mirror/master synchronisation after GraphSum,
-// no clearing of mirror rows before the weight gradient, no weight broadcast/reduce.
+// With a vertex cut over several workers GraphSum synchronises the replicated rows after its SpMM, full or through
+// the stale-row cache on the reference's schedule, and Matmul leaves the mirrors' rows out of the weight gradient,
+// as CUDAGraphSum / CUDAMatmul do.  Not here: the weight broadcast / gradient reduce over workers
+// (cuda_communicate.cu:99-115), which belongs to the wire.
 //
 // Header-only on purpose: it holds host logic only and links against libdrone_hip.so + libamdhip64.
 #pragma once
@@ -154,25 +156,79 @@ struct Adjacency {
     }
 };
 
-// cuda_module.cu:210-250 forward: out = A^T * in (pull over in-edges); :310-341 backward: in.grad = A * out.grad.
+// The replicas of a vertex cut, as CUDAGraphSum receives them (cuda_module.cu:149-160): the subgraph with its routing
+// tables, the communicator (Comm::comm holds a drone_transport), this worker's place, and the two switches the
+// reference keeps in globals (cuda_communicate.cuh: `compress`, `batch_type == SEMI_BATCH`).
+struct Replicas {
+    Graph *graph = nullptr;
+    Comm *comm = nullptr;
+    int workerId = 0, workerNum = 1;
+    bool compress = false;    // uint8 rows on the wire (cuda_compress.cu)
+    bool semi_batch = false;  // stale-row cache between full synchronisations (cuda_cache.cu)
+};
+
+// cuda_module.cu:210-307 forward: out = A^T * in (pull over in-edges), then the replicas' rows are summed at the
+// master and assigned back; :310-389 backward: in.grad = A * out.grad, then the same for the gradient rows.
 class GraphSum : public Module {
     Variable *in, *out;
     Adjacency *adj;
     int dim;
     drone_stream_t s;
+    Replicas rep;
+    drone_row_cache *cache = nullptr;  // CacheBuffer (cuda_module.cu:156-158), SEMI_BATCH only
+    int train_step = 0;                // cuda_module.cu:159, advanced at the end of backward (:388)
+    // values: full at step 0 and when step % 100 == 5 (cuda_module.cu:268); gradients: full when step % 10 == 0 (:364)
+    void sync(int kind, float *rows, int ld)
+    {
+        if (rep.workerNum <= 1) return;
+        // the synchronisation runs on the communicator's stream and blocks the host; the product must be there first
+        if (rep.comm->s != s) DRONE_GCN_HIP(hipStreamSynchronize(static_cast<hipStream_t>(s)));
+        const bool full = !rep.semi_batch ||
+                          (kind == 0 ? (train_step == 0 || train_step % 100 == 5) : (train_step % 10 == 0));
+        int up = 0, down = 0;
+        if (!rep.semi_batch) {
+            DRONE_GCN_CHECK(drone_graphsum_sync_rows_f32(rep.graph, rows, ld, dim, rep.workerId, rep.workerNum, rep.comm,
+                                                         rep.compress, &up, &down));
+        } else if (full) {
+            DRONE_GCN_CHECK(drone_graphsum_refresh_rows_cached_f32(rep.graph, cache, kind, rows, ld, dim, rep.workerId,
+                                                                   rep.workerNum, rep.comm, rep.compress, &up, &down));
+        } else {
+            DRONE_GCN_CHECK(drone_graphsum_sync_rows_cached_f32(rep.graph, cache, kind, error_rate[kind], rows, ld, dim,
+                                                                rep.workerId, rep.workerNum, rep.comm, rep.compress, &up,
+                                                                &down));
+            if (kind == 0 && update_threshold) error_rate[0] *= 0.9f;  // cuda_cache.cu:416-418
+        }
+        received[kind][0] += up;
+        received[kind][1] += down;
+    }
 public:
-    GraphSum(Variable *in_, Variable *out_, Adjacency *adj_, int dim_, std::string name, drone_stream_t stream)
-        : in(in_), out(out_), adj(adj_), dim(dim_), s(stream) { ModuleName = std::move(name); }
+    float error_rate[2] = {0.1f, 0.0f};  // cuda_cache.cu:70-71
+    bool update_threshold = false;       // cuda_cache.cu:416
+    long long received[2][2] = {{0, 0}, {0, 0}};  // rows that arrived: [values | gradients][mirror->master | master->mirror]
+    GraphSum(Variable *in_, Variable *out_, Adjacency *adj_, int dim_, std::string name, drone_stream_t stream,
+             const Replicas *replicas = nullptr)
+        : in(in_), out(out_), adj(adj_), dim(dim_), s(stream)
+    {
+        ModuleName = std::move(name);
+        if (replicas) rep = *replicas;
+        if (rep.workerNum > 1 && rep.semi_batch)
+            DRONE_GCN_CHECK(drone_row_cache_create(&cache, rep.graph, rep.workerNum, dim));
+    }
+    ~GraphSum() override { if (cache) drone_row_cache_destroy(cache); }
     void forward(bool) override
     {
         DRONE_GCN_CHECK(drone_spmm_csr_f32(adj->planT, adj->rpT, adj->ciT, adj->valT, in->data, in->ld, out->data,
                                            out->ld, dim, 1.0f, 0.0f, s));
+        sync(0, out->data, out->ld);
     }
     void backward() override
     {
         DRONE_GCN_CHECK(drone_spmm_csr_f32(adj->plan, adj->rp, adj->ci, adj->val, out->grad, out->ld, in->grad,
                                            in->ld, dim, 1.0f, 0.0f, s));
+        sync(1, in->grad, in->ld);
+        train_step++;
     }
+    int step() const { return train_step; }
 };
 
 // cuda_module.cu:498-523.  The mask covers the padded rows x ld extent (padding stays zero).
@@ -313,6 +369,12 @@ struct GCNParams {
     bool use_adam = true;       // reference optimiser; false = SGD
     bool mean_gradient = false; // false = sum-reduced loss gradient as in the reference (cuda_module.cu:452)
     uint64_t seed = 1234;       // cuda_kernel.cu:426 seeds cuRAND with 1234
+    // The input features carry no gradient (cuda_gcn.cu:32) and no module changes them, so A^T (X W1) = (A^T X) W1:
+    // with this switch A^T X is aggregated once, when the model is made, and layer 1 becomes a single product with
+    // it, forward (H1 = (A^T X) W1) and backward (dW1 = (A^T X)^T dH1); both 'hidden_dim'-wide aggregations leave
+    // the step.  Same numbers up to summation order.  Single subgraph only: with replicas the aggregated rows of X
+    // would have to be synchronised first, and the reference has no such step.
+    bool fold_input_aggregation = false;
 };
 
 // cuda_gcn.cu:9-99 (module list) and :119-170, 287-306 (forward / backward / train_epoch).
@@ -325,6 +387,11 @@ public:
     std::unique_ptr<Optimizer> optimizer;
     Variable *input = nullptr, *layer1_var1 = nullptr, *layer1_weight = nullptr, *layer1_var2 = nullptr,
              *layer2_var1 = nullptr, *layer2_weight = nullptr, *output = nullptr;
+    Variable *aggregated_input = nullptr;  // A^T X, with fold_input_aggregation
+    GraphSum *graphsum1 = nullptr, *graphsum2 = nullptr;
+    Replicas replicas;
+    const int *mirror2worker = nullptr;    // device [N] (Graph::Mirror2Worker) with replicas, else null
+    float *l2_sum = nullptr;               // device scalar: sum of W1^2 (cuda_gcn.cu:254-260)
     CrossEntropyLoss *ce = nullptr;
     ReLU *relu = nullptr;
     Dropout *drop = nullptr;
@@ -335,14 +402,24 @@ public:
     drone_stream_t s;
 
     // X: device N x input_dim with leading dimension ldx (borrowed).  W1 / W2: device initial weights (copied).
+    // rep: the vertex cut this subgraph belongs to (null: a whole graph).  rp / ci: the subgraph's out-edge CSR
+    // (Graph::index / Graph::dst with replicas); in_degree / out_degree: global degrees per local vertex.
     GCN(const GCNParams &p, int64_t nnz, const int *rp, const int *ci, const int *in_degree, const int *out_degree,
-        float *X, int ldx, const int *label_, const int *split_, const float *W1, const float *W2, drone_stream_t stream)
+        float *X, int ldx, const int *label_, const int *split_, const float *W1, const float *W2, drone_stream_t stream,
+        const Replicas *rep = nullptr)
         : params(p), label(label_), split(split_), s(stream)
     {
         const int N = p.localVertexSize;
+        if (rep) replicas = *rep;
+        const bool cut = replicas.workerNum > 1;
+        if (cut) mirror2worker = replicas.graph->Mirror2Worker;  // cuda_gcn.cu:44,72
+        if (cut && p.fold_input_aggregation) {
+            printf("drone_gcn: fold_input_aggregation needs a single subgraph (workerNum = %d)\n", replicas.workerNum);
+            exit(EXIT_FAILURE);
+        }
         auto add = [&](Variable *v) { variables.emplace_back(v); return v; };
         input = add(new Variable(N, p.input_dim, false, false, X, ldx));
-        layer1_var1 = add(new Variable(N, p.hidden_dim, true, false));
+        if (!p.fold_input_aggregation) layer1_var1 = add(new Variable(N, p.hidden_dim, true, false));
         layer1_weight = add(new Variable(p.input_dim, p.hidden_dim, true, true));
         layer1_var2 = add(new Variable(N, p.hidden_dim, true, false));
         layer2_var1 = add(new Variable(N, p.output_dim, true, false));
@@ -354,17 +431,35 @@ public:
         adj.reset(new Adjacency(N, nnz, rp, ci, in_degree, out_degree, max_dim, s));
         DRONE_GCN_HIP(hipMalloc(&truth, sizeof(int) * (size_t)N));
         DRONE_GCN_HIP(hipMalloc(&counts, sizeof(int) * 2));
+        DRONE_GCN_HIP(hipMalloc(&l2_sum, sizeof(float)));
+        const Replicas *r = cut ? &replicas : nullptr;
 
-        modules.emplace_back(new Matmul(input, layer1_weight, layer1_var1, N, p.input_dim, p.hidden_dim, "matmul_layer1", s));
-        modules.emplace_back(new GraphSum(layer1_var1, layer1_var2, adj.get(), p.hidden_dim, "graphSum_layer1", s));
+        if (p.fold_input_aggregation) {
+            // A^T X once, max_dim columns at a time (the plan's width); layer 1 is then one product with it
+            aggregated_input = add(new Variable(N, p.input_dim, false, false));
+            for (int c0 = 0; c0 < p.input_dim; c0 += max_dim) {
+                const int k = p.input_dim - c0 < max_dim ? p.input_dim - c0 : max_dim;
+                DRONE_GCN_CHECK(drone_spmm_csr_f32(adj->planT, adj->rpT, adj->ciT, adj->valT, input->data + c0, input->ld,
+                                                   aggregated_input->data + c0, aggregated_input->ld, k, 1.0f, 0.0f, s));
+            }
+            modules.emplace_back(new Matmul(aggregated_input, layer1_weight, layer1_var2, N, p.input_dim, p.hidden_dim,
+                                            "matmul_layer1_folded", s));
+        } else {
+            modules.emplace_back(new Matmul(input, layer1_weight, layer1_var1, N, p.input_dim, p.hidden_dim, "matmul_layer1", s,
+                                            mirror2worker));
+            graphsum1 = new GraphSum(layer1_var1, layer1_var2, adj.get(), p.hidden_dim, "graphSum_layer1", s, r);
+            modules.emplace_back(graphsum1);
+        }
         relu = new ReLU(layer1_var2, "Relu", s);
         modules.emplace_back(relu);
         if (p.use_dropout) {
             drop = new Dropout(layer1_var2, p.dropout, p.seed, "dropout_layer1", s);
             modules.emplace_back(drop);
         }
-        modules.emplace_back(new Matmul(layer1_var2, layer2_weight, layer2_var1, N, p.hidden_dim, p.output_dim, "matmul_layer2", s));
-        modules.emplace_back(new GraphSum(layer2_var1, output, adj.get(), p.output_dim, "graphSum_layer2", s));
+        modules.emplace_back(new Matmul(layer1_var2, layer2_weight, layer2_var1, N, p.hidden_dim, p.output_dim, "matmul_layer2", s,
+                                        mirror2worker));
+        graphsum2 = new GraphSum(layer2_var1, output, adj.get(), p.output_dim, "graphSum_layer2", s, r);
+        modules.emplace_back(graphsum2);
         ce = new CrossEntropyLoss(output, truth, p.output_dim, "CrossEntropy", s);
         modules.emplace_back(ce);
         if (p.use_adam) {
@@ -382,10 +477,17 @@ public:
     {
         (void)hipFree(truth);
         (void)hipFree(counts);
+        (void)hipFree(l2_sum);
     }
 
     void set_truth(int current_split);  // cuda_gcn.cu:211-223; defined in gcn_model.hip (needs a kernel)
-    void forward(bool training) { for (auto &m : modules) m->forward(training); }
+    // The modules in order, then the counts and sums read_metrics() reports (cuda_gcn.cu:298-299 takes them right
+    // after the forward pass too).
+    void forward(bool training)
+    {
+        for (auto &m : modules) m->forward(training);
+        metrics_async();
+    }
     void backward() { for (int i = (int)modules.size() - 1; i >= 0; --i) modules[i]->backward(); }
 
     // Enqueues one training step (cuda_gcn.cu:287-306 without the host read-backs): forward, accuracy counts,
@@ -393,20 +495,31 @@ public:
     void train_step_async()
     {
         forward(true);
-        DRONE_GCN_HIP(hipMemsetAsync(counts, 0, sizeof(int) * 2, static_cast<hipStream_t>(s)));
-        DRONE_GCN_CHECK(drone_accuracy_f32(params.localVertexSize, params.output_dim, output->data, output->ld, truth,
-                                           nullptr, counts, s));
         backward();
         optimizer->step();
     }
-    std::pair<float, float> read_metrics()
+    // cuda_gcn.cu:298-299, 314-315: what train_epoch / eval report besides the loss - the accuracy over the labelled
+    // rows that are not mirrors (:226-246) and the L2 penalty weight_decay * sum(W1^2) / 2 (:254-260) - taken from the
+    // weights as they are before the optimiser step, left on the device.
+    void metrics_async()
     {
-        float loss = 0.0f;
+        DRONE_GCN_HIP(hipMemsetAsync(counts, 0, sizeof(int) * 2, static_cast<hipStream_t>(s)));
+        DRONE_GCN_CHECK(drone_accuracy_f32(params.localVertexSize, params.output_dim, output->data, output->ld, truth,
+                                           mirror2worker, nullptr, counts, s));
+        DRONE_GCN_CHECK(drone_sum_squares_f32(layer1_weight->data, (int64_t)layer1_weight->rows * layer1_weight->ld, l2_sum, s));
+    }
+    // {loss + L2 penalty, accuracy} of the last forward pass, as CUDAGCN::train_epoch / eval return them.
+    // cross_entropy (optional): the mean cross-entropy alone.
+    std::pair<float, float> read_metrics(float *cross_entropy = nullptr)
+    {
+        float loss = 0.0f, l2 = 0.0f;
         int c[2] = {0, 0};
         DRONE_GCN_HIP(hipStreamSynchronize(static_cast<hipStream_t>(s)));
         DRONE_GCN_HIP(hipMemcpy(&loss, ce->d_loss, sizeof(float), hipMemcpyDeviceToHost));
+        DRONE_GCN_HIP(hipMemcpy(&l2, l2_sum, sizeof(float), hipMemcpyDeviceToHost));
         DRONE_GCN_HIP(hipMemcpy(c, counts, sizeof(int) * 2, hipMemcpyDeviceToHost));
-        return {loss, c[1] ? (float)c[0] / (float)c[1] : 0.0f};
+        if (cross_entropy) *cross_entropy = loss;
+        return {loss + params.weight_decay * l2 / 2, c[1] ? (float)c[0] / (float)c[1] : 0.0f};
     }
     std::pair<float, float> train_epoch()
     {
@@ -418,9 +531,6 @@ public:
     {
         set_truth(current_split);
         forward(false);
-        DRONE_GCN_HIP(hipMemsetAsync(counts, 0, sizeof(int) * 2, static_cast<hipStream_t>(s)));
-        DRONE_GCN_CHECK(drone_accuracy_f32(params.localVertexSize, params.output_dim, output->data, output->ld, truth,
-                                           nullptr, counts, s));
         return read_metrics();
     }
 };

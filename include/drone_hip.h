@@ -240,17 +240,21 @@ int drone_relu_backward_f32(float *grad, const uint8_t *mask, int64_t n, drone_s
  * forward activations and the backward gradients. */
 int drone_dropout_mask(uint8_t *keep, int64_t n, uint64_t seed, uint64_t step, float p, drone_stream_t stream);
 int drone_dropout_apply_f32(float *x, const uint8_t *keep, int64_t n, float p, drone_stream_t stream);
-/* cuda_kernel.cu:295-379 + cuda_module.cu:406-483.  truth[i] < 0 = unlabelled.  grad (optional) receives
+/* cuda_kernel.cu:295-379 + cuda_module.cu:406-483.  truth[i] < 0 (or >= classes) = unlabelled.  grad (optional) receives
  * grad_scale * (softmax - onehot) on labelled rows and 0 elsewhere.  grad_scale = 1 is the reference's
  * SUM-reduced gradient (count_grad = 1, cuda_module.cu:452); 1/labelled-count gives the mean-reduced one.
  * *loss_out (device) = mean loss over labelled rows, *count_out (device) = their number. */
 int drone_cross_entropy_f32(int n, int classes, const float *logits, int ld, const int *truth, float *grad,
                             int ldg, float grad_scale, float *loss_out, int *count_out, drone_stream_t stream);
 /* cuda_gcn.cu:226-246: a labelled row is correct unless some logit is strictly greater than the true-class
- * logit.  counts[0] += correct, counts[1] += labelled (device ints, zeroed by the caller); pred (optional)
- * receives the arg-max with ties to the lowest index. */
-int drone_accuracy_f32(int n, int classes, const float *logits, int ld, const int *truth, int *pred,
-                       int *counts, drone_stream_t stream);
+ * logit; rows with skip[row] != -1 are not counted (:234 passes Mirror2Worker, so a replicated vertex is counted
+ * on its master's worker only; skip may be NULL).  counts[0] += correct, counts[1] += counted (device ints,
+ * zeroed by the caller); pred (optional) receives the arg-max with ties to the lowest index. */
+int drone_accuracy_f32(int n, int classes, const float *logits, int ld, const int *truth, const int *skip,
+                       int *pred, int *counts, drone_stream_t stream);
+/* out[0] (device) = sum of x[i]^2: the thrust transform + reduce of CUDAGCN::get_l2_penalty (cuda_gcn.cu:254-260),
+ * whose caller multiplies by weight_decay / 2. */
+int drone_sum_squares_f32(const float *x, int64_t n, float *out, drone_stream_t stream);
 /* w -= lr * g (the optimiser the benchmark configuration names). */
 int drone_sgd_step_f32(float *w, const float *g, int64_t n, float lr, drone_stream_t stream);
 /* cuda_module.cu:590-600 + cuda_kernel.cu:450-460; step_count is the value after the increment. */
@@ -276,10 +280,29 @@ typedef struct drone_gcn_config {
     int mean_gradient; /* 0 = sum-reduced loss gradient as in the reference (cuda_module.cu:452); 1 = divided by
                           the number of labelled rows, which a plain SGD step needs to stay stable */
     uint64_t seed;   /* dropout mask stream */
+    int fold_input_aggregation; /* 0 = the reference's module list.  1 = the input features carry no gradient
+                          (cuda_gcn.cu:32), so A^T (X W1) = (A^T X) W1: A^T X is aggregated once at creation and
+                          layer 1 becomes one product with it, forward and backward; both hidden_dim-wide
+                          aggregations leave the step (same results up to summation order; tensors T1 / dT1 do not
+                          exist then, AX does).  Single subgraph only. */
 } drone_gcn_config;
 int drone_gcn_create(drone_gcn **handle, const drone_gcn_config *cfg, int64_t nnz, const int *rp, const int *ci,
                      const int *in_degree, const int *out_degree, float *X, int ldx, const int *label,
                      const int *split, const float *W1, const float *W2, drone_stream_t stream);
+/* The model of one worker of a vertex cut, as CUDAGCN is built per worker (cuda_gcn.cu:9-99): the subgraph `g`
+ * (build_graph + addMasterRoute / addMirrorRoute; its out-edge CSR Graph::index / Graph::dst is the adjacency), the
+ * communicator whose Comm::comm holds the transport and whose stream the model works on, and the reference's two
+ * global switches: semi_batch (stale-row cache between full synchronisations, cuda_module.cu:268, :364) and compress
+ * (uint8 rows on the wire).  in_degree / out_degree: GLOBAL degrees per local vertex (parser.cu:135-160), X / label /
+ * split per local vertex.  Both GraphSum layers then synchronise the replicated rows after their products
+ * (cuda_module.cu:250-307, :343-389), the weight gradients leave out the mirrors' rows (cuda_gcn.cu:44,72), and the
+ * accuracy counts a replicated vertex on its master's worker only (cuda_gcn.cu:234).  Every forward / backward /
+ * train / eval call on such a handle meets the other workers on the wire: drive each worker from its own thread.
+ * The weight broadcast / gradient reduce of cuda_gcn.cu:122,156 is left to the caller (read dW1 / dW2, reduce,
+ * write W1 / W2). */
+int drone_gcn_create_worker(drone_gcn **handle, const drone_gcn_config *cfg, Graph *g, Comm *comm, int workerId,
+                            int workerNum, int semi_batch, int compress, const int *in_degree, const int *out_degree,
+                            float *X, int ldx, const int *label, const int *split, const float *W1, const float *W2);
 int drone_gcn_destroy(drone_gcn *handle);
 int drone_gcn_set_truth(drone_gcn *handle, int split);   /* cuda_gcn.cu:211-223 */
 int drone_gcn_forward(drone_gcn *handle, int training);  /* cuda_gcn.cu:119-144 */
@@ -288,10 +311,18 @@ int drone_gcn_optimizer_step(drone_gcn *handle);         /* cuda_gcn.cu:303 */
 /* forward(training) + accuracy counts + backward + optimiser step, enqueued without host synchronisation;
  * drone_gcn_read_metrics waits and returns the mean training loss and accuracy of the last step. */
 int drone_gcn_train_step_async(drone_gcn *handle);
+/* loss = mean cross-entropy + weight_decay * sum(W1^2) / 2, the train_loss / test_loss of cuda_gcn.cu:298, :314;
+ * accuracy over the labelled rows that are not mirrors (cuda_gcn.cu:226-246). */
 int drone_gcn_read_metrics(drone_gcn *handle, float *loss, float *accuracy);
+/* The two terms of that loss on their own (either may be NULL). */
+int drone_gcn_read_losses(drone_gcn *handle, float *cross_entropy, float *l2_penalty);
+/* Rows that arrived at this worker in the synchronisations of GraphSum layer 0 / 1 so far: out4 = {values
+ * mirror->master, values master->mirror, gradients mirror->master, gradients master->mirror} (the reference's
+ * mirror2master_*_total / master2mirror_*_total counters). */
+int drone_gcn_rows_received(drone_gcn *handle, int layer, long long *out4);
 int drone_gcn_train_epoch(drone_gcn *handle, float *loss, float *accuracy);     /* cuda_gcn.cu:287-306 */
 int drone_gcn_eval(drone_gcn *handle, int split, float *loss, float *accuracy); /* cuda_gcn.cu:308-318 */
-/* Device pointer and shape of a named tensor: X T1 dT1 W1 dW1 H1 dH1 T2 dT2 W2 dW2 Z dZ (float),
+/* Device pointer and shape of a named tensor: X T1 dT1 W1 dW1 H1 dH1 T2 dT2 W2 dW2 Z dZ AX (float),
  * relu_mask keep1 (uint8), truth rpT ciT (int), val valT (float). */
 int drone_gcn_tensor(drone_gcn *handle, const char *name, void **ptr, int *rows, int *cols, int *ld);
 

@@ -403,10 +403,19 @@ def cross_entropy(logits, truth, training=True):
     return loss, grad, cnt.value
 
 
-def accuracy(logits, truth):
+def accuracy(logits, truth, mirror2worker=None):
+    """cuda_gcn.cu:226-246; rows of mirrors (mirror2worker != -1) are skipped like unlabelled ones (:234)."""
     logits, truth = _f32(logits), _i32(truth)
+    if mirror2worker is not None:
+        truth = _i32(np.where(np.asarray(mirror2worker) != -1, -1, truth))
     n, c = logits.shape
     return lib().orc_accuracy(C.c_int(n), C.c_int(c), _p(logits), C.c_int(c), _p(truth))
+
+
+def l2_penalty(W1, weight_decay):
+    """cuda_gcn.cu:254-260 get_l2_penalty: weight_decay * sum(W1^2) / 2, squares and sum in float."""
+    w = _f32(W1).ravel()
+    return float(np.float32(weight_decay) * np.sum(w * w, dtype=np.float32) / np.float32(2))
 
 
 def argmax(logits):
@@ -446,6 +455,39 @@ def gcn_forward_backward(rp, ci, v, rpT, ciT, vT, X, W1, W2, truth, keep1=None, 
         _p(ciT), _p(vT), _p(X), _p(W1), _p(W2), _p(truth), _p(keep1), C.c_float(p_drop), _p(Z), _p(H1),
         _p(dW1), _p(dW2), _p(dT1))
     return dict(loss=loss, Z=Z, H1=H1, dW1=dW1, dW2=dW2, dT1=dT1)
+
+
+def gcn_group_step(tops, graphs, X, W1, W2, truth, compress=False):
+    """One forward + backward pass of every worker of a vertex cut at once: the module list of cuda_gcn.cu:9-99 run
+    per worker (CUDAGCN::forward / backward, :119-170, without the weight broadcast / gradient reduce), with the
+    replicated rows synchronised over all workers after each GraphSum product (values cuda_module.cu:268 ->
+    cuda_communicate.cu:374-448, gradients :364 -> :502-556, full-batch branch) and the mirrors' rows cleared before
+    each weight gradient (cuda_module.cu:89-90).  tops[w]: Part; graphs[w]: dict(rp, ci, val, rpT, ciT, valT) of the
+    worker's local out-edge CSR and its transpose; X[w] / truth[w]: per local vertex.  No dropout (the reference
+    runs without).  Returns per worker dict(loss, count, Z, H1, dT1, dW1, dW2); dT1 as the weight gradient saw it."""
+    W = len(tops)
+    W1, W2 = _f32(W1), _f32(W2)
+    T1 = [sgemm_f32(0, 0, _f32(X[w]), W1) for w in range(W)]
+    P1 = [spmm_f32(g["rpT"], g["ciT"], g["valT"], T1[w]) for w, g in enumerate(graphs)]
+    graphsum_sync_rows(tops, P1, compress)
+    H1, mask = zip(*[relu_forward(P1[w]) for w in range(W)])
+    T2 = [sgemm_f32(0, 0, H1[w], W2) for w in range(W)]
+    Z = [spmm_f32(g["rpT"], g["ciT"], g["valT"], T2[w]) for w, g in enumerate(graphs)]
+    graphsum_sync_rows(tops, Z, compress)
+    ce = [cross_entropy(Z[w], truth[w]) for w in range(W)]              # (mean loss, sum-reduced gradient, count)
+    dT2 = [spmm_f32(g["rp"], g["ci"], g["val"], ce[w][1]) for w, g in enumerate(graphs)]
+    graphsum_sync_rows(tops, dT2, compress)
+    dH1 = [sgemm_f32(0, 1, dT2[w], W2) for w in range(W)]
+    for w in range(W):
+        dT2[w][tops[w].m2w != -1] = 0.0
+    dW2 = [sgemm_f32(1, 0, H1[w], dT2[w]) for w in range(W)]
+    dP1 = [relu_backward(dH1[w], mask[w]) for w in range(W)]
+    dT1 = [spmm_f32(g["rp"], g["ci"], g["val"], dP1[w]) for w, g in enumerate(graphs)]
+    graphsum_sync_rows(tops, dT1, compress)
+    for w in range(W):
+        dT1[w][tops[w].m2w != -1] = 0.0
+    dW1 = [sgemm_f32(1, 0, _f32(X[w]), dT1[w]) for w in range(W)]
+    return [dict(loss=ce[w][0], count=ce[w][2], Z=Z[w], H1=H1[w], dT1=dT1[w], dW1=dW1[w], dW2=dW2[w]) for w in range(W)]
 
 
 # ---- GraphSum replica sync of K-wide rows and the uint8 row compression ----------------------------------------

@@ -102,7 +102,8 @@ def test_tiny_fixture_step(T, oracle, use_dropout, fixture):
     for name in ("Z", "H1", "dW1", "dW2", "dT1"):
         close(m.tensor(name), ref[name], scale=sc[name])
     loss, acc = m.read_metrics()
-    assert loss == pytest.approx(ref["loss"], rel=1e-5)
+    assert m.read_losses()[0] == pytest.approx(ref["loss"], rel=1e-5)
+    assert loss == pytest.approx(ref["loss"] + oracle.l2_penalty(d["W1"], 5e-4), rel=1e-5)   # cuda_gcn.cu:298
     m.optimizer_step()
     W1n = d["W1"].astype(np.float32).copy()
     oracle.sgd_step(W1n, ref["dW1"], 0.01)
@@ -127,12 +128,14 @@ def directed_graph_np(scale, ef, seed):
     return dict(n=n, rp=rp, ci=dst.astype(np.int32), val=val, in_deg=in_deg, out_deg=out_deg)
 
 
+@pytest.mark.parametrize("fold", [False, True], ids=["module-list", "folded-layer1"])
 @pytest.mark.parametrize("scale,ef,fin,hid,cls,use_dropout,directed",
                          [(10, 8, 50, 16, 7, False, False), (11, 16, 602, 128, 41, True, False),
                           (11, 12, 70, 32, 9, True, True)])
-def test_rmat_step_against_oracle(T, oracle, scale, ef, fin, hid, cls, use_dropout, directed):
+def test_rmat_step_against_oracle(T, oracle, scale, ef, fin, hid, cls, use_dropout, directed, fold):
     """Second case keeps the fourth configuration's widths (602 -> 128 -> 41, dropout 0.5, SGD 0.01, 66 % train); the
-    third runs on a directed graph (transpose != itself, in-degree != out-degree)."""
+    third runs on a directed graph (transpose != itself, in-degree != out-degree).  fold: the model aggregates the
+    input features once (A^T X) and runs layer 1 as a single product with them - the same oracle step applies."""
     from drone_amd import graphs, rmat
     g = directed_graph_np(scale, ef, seed=4) if directed else graphs.gcn_graph_np(scale, ef, seed=4)
     n = g["n"]
@@ -143,7 +146,8 @@ def test_rmat_step_against_oracle(T, oracle, scale, ef, fin, hid, cls, use_dropo
     label = rmat.randint_i32(n, seed=43, bound=cls)
     split = np.where(rmat.uniform_f32(n, seed=44, lo=0, hi=1) < 0.66, 1, 2).astype(np.int32)
     truth = np.where(split == 1, label, -1).astype(np.int32)
-    m = make_model(T, g, X, W1, W2, label, split, use_dropout=use_dropout, use_adam=False, lr=0.01, seed=4)
+    m = make_model(T, g, X, W1, W2, label, split, use_dropout=use_dropout, use_adam=False, lr=0.01, seed=4,
+                   fold_input_aggregation=fold)
     # set-up products: edge values and the transposed CSR are exact
     np.testing.assert_array_equal(m.tensor("val"), g["val"])
     rpT, ciT, vT = oracle.csr_transpose(n, n, g["rp"], g["ci"], g["val"])
@@ -159,9 +163,17 @@ def test_rmat_step_against_oracle(T, oracle, scale, ef, fin, hid, cls, use_dropo
         assert abs(keep.mean() - 0.5) < 0.02
     ref = oracle.gcn_forward_backward(g["rp"], g["ci"], g["val"], rpT, ciT, vT, X, W1, W2, truth, keep, 0.5)
     sc = step_scales(n, g["rp"], g["ci"], g["val"], rpT, ciT, vT, X, W1, W2, truth, ref, keep)
-    for name in ("Z", "H1", "dW1", "dW2", "dT1"):
+    for name in ("Z", "H1", "dW1", "dW2") + (() if fold else ("dT1",)):
         close(m.tensor(name), ref[name], scale=sc[name])
-    assert loss == pytest.approx(ref["loss"], rel=1e-4)
+    if fold:
+        import scipy.sparse as sp
+        AX = sp.csr_matrix((vT.astype(np.float64), ciT, rpT), shape=(n, n)) @ X.astype(np.float64)
+        mag = sp.csr_matrix((np.abs(vT).astype(np.float64), ciT, rpT), shape=(n, n)) @ np.abs(X).astype(np.float64)
+        close(m.tensor("AX"), AX, scale=mag)
+        with pytest.raises(Exception, match="unknown tensor"):
+            m.tensor("dT1")
+    assert m.read_losses()[0] == pytest.approx(ref["loss"], rel=1e-4)
+    assert loss == pytest.approx(ref["loss"] + oracle.l2_penalty(W1, 5e-4), rel=1e-4)
     assert acc == pytest.approx(oracle.accuracy(ref["Z"], truth), abs=2.0 / n)
     # identical arg-max predictions
     from drone_amd import gcn

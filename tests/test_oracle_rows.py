@@ -180,3 +180,59 @@ def test_row_cache_staleness_is_bounded_by_the_threshold(oracle):
     assert grp.sync(0, data, 10.0) == ([0] * W, [0] * W)
     for d, p, c in zip(data, prev, grp.cached):
         np.testing.assert_array_equal(d[c], p[c])
+
+
+@pytest.mark.parametrize("W,scale,seed", [(2, 7, 1), (4, 9, 2)])
+def test_gcn_step_over_a_vertex_cut_equals_the_whole_graph(oracle, W, scale, seed):
+    """Partition independence pins the multi-worker step (module order, where the rows are synchronised, which
+    orientation each product aggregates over, the mirrors' rows leaving the weight gradients): summed over the
+    workers the weight gradients equal the whole graph's, every replica's logits equal the whole graph's row, and
+    a worker's loss is the mean cross-entropy of the whole graph's logits over its local labelled rows (mirrors
+    included, as in the reference, whose loss kernel does not look at Mirror2Worker)."""
+    from partition_util import gcn_cut_inputs
+    g, ws = gcn_cut_inputs(oracle, scale, 6, W, seed, fin=11, hid=8, cls=5)
+    ref = oracle.gcn_forward_backward(g["rp"], g["ci"], g["val"], g["rpT"], g["ciT"], g["valT"], g["X"], g["W1"], g["W2"],
+                                      g["truth"])
+    got = oracle.gcn_group_step([w["top"] for w in ws], [w["graph"] for w in ws], [w["X"] for w in ws], g["W1"], g["W2"],
+                                [w["truth"] for w in ws])
+    assert sum(len(w["part"]["mirror_vertex"]) for w in ws) > 0
+    for name in ("dW1", "dW2"):
+        total = sum(r[name].astype(np.float64) for r in got)
+        np.testing.assert_allclose(total, ref[name], rtol=0, atol=2e-5 * np.abs(ref[name]).max())
+    for w, r in zip(ws, got):
+        np.testing.assert_allclose(r["Z"], ref["Z"][w["l2g"]], rtol=0, atol=2e-5 * np.abs(ref["Z"]).max())
+        np.testing.assert_allclose(r["H1"], ref["H1"][w["l2g"]], rtol=0, atol=2e-5 * np.abs(ref["H1"]).max())
+        masters = w["top"].m2w == -1
+        np.testing.assert_allclose(r["dT1"][masters], ref["dT1"][w["l2g"]][masters], rtol=0,
+                                   atol=2e-5 * np.abs(ref["dT1"]).max())
+        assert not r["dT1"][~masters].any()
+        want_loss, _, want_cnt = oracle.cross_entropy(ref["Z"][w["l2g"]], w["truth"])
+        assert r["count"] == want_cnt == int((w["truth"] >= 0).sum())
+        assert r["loss"] == pytest.approx(want_loss, rel=1e-5)
+    masters_labelled = sum(int(((w["truth"] >= 0) & (w["top"].m2w == -1)).sum()) for w in ws)
+    assert masters_labelled == int((g["truth"] >= 0).sum())          # every labelled vertex has exactly one master
+    # leaving the mirrors' rows in would count replicated vertices more than once
+    bad = sum(oracle.sgemm_f32(1, 0, w["X"], _synced_dT1(oracle, ws, got, i)) for i, w in enumerate(ws))
+    assert np.abs(bad - ref["dW1"]).max() > 1e-3 * np.abs(ref["dW1"]).max()
+
+
+def _synced_dT1(oracle, ws, got, i):
+    """dT1 of worker i with its mirrors' rows filled back in from their masters (what the rows held before they were
+    cleared)."""
+    full = got[i]["dT1"].copy()
+    top = ws[i]["top"]
+    for l in np.nonzero(top.m2w != -1)[0]:
+        m = top.m2w[l]
+        full[l] = got[m]["dT1"][ws[m]["top"].g2l[top.l2g[l]]]
+    return full
+
+
+def test_l2_penalty_and_mirror_aware_accuracy(oracle):
+    rng = np.random.default_rng(5)
+    W1 = rng.normal(size=(30, 7)).astype(np.float32)
+    assert oracle.l2_penalty(W1, 5e-4) == pytest.approx(5e-4 * float((W1.astype(np.float64) ** 2).sum()) / 2, rel=1e-5)
+    z = np.array([[1, 2, 0], [5, 1, 0], [0, 3, 0], [1, 0, 2]], np.float32)
+    truth = np.array([1, 1, 1, 2], np.int32)
+    assert oracle.accuracy(z, truth) == pytest.approx(3 / 4)
+    # rows 1 (wrong) and 3 (right) belong to mirrors: only rows 0 and 2 count
+    assert oracle.accuracy(z, truth, np.array([-1, 0, -1, 2])) == 1.0
