@@ -28,6 +28,39 @@ def log(*a):
     print("[bench]", *a, file=sys.stderr, flush=True)
 
 
+PR_KERNELS = ("pr_rowblock_kernel<drone::PrF64Epi>", "pr_rowblock_merge_kernel<drone::PrF64Epi>")
+PR_TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "pr_rowblock_pagerank_c2.hbm_traffic.txt")
+
+
+def pr_traffic_from_profile(path=PR_TRAFFIC_PROFILE):
+    """Fabric bytes per iteration of the PageRank aggregation, from the committed rocprofv3 counter summary: the mean
+    FETCH_SIZE and WRITE_SIZE (KiB per dispatch) of the iteration's kernels, each scaled by what the same counter read
+    for the 1 GiB stream-copy kernel in the same run.  None when the file is missing or does not name these kernels
+    (the summary then describes other code and must be taken again)."""
+    try:
+        rows = {}
+        for line in open(path):
+            if line.startswith("#") or "dispatches" not in line:
+                continue
+            for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+                if f" {counter} " in line:
+                    name = line.split(counter)[0].strip()
+                    rows[(name, counter)] = float(line.split("mean")[1].split()[0])
+        def mean(kernel, counter):
+            hits = [v for (name, c), v in rows.items() if c == counter and kernel in name]
+            return hits[0] if len(hits) == 1 else None
+        total = 0.0
+        for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+            copy = mean("stream_copy_f64_kernel", counter)
+            parts = [mean(k, counter) for k in PR_KERNELS]
+            if not copy or any(p is None for p in parts):
+                return None
+            total += sum(parts) * (1048576.0 / copy) * 1024.0
+        return total
+    except OSError:
+        return None
+
+
 def cpu_baselines(x_host, alpha, threads):
     """Oracle timings on the host cores: (a) fp64 pull over the same CSR, a bounded number of iterations;
     (b) the map-based float delta-push restatement of DRONE's Go 'pr' job on configs[0] (scale 16)."""
@@ -137,6 +170,26 @@ def bench_gcn_step(steps, warmup, cpu_baseline=False):
     loss1, acc1 = model.read_metrics()
     log(f"GCN step: {step_ms:.2f} ms (loss {loss0:.4f} -> {loss1:.4f}, train acc {acc1:.3f}); set-up (edge values, "
         f"transpose, plans) {setup_s*1e3:.0f} ms one-off")
+    model.close()
+    # the same step with layer 1 folded: A^T X aggregated once at creation, so the two 128-wide aggregations leave
+    # the step (the step then holds the K = 41 forward and backward products only)
+    t0 = time.time()
+    folded = gcn.GcnModel(g["rp"], g["ci"], g["deg"], g["deg"], X, label, split, W1, W2, dropout=0.5, lr=0.01,
+                          use_dropout=True, use_adam=False, mean_gradient=True, seed=4, fold_input_aggregation=True)
+    torch.cuda.synchronize()
+    folded_setup_s = time.time() - t0
+    folded.set_truth(1)
+    for _ in range(warmup):
+        folded.train_step_async()
+    floss0, _ = folded.read_metrics()
+    t.start()
+    for _ in range(steps):
+        folded.train_step_async()
+    folded_ms = t.stop_ms() / steps
+    floss1, facc1 = folded.read_metrics()
+    folded.close()
+    log(f"GCN step, layer 1 folded: {folded_ms:.2f} ms (loss {floss0:.4f} -> {floss1:.4f}); set-up incl. A^T X "
+        f"{folded_setup_s*1e3:.0f} ms one-off")
     # the four SpMMs of the step, timed alone on operands of the same shape
     rp, ci = g["rp"], g["ci"]
     val = gcn.edge_values(rp, ci, g["deg"], g["deg"])
@@ -163,29 +216,41 @@ def bench_gcn_step(steps, warmup, cpu_baseline=False):
     # CPU baseline: the oracle's CSR SpMM of identical semantics (OpenMP, all host cores) on the same matrix, K=128
     cpu = None
     if cpu_baseline:
-        from oracle import oracle as orc
-        orc.build()
-        h_rp, h_ci, h_val = rp.cpu().numpy(), ci.cpu().numpy(), val.cpu().numpy()
-        Bh = rmat.uniform_f32((N, HID), seed=7)
-        t0 = time.time()
-        orc.spmm_f32(h_rp, h_ci, h_val, Bh)
-        dt = time.time() - t0
-        threads = min(16, os.cpu_count() or 1)
-        cpu = {"value": dt * 1e3, "unit": "ms per SpMM (K=128)", "cores": threads, "kind": "port",
-               "sample": f"oracle fp32 CSR SpMM (OpenMP) on the same {nnz}-entry matrix, one product, {dt:.1f} s",
-               "gpu_ms": kernels[0]["ms"]}
-        log(f"cpu baseline SpMM K=128: {dt*1e3:.0f} ms on {threads} threads (GPU {kernels[0]['ms']:.2f} ms)")
+        cpu = cpu_spmm_baseline(rp, ci, val, N, HID, nnz)
+        cpu["gpu_ms"] = kernels[0]["ms"]
+        log(f"cpu baseline SpMM K=128: {cpu['value']:.0f} ms on {cpu['cores']} threads (GPU {kernels[0]['ms']:.2f} ms)")
     plan.close()
-    model.close()
     return {"cpu_baseline_spmm": cpu,
             "workload": f"2-layer GCN training step (configs[3]): N={N}, nnz={nnz}, 602->128->41, ReLU, dropout 0.5, "
                         "softmax cross-entropy, SGD lr 0.01, fp32",
-            "step_ms": step_ms, "steps": steps, "setup_ms_one_off": setup_s * 1e3, "spmm_kernels": kernels,
+            "step_ms": step_ms, "steps": steps, "setup_ms_one_off": setup_s * 1e3,
+            "step_contains": "SpMM K=128 forward, K=41 forward, K=41 backward, K=128 backward; 5 GEMMs; glue",
+            "folded_layer1": {"step_ms": folded_ms, "setup_ms_one_off": folded_setup_s * 1e3,
+                              "loss_first_last": [floss0, floss1],
+                              "step_contains": "SpMM K=41 forward, K=41 backward (A^T X aggregated once at creation: "
+                                               "fold_input_aggregation); 4 GEMMs; glue"},
+            "loss_first_last": [loss0, loss1], "spmm_kernels": kernels,
             "spmm_ms_per_step": spmm_ms, "spmm_plan": plan_info,
             "spmm_frac_of_hbm_peak": spmm_bytes / (spmm_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "gemms": gemms}
 
 
-def bench_gcn_layer():
+def cpu_spmm_baseline(rp, ci, val, N, K, nnz, seed=7):
+    """The oracle's fp32 CSR SpMM of identical semantics (OpenMP over rows, all host cores) on the same matrix, one
+    product of width K."""
+    from oracle import oracle as orc
+    from drone_amd import rmat
+    orc.build()
+    h_rp, h_ci, h_val = rp.cpu().numpy(), ci.cpu().numpy(), val.cpu().numpy()
+    Bh = rmat.uniform_f32((N, K), seed=seed)
+    t0 = time.time()
+    orc.spmm_f32(h_rp, h_ci, h_val, Bh)
+    dt = time.time() - t0
+    threads = min(16, os.cpu_count() or 1)
+    return {"value": dt * 1e3, "unit": f"ms per SpMM (K={K})", "cores": threads, "kind": "port",
+            "sample": f"oracle fp32 CSR SpMM (OpenMP) on the same {nnz}-entry matrix, one product, {dt:.2f} s"}
+
+
+def bench_gcn_layer(cpu_baseline=False):
     """configs[2]: one GCN layer forward ReLU(A_hat * (H * W)), R-MAT scale 20."""
     import torch
     from drone_amd import gcn, graphs, rmat
@@ -209,12 +274,18 @@ def bench_gcn_layer():
     ms_spmm = time_call(lambda: gcn.spmm(plan, g["rp"], g["ci"], val, T1, out=out), reps=10)
     ms_gemm = time_call(lambda: gcn.sgemm(0, 0, H, W, out=T1), reps=10)
     plan.close()
+    cpu = cpu_spmm_baseline(g["rp"], g["ci"], val, N, K, nnz) if cpu_baseline else None
+    if cpu:
+        cpu["gpu_ms"] = ms_spmm
+    log(f"GCN layer (configs[2]): {ms:.2f} ms, SpMM {ms_spmm:.2f} ms, GEMM {ms_gemm:.2f} ms" +
+        (f"; CPU SpMM {cpu['value']:.0f} ms on {cpu['cores']} threads" if cpu else ""))
     return {"workload": f"GCN layer forward (configs[2]): R-MAT scale 20 undirected + self-loops, N={N}, nnz={nnz}, K=128",
             "layer_ms": ms, "spmm": spmm_report("spmm (rows + band pieces + dense core) K=128", N, nnz, K, ms_spmm),
-            "gemm_ms": ms_gemm, "gemm_tflops": 2.0 * N * K * K / (ms_gemm * 1e-3) / 1e12}
+            "gemm_ms": ms_gemm, "gemm_tflops": 2.0 * N * K * K / (ms_gemm * 1e-3) / 1e12,
+            "gemm_frac_of_fp32_mfma_peak": 2.0 * N * K * K / (ms_gemm * 1e-3) / 1e12 / 157.3, "cpu_baseline_spmm": cpu}
 
 
-def bench_spmm_sweep():
+def bench_spmm_sweep(cpu_baseline=False):
     """configs[4]: skew-stress SpMM sweep, R-MAT scale 22 ef 32 a/b/c = .70/.12/.12, row-normalised, K in 16/64/256,
     forward (A*H) and transpose (A^T*G)."""
     import torch
@@ -236,6 +307,13 @@ def bench_spmm_sweep():
             ms = time_call(lambda: gcn.spmm(plan, a, b, c, H, out=C_), reps=5)
             plan.close()
             out["kernels"].append(spmm_report(f"{name} K={K}", N, nnz, K, ms))
+            log(f"SpMM sweep (configs[4]) {name} K={K}: {ms:.2f} ms = {out['kernels'][-1]['frac_of_hbm_peak']*100:.1f} % of "
+                f"the HBM roofline")
+        del H, C_
+    if cpu_baseline:
+        out["cpu_baseline_spmm"] = cpu_spmm_baseline(rp, ci, val, N, 64, nnz)
+        out["cpu_baseline_spmm"]["gpu_ms"] = [k["ms"] for k in out["kernels"] if k["K"] == 64][0]
+        log(f"cpu baseline SpMM K=64 forward: {out['cpu_baseline_spmm']['value']:.0f} ms")
     return out
 
 
@@ -412,8 +490,9 @@ def main():
                          "rocprofv3 byte counters by)")
     ap.add_argument("--suite", default="default", choices=["pr", "default", "full", "gcn", "sweep", "traverse", "exchange"],
                     help="pr: PageRank only (fp64 pull plan, then the reference's PR_PEVal / PR_IncEVal on the same "
-                         "graph); default: + GCN training step (configs[3]); full: + configs[2], [4] and the "
-                         "SSSP / CC jobs and the replica exchange; gcn, sweep, traverse, exchange: that part alone")
+                         "graph); default: + the GCN training step (configs[3]), the GCN layer (configs[2]) and the "
+                         "SpMM sweep (configs[4]); full: + the SSSP / CC jobs and the replica exchange; gcn, sweep, "
+                         "traverse, exchange: that part alone")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs one subgraph on ONE GPU; there is no multi-GPU path to time "
@@ -490,8 +569,10 @@ def main():
                      "frac": achieved / HBM_PEAK_GBS,
                      # fabric bytes per launch: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by the 1 GiB copy
                      # kernel; measured for this workload only (profiles/pr_rowblock_pagerank_c2.hbm_traffic.txt)
-                     "traffic": 3.48e9 if (args.scale == 24 and n == 16777216) else None,
-                     "kernel": "pr_rowblock_kernel<PrF64Epi> + pr_rowblock_merge_kernel<PrF64Epi> (one iteration)",
+                     "traffic": pr_traffic_from_profile() if (args.scale == 24 and n == 16777216) else None,
+                     "traffic_source": "profiles/pr_rowblock_pagerank_c2.hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / "
+                                       "WRITE_SIZE of this command, scaled by the 1 GiB copy kernel)",
+                     "kernel": "one iteration: " + " + ".join(PR_KERNELS) + " + row fix-up + dangling-mass reduction",
                      "algorithmic_bytes_per_launch": bytes_iter, "mean_launch_ms": prof["mean_ms"],
                      "launches_timed": prof["launches"]},
         "plan_ms_one_off": plan_s * 1e3,
@@ -519,11 +600,11 @@ def main():
         result["gcn_step"] = bench_gcn_step(steps=max(3, args.steps), warmup=max(1, args.warmup),
                                             cpu_baseline=not args.no_cpu_baseline)
         torch.cuda.empty_cache()
+        result["gcn_layer"] = bench_gcn_layer(cpu_baseline=not args.no_cpu_baseline)
+        torch.cuda.empty_cache()
+        result["spmm_sweep"] = bench_spmm_sweep(cpu_baseline=not args.no_cpu_baseline)
+        torch.cuda.empty_cache()
     if args.suite == "full":
-        result["gcn_layer"] = bench_gcn_layer()
-        torch.cuda.empty_cache()
-        result["spmm_sweep"] = bench_spmm_sweep()
-        torch.cuda.empty_cache()
         result["traverse"] = bench_traverse(cpu_baseline=not args.no_cpu_baseline)
         torch.cuda.empty_cache()
         result["exchange"] = bench_exchange()

@@ -274,12 +274,12 @@ extern "C" int drone_pr_run_f64(drone_pr_plan *p, double alpha, int iters, doubl
                     p->rb.split_block, p->rb.block_row, p->rb.block_units, p->rb.block_partial, p->rb.partial, epi, carry,
                     p->ms.tile_stat);
         }
-        if (prof) DRONE_HIP_TRY(hipEventRecord(p->ev1[p->prof_n++], s));
         spmv_fixup_kernel<double, PrF64Epi><<<fb, kSpmvBlock, 0, s>>>(
             p->units, p->deterministic ? p->mt.tile_row : p->rb.block_row,
             p->deterministic ? p->mt.walk_len : p->rb.walk_len, carry, p->ms.tile_stat, epi, p->ms.block_stat);
         // dang is read by the kernels above and overwritten here, in stream order
         reduce_stat_kernel<0><<<1, kSpmvBlock, 0, s>>>(p->ms.block_stat, fb, p->dang);
+        if (prof) DRONE_HIP_TRY(hipEventRecord(p->ev1[p->prof_n++], s));  // the whole iteration, small kernels included
     }
     DRONE_HIP_TRY(hipGetLastError());
     return DRONE_OK;

@@ -155,9 +155,10 @@ int drone_pr_plan_destroy(drone_pr_plan *plan);
  * Asynchronous on `stream`; allocates nothing. */
 int drone_pr_run_f64(drone_pr_plan *plan, double alpha, int iters, double *rank_out,
                      drone_stream_t stream);
-/* Per-kernel timing with HIP events on the launch stream.  When enabled, every launch of the
- * aggregation kernel inside drone_pr_run_f64 is bracketed by an event pair (at most `max_launches`
- * are kept).  drone_pr_profile_read synchronises the events and returns the mean duration. */
+/* Per-iteration timing with HIP events on the launch stream.  When enabled, every iteration inside
+ * drone_pr_run_f64 - the aggregation kernel, the merge of shared blocks, the row fix-up and the dangling-mass
+ * reduction, i.e. everything the algorithmic bytes of one iteration pay for - is bracketed by an event pair (at
+ * most `max_launches` are kept).  drone_pr_profile_read synchronises the events and returns the mean duration. */
 int drone_pr_profile_enable(drone_pr_plan *plan, int max_launches);
 int drone_pr_profile_read(drone_pr_plan *plan, int *launches, double *mean_ms, double *min_ms,
                           double *max_ms);
