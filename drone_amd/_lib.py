@@ -83,6 +83,7 @@ SIGNATURES = {
     "drone_last_error": (_I, []),
     "drone_last_error_string": (C.c_char_p, []),
     "drone_version": (C.c_char_p, []),
+    "drone_abi_sizes": (_I, [C.POINTER(_I), C.POINTER(C.c_size_t)]),
     "build_graph": (C.POINTER(Graph), [_I, _I, _P, _P, _I, _I, C.POINTER(Comm)]),
     "getLocalVertexSize": (_I, [C.POINTER(Graph)]),
     "getGlobalVertexSize": (_I, [C.POINTER(Graph)]),

@@ -43,6 +43,18 @@ extern "C" int drone_last_error(void) { return g_err_code; }
 extern "C" const char *drone_last_error_string(void) { return g_err_msg; }
 extern "C" const char *drone_version(void) { return "drone_hip 0.1 (gfx950)"; }
 
+// sizeof of the structs that cross the boundary by layout, in the order of the DRONE_ABI_* indices.
+extern "C" int drone_abi_sizes(int *count, size_t *sizes)
+{
+    const size_t all[DRONE_ABI_COUNT] = {sizeof(Graph), sizeof(Comm), sizeof(Response), sizeof(PRValues), sizeof(CCValues),
+                                         sizeof(SSSPValues)};
+    if (!count) return DRONE_ERR_INVALID;
+    if (sizes)
+        for (int i = 0; i < *count && i < DRONE_ABI_COUNT; ++i) sizes[i] = all[i];
+    *count = DRONE_ABI_COUNT;
+    return DRONE_OK;
+}
+
 extern "C" int drone_rmat_edges(int scale, int64_t n_edges, double a, double b, double c, uint64_t seed,
                                 int64_t first_edge, uint32_t *src, uint32_t *dst)
 {

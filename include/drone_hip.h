@@ -39,6 +39,17 @@ int drone_last_error(void);
 const char *drone_last_error_string(void);
 /* Library version and the code-object architecture it was built for ("gfx950"). */
 const char *drone_version(void);
+/* Sizes of the structs the caller allocates or reads by layout, as THIS library was compiled: sizes[DRONE_ABI_GRAPH]
+ * = sizeof(Graph), ... A worker allocates PRValues / CCValues / SSSPValues / Comm itself (PRWorkerCUDA.go:120-123)
+ * and the library writes every field, including the `ext` pointer these structs have beyond the reference's
+ * (DRONE/src/cuda/algorithm/pr.h:7-16 is 80 bytes, PRValues here 88): a worker compiled against the reference's
+ * headers would be overrun.  Compare at start-up (`*count` in: capacity of sizes, out: DRONE_ABI_COUNT), e.g. in Go:
+ *   func init() { if unsafe.Sizeof(CUDA_PRValues{}) != abiSize(C.DRONE_ABI_PRVALUES) { panic("stale drone header") } } */
+enum drone_abi_struct {
+    DRONE_ABI_GRAPH = 0, DRONE_ABI_COMM = 1, DRONE_ABI_RESPONSE = 2, DRONE_ABI_PRVALUES = 3, DRONE_ABI_CCVALUES = 4,
+    DRONE_ABI_SSSPVALUES = 5, DRONE_ABI_COUNT = 6
+};
+int drone_abi_sizes(int *count, size_t *sizes);
 
 /* ====================================================================================== */
 /* A. DRONE worker boundary (replaces DRONE/src/cuda/{graph.cu,algorithm/pr.cu,common.cu}) */

@@ -55,6 +55,49 @@ def test_struct_layouts_match_reference():
     assert _lib.SSSPValues.distance.offset == 32 and _lib.SSSPValues.ext.offset == 40
 
 
+ABI_STRUCTS = [("Graph", _lib.Graph), ("Comm", _lib.Comm), ("Response", _lib.Response), ("PRValues", _lib.PRValues),
+               ("CCValues", _lib.CCValues), ("SSSPValues", _lib.SSSPValues)]
+
+
+def test_header_layouts_compiled_by_a_c_compiler(tmp_path):
+    """The layouts a C (or cgo) caller gets from include/drone_hip.h, taken from the header itself: a C program that
+    includes it prints sizeof and every field's offsetof; they must equal the ctypes mirrors the tests call through,
+    the sizes the library was compiled with (drone_abi_sizes), and - for the leading fields - the reference's layouts
+    (pr.h:7-16 is ten pointers = 80 bytes; cc.h / sssp.h:17-25 five pointers; graph.h:16-38 ends with GID)."""
+    import shutil
+    import subprocess
+    cc = shutil.which("gcc") or shutil.which("cc")
+    assert cc, "no C compiler"
+    lines = ["#include <stddef.h>", "#include <stdio.h>", '#include "drone_hip.h"',
+             '_Static_assert(sizeof(Response) == 32, "Response is 6 int + 2 float, returned by value");',
+             '_Static_assert(sizeof(Comm) == 2 * sizeof(void *), "Comm is two pointers");',
+             '_Static_assert(offsetof(PRValues, ext) == 10 * sizeof(void *), "ext follows the reference\'s ten pointers");',
+             '_Static_assert(offsetof(CCValues, ext) == 5 * sizeof(void *) && offsetof(SSSPValues, ext) == 5 * sizeof(void *), "ext");',
+             '_Static_assert(offsetof(Graph, ext) >= offsetof(Graph, GID) + sizeof(int), "ext follows GID");',
+             "int main(void) {"]
+    for name, cls in ABI_STRUCTS:
+        lines.append(f'    printf("{name} size %zu\\n", sizeof({name}));')
+        for field, _ in cls._fields_:
+            lines.append(f'    printf("{name} {field} %zu\\n", offsetof({name}, {field}));')
+    lines += ["    return 0;", "}"]
+    src = tmp_path / "abi.c"
+    src.write_text("\n".join(lines) + "\n")
+    exe = tmp_path / "abi"
+    subprocess.check_call([cc, "-std=c11", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
+    got = {}
+    for line in subprocess.check_output([str(exe)], text=True).splitlines():
+        name, field, value = line.split()
+        got[(name, field)] = int(value)
+    count = C.c_int(16)
+    sizes = (C.c_size_t * 16)()
+    assert _lib.lib().drone_abi_sizes(C.byref(count), sizes) == 0 and count.value == len(ABI_STRUCTS)
+    for i, (name, cls) in enumerate(ABI_STRUCTS):
+        assert got[(name, "size")] == C.sizeof(cls) == sizes[i], name
+        for field, _ in cls._fields_:
+            assert got[(name, field)] == getattr(cls, field).offset, (name, field)
+    assert got[("PRValues", "size")] == 88 and got[("CCValues", "size")] == got[("SSSPValues", "size")] == 48
+
+
 def test_version_and_error_channel():
     L = _lib.lib()
     assert b"gfx950" in L.drone_version()
