@@ -103,6 +103,7 @@ SIGNATURES = {
     "drone_pr_profile_read": (_I, [_P, C.POINTER(_I), C.POINTER(_D), C.POINTER(_D), C.POINTER(_D)]),
     "drone_pr_bytes_per_iteration": (_I64, [_I64, _I64]),
     "drone_pr_run_graph_f64": (_I, [C.POINTER(Graph), C.POINTER(PRValues), _D, _I, _P]),
+    "drone_pr_run_workers_f64": (_I, [C.POINTER(Graph), C.POINTER(PRValues), _I, _I, C.POINTER(Comm), _D, _I, _P]),
     "drone_gcn_edge_values": (_I, [_I, _P, _P, _P, _P, _P, _P]),
     "drone_csr_transpose_f32": (_I, [_I, _I, _I64, _P, _P, _P, _P, _P, _P, _P]),
     "drone_spmm_plan_create": (_I, [C.POINTER(_P), _I, _I, _I64, _P, _P, _P, _I, _P]),

@@ -468,7 +468,7 @@ extern "C" int drone_pr_run_graph_f64(Graph *g, PRValues *values, double alpha, 
     GraphExt *x = static_cast<GraphExt *>(g->ext);
     DRONE_REQUIRE(x->n > 0, "empty graph");
     DRONE_REQUIRE(g->MirrorSize == 0 && g->MirrorWorkerSize == 0,
-                  "the fp64 pull run covers one whole subgraph: this graph has replicated vertices");
+                  "this graph has replicated vertices: use drone_pr_run_workers_f64, which exchanges them");
     if (!x->plan64) {
         DRONE_HIP_TRY(hipMalloc(&x->row_ptr64, sizeof(int64_t) * ((size_t)x->n + 1)));
         DRONE_HIP_TRY(hipMalloc(&x->inv64, sizeof(double) * (size_t)x->n));

@@ -333,6 +333,8 @@ extern "C" int drone_pr_worker_run_f64(drone_pr_worker *w, double alpha, int ite
 {
     clear_error();
     DRONE_REQUIRE(w != nullptr, "worker");
+    if (w->worker_num > 1)
+        return drone_pr_run_workers_f64(w->g, &w->values, w->self_id - 1, w->worker_num, &w->comm, alpha, iters, rank_out);
     return drone_pr_run_graph_f64(w->g, &w->values, alpha, iters, rank_out);
 }
 

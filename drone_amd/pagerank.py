@@ -160,9 +160,15 @@ class PRWorkerCUDA:
                     index=self._i32(g.index, self.n + 1), dst=self._i32(g.dst, E))
 
     def run_f64(self, alpha, iters):
+        """Normalised fp64 ranks after `iters` fixed iterations, local vertex order.  With several workers every
+        worker calls this from its own thread (drone_pr_run_workers_f64 exchanges the replicated vertices)."""
         out = np.empty(self.n, np.float64)
-        check(lib().drone_pr_run_graph_f64(self.g, C.byref(self.values), float(alpha), int(iters),
-                                           out.ctypes.data_as(C.c_void_p)))
+        if self.workerNum > 1:
+            check(lib().drone_pr_run_workers_f64(self.g, C.byref(self.values), self.id, self.workerNum, C.byref(self.comm),
+                                                 float(alpha), int(iters), out.ctypes.data_as(C.c_void_p)))
+        else:
+            check(lib().drone_pr_run_graph_f64(self.g, C.byref(self.values), float(alpha), int(iters),
+                                               out.ctypes.data_as(C.c_void_p)))
         return out
 
     def aggregation(self):

@@ -179,6 +179,15 @@ int64_t drone_pr_bytes_per_iteration(int64_t n, int64_t nnz);
 /* Same iteration driven from a Graph built by build_graph + loadOutDegree (local out-degrees are
  * taken from PRValues.outDegree).  rank_out: host [localVertexSize], normalised ranks. */
 int drone_pr_run_graph_f64(Graph *g, PRValues *values, double alpha, int iters, double *rank_out);
+/* The same fixed-iteration fp64 PageRank over the subgraphs of a vertex cut, one call per worker (each from its own
+ * thread; they meet on the wire): per iteration the partial row sums of a replicated vertex are added at its master
+ * and assigned back to its mirrors, and the dangling mass is summed over the workers - the two exchange phases and
+ * the all-reduce of DRONE/src/cuda/algorithm/pr.cu:215-373, in double.  N = the distinct vertices of all subgraphs,
+ * PRValues.outDegree holds GLOBAL out-degrees (loadOutDegree).  Every replica of a vertex ends with the same value,
+ * equal to the single-subgraph run of the whole graph up to summation order.  rank_out: host [localVertexSize].
+ * Runs on comm->s; with workerNum == 1 no transport is needed. */
+int drone_pr_run_workers_f64(Graph *g, PRValues *values, int workerId, int workerNum, Comm *comm, double alpha,
+                             int iters, double *rank_out);
 
 /* ====================================================================================== */
 /* C. GCN layer kernels (replace the vendor calls and glue kernels of cuda_gcn's modules)   */

@@ -151,8 +151,14 @@ def test_workers_from_files_with_replicas_match_oracle_group(tmp_path, oracle):
             ids, pr = w.read()
             np.testing.assert_array_equal(ids, tops[i].l2g)
             np.testing.assert_allclose(pr, states[i].pr, rtol=2e-5)
-            with pytest.raises(_lib.DroneError, match="replicated"):
-                w.run_f64(0.85, 2)
+        # the fp64 pull run exchanges the replicated vertices too: all replicas of a vertex agree, ranks sum to 1
+        ranks = run_workers([(lambda w=w: w.run_f64(0.85, 10)) for w in ws])
+        glob = np.full(gN, -1.0)
+        for t, r in zip(tops, ranks):
+            seen = glob[t.l2g] >= 0
+            np.testing.assert_array_equal(glob[t.l2g][seen], r[seen])
+            glob[t.l2g] = r
+        assert abs(glob[glob >= 0].sum() - 1.0) < 1e-12
     finally:
         for w in ws:
             w.close()
