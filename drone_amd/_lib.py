@@ -93,6 +93,7 @@ SIGNATURES = {
     "PR_PEVal": (Response, [C.POINTER(Graph), C.POINTER(PRValues), _I, _I, C.POINTER(Comm)]),
     "PR_IncEVal": (Response, [C.POINTER(Graph), C.POINTER(PRValues), _I, _I, C.POINTER(Comm)]),
     "drone_graph_destroy": (None, [C.POINTER(Graph)]),
+    "drone_check_routes": (_I, [C.POINTER(Graph), _P, _P, _I, _I, _P, _I]),
     "drone_pr_aggregation": (C.c_int, [C.POINTER(Graph)]),
     "drone_pr_values_destroy": (None, [C.POINTER(Graph), C.POINTER(PRValues)]),
     "drone_pr_plan_create": (_I, [C.POINTER(_P), _I64, _I64, _P, _P, _P, _P]),

@@ -241,12 +241,61 @@ extern "C" Graph *build_graph(int globalVertexSize, int edgeSize, int *u, int *v
 extern "C" int getLocalVertexSize(Graph *g) { return *g->localVertexSize; }
 extern "C" int getGlobalVertexSize(Graph *g) { return *g->globalVertexSize; }
 
+// What Master.<i> / Mirror.<i> may hold for this graph: every listed vertex is a global id that is local here,
+// mirror counts are not negative and add up to the length of the worker list.  (The reference indexes with whatever
+// the files say, graph.cu:272-290, :301-309.)
+extern "C" int drone_check_routes(Graph *g, const int *masterVertex, const int *mirrorNumber, int masterSize,
+                                  int mirrorWorkerSize, const int *mirrorVertex, int mirrorSize)
+{
+    clear_error();
+    DRONE_REQUIRE(g && g->ext, "graph");
+    DRONE_REQUIRE(masterSize >= 0 && mirrorWorkerSize >= 0 && mirrorSize >= 0, "negative count");
+    DRONE_REQUIRE((masterSize == 0 || (masterVertex && mirrorNumber)) && (mirrorSize == 0 || mirrorVertex), "null list");
+    DRONE_HIP_TRY(hipSetDevice(g->GID));
+    const int nglobal = *g->globalVertexSize;
+    std::vector<int> g2l((size_t)nglobal);
+    if (nglobal > 0) DRONE_HIP_TRY(hipMemcpy(g2l.data(), g->Global2Local, sizeof(int) * g2l.size(), hipMemcpyDeviceToHost));
+    auto local = [&](int v) { return v >= 0 && v < nglobal && g2l[(size_t)v] >= 0; };
+    long long listed = 0;
+    for (int i = 0; i < masterSize; ++i) {
+        if (!local(masterVertex[i])) {
+            set_error(DRONE_ERR_INVALID, "master route %d: vertex %d is not a vertex of this subgraph", i, masterVertex[i]);
+            return DRONE_ERR_INVALID;
+        }
+        if (mirrorNumber[i] < 0) {
+            set_error(DRONE_ERR_INVALID, "master route %d: vertex %d has a negative mirror count", i, masterVertex[i]);
+            return DRONE_ERR_INVALID;
+        }
+        listed += mirrorNumber[i];
+    }
+    if (listed != mirrorWorkerSize) {
+        set_error(DRONE_ERR_INVALID, "master routes list %lld mirror workers, mirrorWorkerSize is %d", listed, mirrorWorkerSize);
+        return DRONE_ERR_INVALID;
+    }
+    for (int i = 0; i < mirrorSize; ++i)
+        if (!local(mirrorVertex[i])) {
+            set_error(DRONE_ERR_INVALID, "mirror route %d: vertex %d is not a vertex of this subgraph", i, mirrorVertex[i]);
+            return DRONE_ERR_INVALID;
+        }
+    return DRONE_OK;
+}
+
+namespace {
+void die_on_bad_routes(int rc, const char *who)
+{
+    if (rc == DRONE_OK) return;
+    printf("Failed: %s: %s\n", who, drone_last_error_string());
+    exit(EXIT_FAILURE);
+}
+}  // namespace
+
 // graph.cu:260-299.  MasterWorkerIndex[l+1]-MasterWorkerIndex[l] = number of mirror workers of master l;
 // Master2Workers lists them.  Built on the host (the tables are tiny next to the edge arrays).
 extern "C" void addMasterRoute(Graph *g, int *masterVertex, int *mirrorNumber, int *mirrorWorkers,
                                int masterSize, int mirrorWorkerSize)
 {
-    clear_error();
+    die_on_bad_routes(drone_check_routes(g, masterVertex, mirrorNumber, masterSize, mirrorWorkerSize, nullptr, 0),
+                      "addMasterRoute");
     DRONE_HIP_OR_DIE(hipSetDevice(g->GID));
     const int n = getLocalVertexSize(g);
     g->MasterSize = masterSize;
@@ -273,7 +322,7 @@ extern "C" void addMasterRoute(Graph *g, int *masterVertex, int *mirrorNumber, i
 // graph.cu:311-331
 extern "C" void addMirrorRoute(Graph *g, int *mirrorVertex, int *masterWorker, int mirrorSize)
 {
-    clear_error();
+    die_on_bad_routes(drone_check_routes(g, nullptr, nullptr, 0, 0, mirrorVertex, mirrorSize), "addMirrorRoute");
     DRONE_HIP_OR_DIE(hipSetDevice(g->GID));
     g->MirrorSize = mirrorSize;
     static_cast<GraphExt *>(g->ext)->routes.ready = false;

@@ -277,6 +277,22 @@ extern "C" int drone_pr_worker_create(drone_pr_worker **out, const char *data_pa
     w->self_id = self_id;
     w->worker_num = worker_num;
     w->g = build_graph(global_vertex_size, edges, u, v, self_id - 1, worker_num, &w->comm);
+    rc = drone_check_routes(w->g, mv, mn, masters, mirror_workers, rv, mirrors);  // a bad file fails here, not in the tables
+    for (int i = 0; rc == DRONE_OK && i < mirror_workers + mirrors; ++i) {
+        const int peer = i < mirror_workers ? mw[i] : rw[i - mirror_workers];
+        if (peer < 0 || peer >= worker_num || peer == self_id - 1) {
+            set_error(DRONE_ERR_INVALID, "%s.%s names worker %d (this is worker %d of %d)", i < mirror_workers ? "Master" : "Mirror",
+                      id.c_str(), peer, self_id - 1, worker_num);
+            rc = DRONE_ERR_INVALID;
+        }
+    }
+    if (rc != DRONE_OK) {
+        if (w->comm.s) (void)hipStreamDestroy(static_cast<hipStream_t>(w->comm.s));
+        drone_graph_destroy(w->g);
+        delete w;
+        cleanup();
+        return rc;
+    }
     addMasterRoute(w->g, mv, mn, mw, masters, mirror_workers);
     addMirrorRoute(w->g, rv, rw, mirrors);
     loadOutDegree(w->g, &w->values, deg);

@@ -8,8 +8,12 @@
 // Here a dense round is one sweep of the merge-path aggregation over the IN-edge CSR with min as the combining
 // operator: value[v] <- min(value[v], min over in-edges u->v of f(value[u])), f = identity for labels and
 // + edge length for distances.  No atomics, hub rows are spread over tiles, and the sweep updates in place,
-// so a change can travel several hops in one sweep.  Both iterations descend monotonically to the same least
-// fixed point below the starting state, so the values are identical to the reference's; g->active keeps the
+// so a change can travel several hops in one sweep.  Both iterations descend monotonically towards the least
+// fixed point below the starting state.  Labels, and distances over unit or integer lengths, are identical to the
+// reference's.  With real-valued lengths the reference can stop short of the fixed point: it stores every lower
+// distance but re-activates a vertex only when the improvement exceeds 1e-6 (sssp.cu:62-68), so an improvement
+// below that is not carried on; the sweeps here carry every improvement on and end at the exact fixed point, at
+// most 1e-6 per hop below the reference's value.  g->active keeps the
 // reference's three classes (> 0 lowered by propagation in this call, 0 activated by a message or initial,
 // -1 untouched), which is all the exchange and countActive (common.cu:17-31) look at.  The round number
 // stored in g->active by the reference depends on its thread schedule and is not reproduced.

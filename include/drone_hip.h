@@ -402,6 +402,12 @@ void drone_free_host(void *p);
 typedef struct drone_pr_worker drone_pr_worker;
 int drone_pr_worker_create(drone_pr_worker **w, const char *data_path, int self_id, int worker_num,
                            int global_vertex_size);
+/* Whether routing lists (the contents of Master.<i> / Mirror.<i>) fit a built graph: every listed vertex is a global
+ * id that is local to `g`, mirror counts are not negative and add up to mirrorWorkerSize.  addMasterRoute /
+ * addMirrorRoute run the same check and print + exit on failure (they have no status to return);
+ * drone_pr_worker_create returns the error.  Either list may be empty. */
+int drone_check_routes(Graph *g, const int *masterVertex, const int *mirrorNumber, int masterSize, int mirrorWorkerSize,
+                       const int *mirrorVertex, int mirrorSize);
 struct drone_loopback;
 int drone_pr_worker_attach_loopback(drone_pr_worker *w, struct drone_loopback *group); /* section F */
 Response drone_pr_worker_peval(drone_pr_worker *w);
@@ -468,8 +474,10 @@ typedef struct SSSPValues {
     void *ext;
 } SSSPValues;
 /* sssp.cu:398-539.  Relaxation over g->edgeLen (1.0 after build_graph) from global vertex startId to the local
- * fixed point, then the exchange.  A relaxation counts as an update when it lowers the distance by more than
- * 1e-6 (sssp.cu:64). */
+ * fixed point, then the exchange.  A relaxation counts as an update (Response.VisitedSize, the exchange's flags)
+ * when it lowers the distance by more than 1e-6 (sssp.cu:64).  Distances over unit or integer lengths equal the
+ * reference's; with real-valued lengths the reference does not carry improvements below 1e-6 on to the next hop,
+ * this library does, so its distances are the exact shortest ones, at most 1e-6 per hop below the reference's. */
 Response SSSP_PEVal(Graph *g, SSSPValues *values, int startId, int workerId, int workerNum, Comm *comm);
 Response SSSP_IncEVal(Graph *g, SSSPValues *values, int workerId, int workerNum, Comm *comm);
 void drone_sssp_values_destroy(Graph *g, SSSPValues *values);

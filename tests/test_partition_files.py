@@ -80,6 +80,23 @@ def test_worker_create_rejects_bad_partitions(tmp_path):
 
 
 @pytest.mark.gpu
+def test_worker_create_rejects_bad_routes(tmp_path):
+    """Routing files that name a vertex the subgraph does not hold, a worker outside the group or the worker itself
+    are refused with an error before they index anything (the graph has vertices 0, 1, 2 of 6 global ids)."""
+    for master, mirror, what in ((b"4 1\n", b"", "not a vertex of this subgraph"),     # vertex 4 has no edge here
+                                 (b"9 1\n", b"", "not a vertex of this subgraph"),     # beyond the global ids
+                                 (b"", b"5 1\n", "not a vertex of this subgraph"),
+                                 (b"1 7\n", b"", "names worker 7"),
+                                 (b"", b"2 0\n", "names worker 0")):                   # worker 0 is this worker
+        write_partition(tmp_path, [0, 1], [1, 2], [1, 1, 0, 0, 0, 0], master=master, mirror=mirror)
+        with pytest.raises(_lib.DroneError, match=what):
+            pf.PRWorkerFromFiles(tmp_path, 6, self_id=1, worker_num=2)
+    write_partition(tmp_path, [0, 1], [1, 2], [1, 1, 0, 0, 0, 0], master=b"1 1\n", mirror=b"2 1\n")
+    w = pf.PRWorkerFromFiles(tmp_path, 6, self_id=1, worker_num=2)                     # a consistent pair is accepted
+    w.close()
+
+
+@pytest.mark.gpu
 def test_worker_from_files_matches_oracle(tmp_path, oracle):
     from drone_amd import rmat
     s, d = rmat.rmat_edges(11, 2048 * 8, seed=6)

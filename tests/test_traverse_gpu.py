@@ -111,6 +111,41 @@ def test_sssp_edge_lengths(oracle):
         w.close()
 
 
+def test_sssp_real_valued_edge_lengths(oracle):
+    """Lengths that are not integers: the reference stores every lower distance but only re-activates a vertex when
+    the improvement exceeds 1e-6 (sssp.cu:62-68), so along a path its result can stay above the true shortest
+    distance by up to 1e-6 per hop, depending on the order of its atomics; the pull sweeps here propagate every
+    improvement and reach the exact fixed point.  Stated tolerance: never above the oracle's serial restatement of the
+    reference by more than float rounding, never below it by more than 1e-6 per hop of the path (32 hops bound this
+    graph's diameter), and equal to scipy's shortest paths to float rounding."""
+    import scipy.sparse as sp
+    from scipy.sparse.csgraph import shortest_path
+    from drone_amd.traverse import SSSPWorkerCUDA
+    u, v = _rmat(11, 8, 7)
+    nglobal = 1 << 11
+    n, g2l, l2g, index, dst = oracle.build_graph(nglobal, u, v)
+    rng = np.random.default_rng(3)
+    length = (rng.random(len(dst)) * 2 + 1e-3).astype(np.float32)
+    length[rng.random(len(dst)) < 0.2] += np.float32(3e-7)            # near-ties below the reference's tolerance
+    start = int(g2l[u[0]])
+    st = oracle.SSSPState(index, dst, length)
+    st.peval(start)
+    w = SSSPWorkerCUDA(nglobal, u, v, startId=int(u[0]))
+    try:
+        w.set_edge_len(length)
+        w.peval()
+        got = w.read()
+    finally:
+        w.close()
+    src = np.repeat(np.arange(n), np.diff(index))
+    A = sp.csr_matrix((length.astype(np.float64), (src, dst)), shape=(n, n))
+    exact = shortest_path(A, method="D", directed=True, indices=start)
+    reached = np.isfinite(exact)
+    np.testing.assert_array_equal(got[~reached], np.float32(1e8))
+    np.testing.assert_allclose(got[reached], exact[reached], rtol=2e-6, atol=0)
+    assert np.all(got <= st.val * (1 + 1e-6)) and np.all(got[reached] >= st.val[reached] - 32e-6)
+
+
 def _group(oracle, kind, nglobal, parts):
     states, tops = [], []
     for p in parts:
