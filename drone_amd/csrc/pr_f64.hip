@@ -63,6 +63,44 @@ __global__ __launch_bounds__(kSpmvBlock) void pr_f64_init_kernel(int64_t n, cons
     if (threadIdx.x == 0) block_stat[blockIdx.x] = total;
 }
 
+// Isolated vertices (rows [live, n) of the plan's order: no entries, gathered by nobody) take no part in the sweep.
+// Their rank is the iteration's constant term, base_k = (1 - alpha) / N + alpha * dang_{k-1} / N; what they add to
+// the dangling mass is base_k times the number of them that are dangling, counted once per run:
+// count[0] = number of i in [live, n) with inv[i] == 0.
+__global__ __launch_bounds__(kSpmvBlock) void pr_f64_count_idle_dangling_kernel(int64_t live, int64_t n,
+                                                                                const double *__restrict__ inv,
+                                                                                double *__restrict__ block_count)
+{
+    __shared__ double s_red[kSpmvBlock / kWave];
+    double c = 0.0;
+    for (int64_t i = live + (int64_t)blockIdx.x * kSpmvBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kSpmvBlock)
+        c += inv[i] == 0.0 ? 1.0 : 0.0;
+    const double total = block_sum_256(c, s_red);
+    if (threadIdx.x == 0) block_count[blockIdx.x] = total;  // summed by reduce_stat_kernel
+}
+
+// dang[0] = sum of the blocks' statistics + idle[0] * base_k (dang[0] still holds dang_{k-1} when this runs).
+__global__ __launch_bounds__(kSpmvBlock) void pr_f64_reduce_dangling_kernel(const double *__restrict__ in, int count,
+                                                                            const double *__restrict__ idle, double alpha,
+                                                                            double inv_n, double *__restrict__ dang)
+{
+    __shared__ double s_red[kSpmvBlock / kWave];
+    double v = 0.0;
+    for (int k = threadIdx.x; k < count; k += kSpmvBlock) v += in[k];
+    const double total = block_sum_256(v, s_red);
+    if (threadIdx.x == 0) dang[0] = total + idle[0] * ((1.0 - alpha) * inv_n + alpha * dang[0] * inv_n);
+}
+
+// Last iteration: the isolated vertices' ranks, r_out[order[i]] = base_k for i in [live, n).
+__global__ void pr_f64_idle_ranks_kernel(int64_t live, int64_t n, const int32_t *__restrict__ order,
+                                         const double *__restrict__ dang, double alpha, double inv_n,
+                                         double *__restrict__ r_out)
+{
+    const double base = (1.0 - alpha) * inv_n + alpha * dang[0] * inv_n;
+    for (int64_t i = live + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        r_out[order[i]] = base;
+}
+
 __global__ void pr_f64_uniform_kernel(int64_t n, double inv_n, double *__restrict__ r)
 {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
@@ -86,6 +124,8 @@ struct drone_pr_plan {
     MergeScratch ms;
     double *c[2] = {nullptr, nullptr};
     double *dang = nullptr;  // device scalar
+    int64_t rows = 0;        // rows the aggregation sweeps: n, or without the isolated vertices at the end of the order
+    double *idle = nullptr;  // device scalar: dangling vertices among the rows left out, counted at every run
     int init_blocks = 0;
     // profiling
     int prof_cap = 0, prof_n = 0;
@@ -121,12 +161,16 @@ extern "C" int drone_pr_plan_create_ex(drone_pr_plan **out, int64_t n, int64_t n
         DRONE_HIP_TRY(hipGetDevice(&p->device));
         int rc = relabel_create(&p->rl, n, nnz, row_ptr, col_idx, inv_outdeg, s);
         if (rc != DRONE_OK) return rc;
+        p->rows = n;
         if (p->deterministic) {
             rc = merge_tiling_create<int64_t>(&p->mt, n, nnz, p->rl.row_ptr, kSpmvBlock * kPrIpt, s);
             if (rc != DRONE_OK) return rc;
             p->units = p->mt.num_tiles;
         } else {
-            rc = row_blocks_create(&p->rb, n, nnz, p->rl.row_ptr, p->rl.col,
+            // R-MAT scale 24: 7.9 M of 16.8 M vertices are isolated; left out, an iteration moves 126 MB less and
+            // loses some 480 work-groups that had next to no entries
+            p->rows = p->rl.live > 0 ? p->rl.live : 1;
+            rc = row_blocks_create(&p->rb, p->rows, nnz, p->rl.row_ptr, p->rl.col,
                                    (flags & DRONE_PR_SHARED_BLOCKS) ? 2 : (flags & DRONE_PR_WHOLE_BLOCKS) ? 1 : 0, s);
             if (rc != DRONE_OK) return rc;
             p->units = p->rb.num_blocks;
@@ -145,6 +189,7 @@ extern "C" int drone_pr_plan_create_ex(drone_pr_plan **out, int64_t n, int64_t n
         DRONE_HIP_TRY(hipMalloc(&p->c[0], sizeof(double) * (size_t)n));
         DRONE_HIP_TRY(hipMalloc(&p->c[1], sizeof(double) * (size_t)n));
         DRONE_HIP_TRY(hipMalloc(&p->dang, sizeof(double)));
+        DRONE_HIP_TRY(hipMalloc(&p->idle, sizeof(double)));
         DRONE_HIP_TRY(hipMalloc(&p->inv, sizeof(double) * (size_t)n));
         DRONE_HIP_TRY(hipStreamSynchronize(s));
         return DRONE_OK;
@@ -174,6 +219,7 @@ extern "C" int drone_pr_plan_destroy(drone_pr_plan *p)
     if (p->c[0]) (void)hipFree(p->c[0]);
     if (p->c[1]) (void)hipFree(p->c[1]);
     if (p->dang) (void)hipFree(p->dang);
+    if (p->idle) (void)hipFree(p->idle);
     for (int i = 0; i < p->prof_cap; ++i) {
         (void)hipEventDestroy(p->ev0[i]);
         (void)hipEventDestroy(p->ev1[i]);
@@ -247,6 +293,9 @@ extern "C" int drone_pr_run_f64(drone_pr_plan *p, double alpha, int iters, doubl
     { int rc = relabel_gather_f64(p->rl, p->inv_user, p->inv, s); if (rc != DRONE_OK) return rc; }
     pr_f64_init_kernel<<<p->init_blocks, kSpmvBlock, 0, s>>>(p->n, p->inv, inv_n, p->c[0], p->ms.block_stat);
     reduce_stat_kernel<0><<<1, kSpmvBlock, 0, s>>>(p->ms.block_stat, p->init_blocks, p->dang);
+    // (the partial counts reuse the statistics array, which the reduction above has just consumed)
+    pr_f64_count_idle_dangling_kernel<<<p->init_blocks, kSpmvBlock, 0, s>>>(p->rows, p->n, p->inv, p->ms.block_stat);
+    reduce_stat_kernel<0><<<1, kSpmvBlock, 0, s>>>(p->ms.block_stat, p->init_blocks, p->idle);
     for (int it = 0; it < iters; ++it) {
         PrF64Epi epi;
         epi.c_in = p->c[it & 1];
@@ -263,7 +312,7 @@ extern "C" int drone_pr_run_f64(drone_pr_plan *p, double alpha, int iters, doubl
         if (prof) DRONE_HIP_TRY(hipEventRecord(p->ev0[p->prof_n], s));
         if (p->deterministic) {
             spmv_merge_kernel<double, int64_t, kPrIpt, PrF64Epi><<<p->mt.num_tiles, kSpmvBlock, 0, s>>>(
-                p->n, p->nnz, p->mt.tile_row, p->rl.row_ptr, p->rl.col, epi, carry, p->ms.tile_stat);
+                p->rows, p->nnz, p->mt.tile_row, p->rl.row_ptr, p->rl.col, epi, carry, p->ms.tile_stat);
         } else {
             pr_rowblock_kernel<PrF64Epi><<<p->rb.num_units, kRbThreads, kRbLdsBytes, s>>>(
                 p->rb.block_row, p->rb.block_nnz, p->rb.col, p->rb.lrow, p->rb.packed, p->rb.batch_base, p->rb.block_batch,
@@ -277,8 +326,10 @@ extern "C" int drone_pr_run_f64(drone_pr_plan *p, double alpha, int iters, doubl
         spmv_fixup_kernel<double, PrF64Epi><<<fb, kSpmvBlock, 0, s>>>(
             p->units, p->deterministic ? p->mt.tile_row : p->rb.block_row,
             p->deterministic ? p->mt.walk_len : p->rb.walk_len, carry, p->ms.tile_stat, epi, p->ms.block_stat);
+        if (epi.r_out && p->rows < p->n)
+            pr_f64_idle_ranks_kernel<<<1024, 256, 0, s>>>(p->rows, p->n, p->rl.order, p->dang, alpha, inv_n, rank_out);
         // dang is read by the kernels above and overwritten here, in stream order
-        reduce_stat_kernel<0><<<1, kSpmvBlock, 0, s>>>(p->ms.block_stat, fb, p->dang);
+        pr_f64_reduce_dangling_kernel<<<1, kSpmvBlock, 0, s>>>(p->ms.block_stat, fb, p->idle, alpha, inv_n, p->dang);
         if (prof) DRONE_HIP_TRY(hipEventRecord(p->ev1[p->prof_n++], s));  // the whole iteration, small kernels included
     }
     DRONE_HIP_TRY(hipGetLastError());

@@ -12,6 +12,10 @@ namespace drone {
 
 struct Relabel {
     int64_t n = 0, nnz = 0;
+    // Vertices that are never gathered sort last, those of them that have no entries of their own (isolated: nothing
+    // to sum, nobody reads them) last of all: rows [live, n) are isolated.  live = n when the counts the order was made
+    // from turn out not to match the matrix (a vertex they call unused is gathered after all), or with keep_rows.
+    int64_t live = 0;
     int32_t *order = nullptr;    // device [n]: new id -> old id
     int64_t *row_ptr = nullptr;  // device [n+1]: relabelled CSR offsets
     int32_t *col = nullptr;      // device [nnz]: relabelled sources, row order kept

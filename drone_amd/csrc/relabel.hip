@@ -35,6 +35,23 @@ __global__ void count_from_offsets_kernel(const int *__restrict__ offsets, int64
         count[i] = (unsigned)(offsets[i + 1] - offsets[i]);
 }
 
+// Sort key (descending): gathered vertices by count, then the never-gathered ones that have entries of their own,
+// then the isolated ones.  live[0] += vertices that are not isolated.
+__global__ void order_keys_kernel(const int64_t *__restrict__ row_ptr, int64_t n, unsigned *__restrict__ count,
+                                  unsigned long long *__restrict__ live)
+{
+    unsigned long long mine = 0;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        const unsigned c = count[i];
+        const bool has_rows = row_ptr[i + 1] > row_ptr[i];
+        count[i] = c > 0 ? (c < 0xFFFFFFFEu ? c + 1 : 0xFFFFFFFFu) : has_rows ? 1u : 0u;
+        mine += (c > 0 || has_rows) ? 1 : 0;
+    }
+#pragma unroll
+    for (int m = kWave / 2; m > 0; m >>= 1) mine += __shfl_xor(mine, m, kWave);
+    if ((threadIdx.x & (kWave - 1)) == 0 && mine) atomicAdd(live, mine);
+}
+
 __global__ void iota_kernel(int32_t *a, int64_t n)
 {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
@@ -74,7 +91,8 @@ __global__ __launch_bounds__(256) void remap_rows_kernel(const int32_t *__restri
                                                          const int32_t *__restrict__ col,
                                                          const int32_t *__restrict__ new_id,
                                                          const int64_t *__restrict__ new_row_ptr, int64_t n,
-                                                         int64_t nnz, int32_t *__restrict__ new_col)
+                                                         int64_t nnz, int32_t *__restrict__ new_col,
+                                                         int *__restrict__ max_col)
 {
     __shared__ int64_t s_dst[kRemapRows + 1];
     __shared__ int64_t s_src[kRemapRows];
@@ -91,6 +109,7 @@ __global__ __launch_bounds__(256) void remap_rows_kernel(const int32_t *__restri
         s_src[r] = row_ptr[order[ra + r]];
     }
     __syncthreads();
+    int biggest = -1;
     for (int64_t p = p0 + threadIdx.x; p < p1; p += blockDim.x) {
         int64_t src;
         if (rows > 0) {
@@ -104,8 +123,17 @@ __global__ __launch_bounds__(256) void remap_rows_kernel(const int32_t *__restri
             const int64_t r = last_row_starting_at_or_before(new_row_ptr, ra, rb, p);
             src = row_ptr[order[r]] + (p - new_row_ptr[r]);
         }
-        new_col[p] = new_id[col[src]];
+        const int32_t c = new_id[col[src]];
+        new_col[p] = c;
+        biggest = c > biggest ? c : biggest;
     }
+    // the largest new id that is gathered at all (checks the counts the order was made from against the matrix)
+#pragma unroll
+    for (int m = kWave / 2; m > 0; m >>= 1) {
+        const int o = __shfl_xor(biggest, m, kWave);
+        biggest = o > biggest ? o : biggest;
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0 && biggest >= 0) atomicMax(max_col, biggest);
 }
 
 __global__ void remap_cols_kernel(const int32_t *__restrict__ col, const int32_t *__restrict__ new_id, int64_t nnz,
@@ -141,10 +169,13 @@ int relabel_create(Relabel *rl, int64_t n, int64_t nnz, const int64_t *row_ptr, 
     int32_t *ids = nullptr, *new_id = nullptr;
     int64_t *len = nullptr;
     void *temp = nullptr;
+    unsigned long long *live = nullptr;  // device: [0] vertices that are not isolated, [1] (as int) largest gathered new id
+    unsigned long long h_live[2] = {0, 0};
     size_t temp_bytes = 0, need = 0;
     const int blocks = 2048, threads = 256;
     rl->n = n;
     rl->nnz = nnz;
+    rl->live = n;
     RL_TRY(hipMalloc(&rl->order, sizeof(int32_t) * (size_t)n));
     RL_TRY(hipMalloc(&rl->row_ptr, sizeof(int64_t) * ((size_t)n + 1)));
     RL_TRY(hipMalloc(&rl->col, sizeof(int32_t) * (size_t)(nnz ? nnz : 1)));
@@ -153,11 +184,15 @@ int relabel_create(Relabel *rl, int64_t n, int64_t nnz, const int64_t *row_ptr, 
     RL_TRY(hipMalloc(&ids, sizeof(int32_t) * (size_t)n));
     RL_TRY(hipMalloc(&new_id, sizeof(int32_t) * (size_t)n));
     RL_TRY(hipMalloc(&len, sizeof(int64_t) * ((size_t)n + 1)));
+    RL_TRY(hipMalloc(&live, sizeof(unsigned long long) * 2));
+    RL_TRY(hipMemsetAsync(live, 0, sizeof(unsigned long long), stream));
+    RL_TRY(hipMemsetAsync(live + 1, 0xFF, sizeof(unsigned long long), stream));  // -1 as an int
     RL_TRY(hipMemsetAsync(count, 0, sizeof(unsigned) * (size_t)n, stream));
     RL_TRY(hipMemsetAsync(len + n, 0, sizeof(int64_t), stream));
     if (inv_outdeg) count_from_inverse_kernel<<<blocks, threads, 0, stream>>>(inv_outdeg, n, count);
     else if (transposed_offsets) count_from_offsets_kernel<<<blocks, threads, 0, stream>>>(transposed_offsets, n, count);
     else if (nnz) count_sources_kernel<<<blocks, threads, 0, stream>>>(col, nnz, count);
+    if (!keep_rows) order_keys_kernel<<<blocks, threads, 0, stream>>>(row_ptr, n, count, live);
     iota_kernel<<<blocks, threads, 0, stream>>>(ids, n);
     // stable descending sort by gather count: order[new] = old
     RL_TRY(rocprim::radix_sort_pairs_desc(nullptr, temp_bytes, count, count_sorted, ids, rl->order, (size_t)n, 0, 32,
@@ -178,9 +213,16 @@ int relabel_create(Relabel *rl, int64_t n, int64_t nnz, const int64_t *row_ptr, 
     }
     if (nnz > 0 && !keep_rows)
         remap_rows_kernel<<<(int)ceil_div(nnz, kRemapChunk), 256, 0, stream>>>(rl->order, row_ptr, col, new_id, rl->row_ptr, n,
-                                                                              nnz, rl->col);
+                                                                              nnz, rl->col, reinterpret_cast<int *>(live + 1));
     RL_TRY(hipGetLastError());
+    RL_TRY(hipMemcpyAsync(h_live, live, sizeof(h_live), hipMemcpyDeviceToHost, stream));
     RL_TRY(hipStreamSynchronize(stream));
+    if (!keep_rows) {
+        int max_col = -1;
+        memcpy(&max_col, &h_live[1], sizeof(int));
+        // rows [live, n) have no entries by construction; they are isolated if nobody gathers them either
+        rl->live = (int64_t)max_col < (int64_t)h_live[0] ? (int64_t)h_live[0] : n;
+    }
 done:
     (void)hipFree(count);
     (void)hipFree(count_sorted);
@@ -188,6 +230,7 @@ done:
     (void)hipFree(new_id);
     (void)hipFree(len);
     (void)hipFree(temp);
+    (void)hipFree(live);
     if (rc != DRONE_OK) relabel_destroy(rl);
     return rc;
 }
