@@ -108,7 +108,10 @@ SIGNATURES = {
     "drone_gcn_edge_values": (_I, [_I, _P, _P, _P, _P, _P, _P]),
     "drone_csr_transpose_f32": (_I, [_I, _I, _I64, _P, _P, _P, _P, _P, _P, _P]),
     "drone_spmm_plan_create": (_I, [C.POINTER(_P), _I, _I, _I64, _P, _P, _P, _I, _P]),
+    "drone_spmm_plan_create_scaled": (_I, [C.POINTER(_P), _I, _I, _I64, _P, _P, _P, _P, _P, _I, _P]),
+    "drone_gcn_degree_scales": (_I, [_I, _P, _P, _P]),
     "drone_spmm_plan_update_values": (_I, [_P, _P, _P]),
+    "drone_spmm_plan_bit_core": (_I, [_P, C.POINTER(_I64), C.POINTER(_I), C.POINTER(_I)]),
     "drone_spmm_plan_destroy": (_I, [_P]),
     "drone_spmm_csr_f32": (_I, [_P, _P, _P, _P, _P, _I, _P, _I, _I, _F, _F, _P]),
     "drone_spmm_bytes": (_I64, [_I, _I64, _I]),

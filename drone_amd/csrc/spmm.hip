@@ -42,6 +42,7 @@
 #include <rocprim/device/device_scan.hpp>
 
 #include "common.h"
+#include "spmm_bits.h"
 
 struct drone_spmm_plan {
     int n_rows = 0, n_cols = 0;
@@ -73,6 +74,10 @@ struct drone_spmm_plan {
     float *dense_a = nullptr;        // device: the rectangles, row-major, one after the other
     float *dense_b = nullptr;        // device [dense_wmax x ldk]: B's rows in rank order
     float *dense_t = nullptr;        // device [dense_rows x ldk]: products in rank order
+    // scaled pattern: the values are row_scale[row] * col_scale[col], and the dense part is kept as bits (spmm_bits.h)
+    bool scaled = false;
+    float *row_scale = nullptr, *col_scale = nullptr;  // device copies [n_rows], [n_cols]
+    drone::BitCore bits;
 };
 
 namespace drone {
@@ -95,7 +100,14 @@ constexpr float kDenseThreshold = 0.12f;  // for feature widths that fill 128-co
 constexpr double kGatherMsPerEntry = 0.19e-9;  // band-piece kernel: 24 ps per entry at K = 128
 constexpr double kDenseMsPerCell = 0.025e-9;   // dense product: 3.2 ps per cell at K = 128
 constexpr double kDenseMinGainMs = 0.25;
-static_assert(kDenseMaxCols / kDenseChunk <= 32, "the density histogram keeps at most 32 chunks per wavefront");
+// Scaled patterns (bit core): row groups of 4096 ranked long rows each, any leading set of 2048-column chunks.
+// Costs per cell of one 32-wide feature tile and per gathered entry of feature width 1, measured on the 232,965-vertex /
+// 229 M-entry graph.
+constexpr int kBitMaxChunks = 128;      // columns considered: the 262,144 most frequent
+constexpr int kBitGroupRows = 4096;
+constexpr int kBitMaxGroups = 1024;
+constexpr double kBitMsPerCellTile = 0.15e-9;   // ms: 0.15 ps per cell and 32 feature columns
+static_assert(kDenseMaxCols / kDenseChunk <= kBitMaxChunks, "the density histogram keeps at most 128 chunks per wavefront");
 
 template <int VEC> struct VecT;
 template <> struct VecT<4> { using type = float4; };
@@ -418,19 +430,19 @@ __global__ void col_rank_kernel(const unsigned *__restrict__ order, int n_cols, 
 
 // hist[group(row) * chunks + col_rank / kDenseChunk] += 1 over the entries of the ranked long rows whose column rank
 // is below chunks * kDenseChunk.  One wavefront per long row, counting in LDS first (the few global counters would
-// serialise 10^8 atomics); group_of_long[i] < 0 = row outside the groups.  chunks <= 32.
+// serialise 10^8 atomics); group_of_long[i] < 0 = row outside the groups.  chunks <= kBitMaxChunks.
 __global__ __launch_bounds__(256) void dense_histogram_kernel(int num_long, const int *__restrict__ long_row,
                                                               const int *__restrict__ group_of_long,
                                                               const int *__restrict__ rp, const int *__restrict__ ci,
                                                               const int *__restrict__ col_rank, int chunks,
                                                               unsigned *__restrict__ hist)
 {
-    __shared__ unsigned s_cnt[256 / kWave][32];
+    __shared__ unsigned s_cnt[256 / kWave][kBitMaxChunks];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     for (int i = (blockIdx.x * blockDim.x + threadIdx.x) / kWave; i < num_long; i += gridDim.x * blockDim.x / kWave) {
         const int g = group_of_long[i];
         if (g < 0) continue;  // the same for the whole wavefront
-        if (lane < 32) s_cnt[wave][lane] = 0;
+        for (int c = lane; c < kBitMaxChunks; c += kWave) s_cnt[wave][c] = 0;
         __builtin_amdgcn_wave_barrier();
         const int r = long_row[i], e0 = rp[r], e1 = rp[r + 1];
         for (int e = e0 + lane; e < e1; e += kWave) {
@@ -438,7 +450,8 @@ __global__ __launch_bounds__(256) void dense_histogram_kernel(int num_long, cons
             if (c < chunks) atomicAdd(&s_cnt[wave][c], 1u);
         }
         __builtin_amdgcn_wave_barrier();
-        if (lane < chunks && s_cnt[wave][lane]) atomicAdd(&hist[g * chunks + lane], s_cnt[wave][lane]);
+        for (int c = lane; c < chunks; c += kWave)
+            if (s_cnt[wave][c]) atomicAdd(&hist[g * chunks + c], s_cnt[wave][c]);
         __builtin_amdgcn_wave_barrier();
     }
 }
@@ -467,8 +480,8 @@ __global__ __launch_bounds__(256) void band_keys_kernel(int num_long, const int 
     }
 }
 
-// dense_a[row_off[rr] + col_rank[col]] = value over the dense entries of ranked row rr (one wavefront per row).
-// Cells without an entry keep the zero they were created with.
+// dense_a[row_off[rr] + col_rank[col]] += value over the dense entries of ranked row rr (one wavefront per row), on
+// cells that start at zero: a cell that the CSR stores more than once (a multigraph) holds the sum.
 __global__ __launch_bounds__(256) void dense_fill_kernel(int dense_rows, const int *__restrict__ seg_begin,
                                                          const int *__restrict__ seg_end, const int64_t *__restrict__ row_off,
                                                          const int *__restrict__ ci2, const float *__restrict__ val2,
@@ -476,7 +489,7 @@ __global__ __launch_bounds__(256) void dense_fill_kernel(int dense_rows, const i
 {
     const int lane = threadIdx.x & (kWave - 1);
     for (int rr = (blockIdx.x * blockDim.x + threadIdx.x) / kWave; rr < dense_rows; rr += gridDim.x * blockDim.x / kWave)
-        for (int p = seg_begin[rr] + lane; p < seg_end[rr]; p += kWave) a[row_off[rr] + col_rank[ci2[p]]] = val2[p];
+        for (int p = seg_begin[rr] + lane; p < seg_end[rr]; p += kWave) atomicAdd(&a[row_off[rr] + col_rank[ci2[p]]], val2[p]);
 }
 
 // dense_b[r, 0..K) = B[order[r], 0..K) for the leading ranks (one wavefront per row)
@@ -558,9 +571,12 @@ int launch_dense(const drone_spmm_plan *plan, const float *B, int ldb, float *C,
     return DRONE_OK;
 }
 
+// *duplicates: a scaled pattern turned out to hold some cell twice, which its bit core cannot represent; the plan is
+// then unusable and the caller builds an unscaled one.
 int build_band_pieces(drone_spmm_plan *p, const std::vector<int> &h_rp, const std::vector<int> &long_row,
-                      const int *rp, const int *ci, const float *v, hipStream_t s)
+                      const int *rp, const int *ci, const float *v, hipStream_t s, bool *duplicates)
 {
+    *duplicates = false;
     const int num_long = (int)long_row.size();
     std::vector<int> long_offset((size_t)num_long + 1, 0);
     for (int i = 0; i < num_long; ++i) long_offset[i + 1] = long_offset[i] + (h_rp[long_row[i] + 1] - h_rp[long_row[i]]);
@@ -585,12 +601,17 @@ int build_band_pieces(drone_spmm_plan *p, const std::vector<int> &h_rp, const st
         return long_offset[a + 1] - long_offset[a] > long_offset[b + 1] - long_offset[b];
     });
     for (int r = 0; r < num_long; ++r) rank_of_long[by_rank[r]] = r;
-    int group_begin[kDenseGroups + 1];
-    int groups = 0;
-    group_begin[0] = 0;
-    for (int g = 0, end = kDenseFirstRows; g < kDenseGroups && end <= num_long; ++g, end *= 2) group_begin[++groups] = end;
-    const int chunks = std::min(kDenseMaxCols, p->n_cols) / kDenseChunk;
-    std::vector<int> dense_width_of_long((size_t)num_long, 0), group_width((size_t)kDenseGroups, 0);
+    std::vector<int> group_begin(1, 0);
+    if (p->scaled) {
+        while ((int)group_begin.size() <= kBitMaxGroups && group_begin.back() < num_long)
+            group_begin.push_back(std::min(num_long, group_begin.back() + kBitGroupRows));
+    } else {
+        for (int g = 0, end = kDenseFirstRows; g < kDenseGroups && end <= num_long; ++g, end *= 2) group_begin.push_back(end);
+    }
+    const int groups = (int)group_begin.size() - 1;
+    const int chunks = p->scaled ? std::min(kBitMaxChunks, p->n_cols / kDenseChunk)
+                                 : std::min(kDenseMaxCols, p->n_cols) / kDenseChunk;
+    std::vector<int> dense_width_of_long((size_t)num_long, 0), group_width((size_t)std::max(groups, 1), 0);
 
     unsigned *counts = nullptr, *counts_sorted = nullptr, *col_ids = nullptr, *col_order = nullptr;
     unsigned char *band_of_col = nullptr;
@@ -654,19 +675,36 @@ int build_band_pieces(drone_spmm_plan *p, const std::vector<int> &h_rp, const st
             const int tile = p->max_k <= 64 ? 64 : (p->max_k + 127) / 128 * 128;
             const double efficiency = (double)p->max_k / tile * (tile == 64 ? 0.5 : 1.0);
             const double threshold = kDenseThreshold / efficiency;
-            double dense_entries = 0.0, dense_cells = 0.0;
-            for (int g = 0; g < groups; ++g) {
-                const double cells = (double)(group_begin[g + 1] - group_begin[g]) * kDenseChunk;
-                int w = 0;
-                while (w < chunks && hist[(size_t)g * chunks + w] / cells >= threshold) ++w;
-                if (w == 0) break;  // density falls with rank: later groups are sparser still
-                group_width[g] = w * kDenseChunk;
-                for (int c = 0; c < w; ++c) dense_entries += hist[(size_t)g * chunks + c];
-                dense_cells += cells * w;
+            double dense_entries = 0.0, dense_cells = 0.0, gain_ms = 0.0;
+            if (p->scaled) {
+                // bit core: per group, the leading chunks that maximise (gathers saved) - (cells multiplied)
+                const int feature_tiles = (int)ceil_div(p->max_k, 32);
+                for (int g = 0; g < groups; ++g) {
+                    const double cells = (double)ceil_div(group_begin[g + 1] - group_begin[g], kBitTileRows) * kBitTileRows * kDenseChunk;
+                    double run = 0.0, best = 0.0;
+                    int w = 0;
+                    for (int c = 0; c < chunks; ++c) {
+                        run += hist[(size_t)g * chunks + c] * p->max_k * kGatherMsPerEntry - cells * feature_tiles * kBitMsPerCellTile;
+                        if (run > best) { best = run; w = c + 1; }
+                    }
+                    if (w == 0) break;  // the dense rows must be a leading run of the ranking
+                    group_width[g] = w * kDenseChunk;
+                    gain_ms += best;
+                }
+            } else {
+                for (int g = 0; g < groups; ++g) {
+                    const double cells = (double)(group_begin[g + 1] - group_begin[g]) * kDenseChunk;
+                    int w = 0;
+                    while (w < chunks && hist[(size_t)g * chunks + w] / cells >= threshold) ++w;
+                    if (w == 0) break;  // density falls with rank: later groups are sparser still
+                    group_width[g] = w * kDenseChunk;
+                    for (int c = 0; c < w; ++c) dense_entries += hist[(size_t)g * chunks + c];
+                    dense_cells += cells * w;
+                }
+                // Worth it only when the estimated saving clears the fixed costs (gathering B's leading rows, the
+                // launches, adding the rows back): measured rates, ms per entry and per cell at feature width 1.
+                gain_ms = dense_entries * p->max_k * kGatherMsPerEntry - dense_cells * (p->max_k / efficiency) * kDenseMsPerCell;
             }
-            // Worth it only when the estimated saving clears the fixed costs (gathering B's leading rows, the
-            // launches, adding the rows back): measured rates, ms per entry and per cell at feature width 1.
-            const double gain_ms = dense_entries * p->max_k * kGatherMsPerEntry - dense_cells * (p->max_k / efficiency) * kDenseMsPerCell;
             if (gain_ms < kDenseMinGainMs) std::fill(group_width.begin(), group_width.end(), 0);
             for (int g = 0; g < groups && group_width[g] > 0; ++g)
                 for (int r = group_begin[g]; r < group_begin[g + 1]; ++r) dense_width_of_long[by_rank[r]] = group_width[g];
@@ -728,8 +766,27 @@ int build_band_pieces(drone_spmm_plan *p, const std::vector<int> &h_rp, const st
         DRONE_HIP_TRY(hipMemcpy(p->piece_begin, pb.data(), sizeof(int) * (size_t)num_pieces, hipMemcpyHostToDevice));
         DRONE_HIP_TRY(hipMemcpy(p->piece_end, pe.data(), sizeof(int) * (size_t)num_pieces, hipMemcpyHostToDevice));
         DRONE_HIP_TRY(hipMemcpy(p->piece_slot, ps.data(), sizeof(int) * (size_t)num_pieces, hipMemcpyHostToDevice));
-        // 5. the dense rectangles
-        if (dense_rows > 0) {
+        // 5. the dense part: bits for a scaled pattern, fp32 rectangles otherwise
+        if (dense_rows > 0 && p->scaled) {
+            std::vector<int> h_row((size_t)dense_rows), h_width((size_t)dense_rows);
+            for (int rr = 0; rr < dense_rows; ++rr) {
+                h_row[rr] = long_row[by_rank[rr]];
+                h_width[rr] = dense_width_of_long[by_rank[rr]];
+            }
+            p->dense_rows = dense_rows;
+            DRONE_HIP_TRY(hipMalloc(&p->dense_row, sizeof(int) * (size_t)dense_rows));
+            DRONE_HIP_TRY(hipMalloc(&p->dense_seg_begin, sizeof(int) * (size_t)dense_rows));
+            DRONE_HIP_TRY(hipMalloc(&p->dense_seg_end, sizeof(int) * (size_t)dense_rows));
+            DRONE_HIP_TRY(hipMemcpy(p->dense_row, h_row.data(), sizeof(int) * (size_t)dense_rows, hipMemcpyHostToDevice));
+            DRONE_HIP_TRY(hipMemcpy(p->dense_seg_begin, seg_begin.data(), sizeof(int) * (size_t)dense_rows, hipMemcpyHostToDevice));
+            DRONE_HIP_TRY(hipMemcpy(p->dense_seg_end, seg_end.data(), sizeof(int) * (size_t)dense_rows, hipMemcpyHostToDevice));
+            const int status = bit_core_create(&p->bits, dense_rows, h_width, p->dense_seg_begin, p->dense_seg_end, p->ci2,
+                                               p->col_rank, p->max_k, s, duplicates);
+            if (status != DRONE_OK) return status;
+            p->dense_wmax = p->bits.wmax;
+            p->col_order = col_order;  // kept: the SpMM reads B's leading rows through it
+            col_order = nullptr;
+        } else if (dense_rows > 0) {
             std::vector<int> h_row((size_t)dense_rows), h_width((size_t)dense_rows);
             std::vector<int64_t> h_off((size_t)dense_rows);
             size_t cells = 0;
@@ -785,13 +842,32 @@ int build_band_pieces(drone_spmm_plan *p, const std::vector<int> &h_rp, const st
 
 using namespace drone;
 
-extern "C" int drone_spmm_plan_create(drone_spmm_plan **out, int n_rows, int n_cols, int64_t nnz, const int *rp,
-                                      const int *ci, const float *v, int max_k, drone_stream_t stream)
+namespace {
+
+// How many entries deviate from row_scale[row] * col_scale[col] by more than a few roundings (one wavefront per row).
+__global__ __launch_bounds__(256) void check_scaled_values_kernel(int n_rows, const int *__restrict__ rp,
+                                                                  const int *__restrict__ ci, const float *__restrict__ v,
+                                                                  const float *__restrict__ row_scale,
+                                                                  const float *__restrict__ col_scale,
+                                                                  unsigned *__restrict__ mismatches)
 {
-    clear_error();
+    const int lane = threadIdx.x & (kWave - 1);
+    unsigned bad = 0;
+    for (int r = (blockIdx.x * blockDim.x + threadIdx.x) / kWave; r < n_rows; r += gridDim.x * blockDim.x / kWave) {
+        const float rs = row_scale[r];
+        for (int e = rp[r] + lane; e < rp[r + 1]; e += kWave) {
+            const float want = rs * col_scale[ci[e]];
+            if (!(fabsf(v[e] - want) <= 4e-6f * fabsf(want))) ++bad;  // also catches NaN and infinities
+        }
+    }
+    if (bad) atomicAdd(mismatches, bad);
+}
+
+int plan_create(drone_spmm_plan **out, int n_rows, int n_cols, int64_t nnz, const int *rp, const int *ci, const float *v,
+                const float *row_scale, const float *col_scale, int max_k, hipStream_t s)
+{
     DRONE_REQUIRE(out && n_rows >= 0 && n_cols >= 0 && nnz >= 0 && nnz < INT32_MAX && max_k > 0, "sizes");
     DRONE_REQUIRE(rp != nullptr && (nnz == 0 || (ci && v)), "null CSR array");
-    hipStream_t s = as_stream(stream);
     std::vector<int> h_rp((size_t)n_rows + 1);
     DRONE_HIP_TRY(hipMemcpyAsync(h_rp.data(), rp, sizeof(int) * h_rp.size(), hipMemcpyDeviceToHost, s));
     DRONE_HIP_TRY(hipStreamSynchronize(s));
@@ -802,28 +878,84 @@ extern "C" int drone_spmm_plan_create(drone_spmm_plan **out, int n_rows, int n_c
         DRONE_REQUIRE(len >= 0, "row_ptr must be non-decreasing");
         if (len > kSplitRow) long_row.push_back(r);
     }
-    drone_spmm_plan *p = new drone_spmm_plan();
-    p->n_rows = n_rows;
-    p->n_cols = n_cols;
-    p->nnz = nnz;
-    p->max_k = max_k;
-    if (!long_row.empty()) {
-        const int rc = build_band_pieces(p, h_rp, long_row, rp, ci, v, s);
-        if (rc != DRONE_OK) { drone_spmm_plan_destroy(p); return rc; }
+    bool scaled = row_scale != nullptr && col_scale != nullptr && !long_row.empty();
+    if (scaled) {  // the bit core stands on value = row_scale * col_scale: check it, entry by entry
+        unsigned *d_bad = nullptr, bad = 0;
+        DRONE_HIP_TRY(hipMalloc(&d_bad, sizeof(unsigned)));
+        (void)hipMemsetAsync(d_bad, 0, sizeof(unsigned), s);
+        int grid = (int)ceil_div(n_rows, 4);
+        if (grid > 65536) grid = 65536;
+        check_scaled_values_kernel<<<grid, 256, 0, s>>>(n_rows, rp, ci, v, row_scale, col_scale, d_bad);
+        const hipError_t e = hipMemcpyAsync(&bad, d_bad, sizeof(unsigned), hipMemcpyDeviceToHost, s);
+        const hipError_t e2 = hipStreamSynchronize(s);
+        (void)hipFree(d_bad);
+        DRONE_HIP_TRY(e);
+        DRONE_HIP_TRY(e2);
+        if (bad != 0) scaled = false;
     }
-    *out = p;
-    return DRONE_OK;
+    for (int attempt = 0; attempt < 2; ++attempt) {
+        drone_spmm_plan *p = new drone_spmm_plan();
+        p->n_rows = n_rows;
+        p->n_cols = n_cols;
+        p->nnz = nnz;
+        p->max_k = max_k;
+        p->scaled = scaled;
+        bool duplicates = false;
+        int rc = DRONE_OK;
+        if (scaled) {
+            const auto copy = [&]() -> int {
+                DRONE_HIP_TRY(hipMalloc(&p->row_scale, sizeof(float) * (size_t)std::max(n_rows, 1)));
+                DRONE_HIP_TRY(hipMalloc(&p->col_scale, sizeof(float) * (size_t)std::max(n_cols, 1)));
+                DRONE_HIP_TRY(hipMemcpyAsync(p->row_scale, row_scale, sizeof(float) * (size_t)n_rows, hipMemcpyDeviceToDevice, s));
+                DRONE_HIP_TRY(hipMemcpyAsync(p->col_scale, col_scale, sizeof(float) * (size_t)n_cols, hipMemcpyDeviceToDevice, s));
+                return DRONE_OK;
+            };
+            rc = copy();
+        }
+        if (rc == DRONE_OK && !long_row.empty()) rc = build_band_pieces(p, h_rp, long_row, rp, ci, v, s, &duplicates);
+        if (rc == DRONE_OK && !duplicates) {
+            *out = p;
+            return DRONE_OK;
+        }
+        drone_spmm_plan_destroy(p);
+        if (rc != DRONE_OK) return rc;
+        scaled = false;  // a multigraph: cells with several entries need the fp32 rectangles
+    }
+    return DRONE_OK;  // not reached: the unscaled build reports no duplicates
+}
+
+}  // namespace
+
+extern "C" int drone_spmm_plan_create(drone_spmm_plan **out, int n_rows, int n_cols, int64_t nnz, const int *rp,
+                                      const int *ci, const float *v, int max_k, drone_stream_t stream)
+{
+    clear_error();
+    return plan_create(out, n_rows, n_cols, nnz, rp, ci, v, nullptr, nullptr, max_k, as_stream(stream));
+}
+
+extern "C" int drone_spmm_plan_create_scaled(drone_spmm_plan **out, int n_rows, int n_cols, int64_t nnz, const int *rp,
+                                             const int *ci, const float *v, const float *row_scale,
+                                             const float *col_scale, int max_k, drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(row_scale != nullptr && col_scale != nullptr, "null scale array");
+    return plan_create(out, n_rows, n_cols, nnz, rp, ci, v, row_scale, col_scale, max_k, as_stream(stream));
 }
 
 extern "C" int drone_spmm_plan_update_values(drone_spmm_plan *p, const float *v, drone_stream_t stream)
 {
     clear_error();
     DRONE_REQUIRE(p != nullptr && (p->nnz == 0 || v), "null argument");
+    DRONE_REQUIRE(p->bits.tiles == 0, "the plan holds a scaled pattern as bits: its values are fixed by the scales");
     if (p->long_nnz > 0) {
         gather_sorted_kernel<<<4096, 256, 0, as_stream(stream)>>>(p->long_nnz, p->perm, nullptr, v, nullptr, p->val2);
-        if (p->dense_rows > 0)  // cells without an entry stay zero, the others are overwritten
+        if (p->dense_rows > 0) {
+            int64_t cells = 0;
+            for (int i = 0; i < p->num_rects; ++i) cells += (int64_t)p->rects[i].rows * p->rects[i].width;
+            DRONE_HIP_TRY(hipMemsetAsync(p->dense_a, 0, sizeof(float) * (size_t)cells, as_stream(stream)));
             dense_fill_kernel<<<(int)ceil_div(p->dense_rows, 4), 256, 0, as_stream(stream)>>>(
                 p->dense_rows, p->dense_seg_begin, p->dense_seg_end, p->dense_row_off, p->ci2, p->val2, p->col_rank, p->dense_a);
+        }
         DRONE_HIP_TRY(hipGetLastError());
     }
     return DRONE_OK;
@@ -851,6 +983,9 @@ extern "C" int drone_spmm_plan_destroy(drone_spmm_plan *p)
     (void)hipFree(p->dense_a);
     (void)hipFree(p->dense_b);
     (void)hipFree(p->dense_t);
+    (void)hipFree(p->row_scale);
+    (void)hipFree(p->col_scale);
+    drone::bit_core_destroy(&p->bits);
     delete p;
     return DRONE_OK;
 }
@@ -862,11 +997,22 @@ extern "C" int drone_spmm_plan_info(const drone_spmm_plan *p, int64_t *long_nnz,
     DRONE_REQUIRE(p != nullptr, "plan");
     int64_t cells = 0;
     for (int i = 0; i < p->num_rects; ++i) cells += (int64_t)p->rects[i].rows * p->rects[i].width;
+    cells += p->bits.cells;
     if (long_nnz) *long_nnz = p->long_nnz;
     if (dense_nnz) *dense_nnz = p->dense_nnz;
     if (dense_cells) *dense_cells = cells;
     if (dense_rows) *dense_rows = p->dense_rows;
     if (dense_cols) *dense_cols = p->dense_wmax;
+    return DRONE_OK;
+}
+
+extern "C" int drone_spmm_plan_bit_core(const drone_spmm_plan *p, int64_t *cells, int *rows, int *cols)
+{
+    clear_error();
+    DRONE_REQUIRE(p != nullptr, "plan");
+    if (cells) *cells = p->bits.cells;
+    if (rows) *rows = p->bits.rows;
+    if (cols) *cols = p->bits.wmax;
     return DRONE_OK;
 }
 
@@ -903,7 +1049,10 @@ extern "C" int drone_spmm_csr_f32(const drone_spmm_plan *plan, const int *rp, co
         else if (K <= 32) launch_spmm<32, 1>(plan, rp, ci, v, B, ldb, C, ldc, K, alpha, beta, s);
         else launch_spmm<64, 1>(plan, rp, ci, v, B, ldb, C, ldc, K, alpha, beta, s);
     }
-    const int dense_status = launch_dense(plan, B, ldb, C, ldc, K, alpha, s);
+    const int dense_status = plan->bits.tiles > 0
+                                 ? bit_core_multiply(&plan->bits, plan->col_order, plan->col_scale, plan->dense_row,
+                                                     plan->row_scale, B, ldb, C, ldc, K, alpha, s)
+                                 : launch_dense(plan, B, ldb, C, ldc, K, alpha, s);
     if (dense_status != DRONE_OK) return dense_status;
     DRONE_HIP_TRY(hipGetLastError());
     return DRONE_OK;
@@ -918,6 +1067,24 @@ extern "C" int drone_gcn_edge_values(int n, const int *rp, const int *ci, const 
     int blocks = (int)ceil_div(n, 4);
     if (blocks > 65536) blocks = 65536;
     edge_values_kernel<<<blocks, 256, 0, as_stream(stream)>>>(n, rp, ci, in_deg, out_deg, v);
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
+namespace {
+__global__ void degree_scales_kernel(int n, const int *__restrict__ degree, float *__restrict__ out)
+{
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
+        out[i] = degree[i] > 0 ? 1.0f / sqrtf((float)degree[i]) : 0.0f;
+}
+}  // namespace
+
+extern "C" int drone_gcn_degree_scales(int n, const int *degree, float *out, drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(n >= 0 && (n == 0 || (degree && out)), "null operand");
+    if (n == 0) return DRONE_OK;
+    degree_scales_kernel<<<(int)std::min<int64_t>(ceil_div(n, 256), 4096), 256, 0, as_stream(stream)>>>(n, degree, out);
     DRONE_HIP_TRY(hipGetLastError());
     return DRONE_OK;
 }

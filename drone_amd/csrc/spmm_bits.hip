@@ -1,0 +1,373 @@
+// Bit-matrix core of the SpMM: see spmm_bits.h for what it computes and why.
+//
+// Layouts (all chosen so that every global and LDS access of the product kernel is a contiguous 16-byte read):
+//  * bits: a tile is 512 ranked rows.  Its cells are kept per 32-row group g and 256-column block b as 64 x 16 bytes:
+//    lane l of a wavefront owns row l % 32 of the group and, in every 16-column step s of the block, the 8 columns
+//    16 s + 8 (l / 32) .. + 8 - byte s of its 16 bytes, least significant bit first.  That byte is exactly the lane's
+//    share of the A operand of one v_mfma_f32_32x32x16_bf16 (8 values of one row).
+//  * split operand: for ranked column q and feature column n, x = col_scale * B is written as hi + mid + lo (bf16
+//    each, round-to-nearest of the running remainder, so the three add up to x exactly).  Eight consecutive q form
+//    a group; a group holds, per part and per 32-wide feature tile, 32 x 16 bytes: feature column n % 32, the
+//    group's 8 ranked columns - a lane's share of the B operand.
+//  * The A and B operands use the same (lane / 32, element) -> column mapping, so the sum over the 16 columns of a
+//    step does not depend on how the instruction numbers them.
+#include <algorithm>
+
+#include "spmm_bits.h"
+
+namespace drone {
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kGroupVecs = 3 * 4 * 32;  // 16-byte words of one 8-column group in `split`: 3 parts x 4 feature tiles x 32
+constexpr int kPartialLd = 128;
+
+// One wavefront per ranked row: sets the bit of every dense entry.
+__global__ __launch_bounds__(256) void bits_fill_kernel(int rows, const int *__restrict__ seg_begin,
+                                                        const int *__restrict__ seg_end, const int *__restrict__ cols,
+                                                        const int *__restrict__ col_rank,
+                                                        const int *__restrict__ tile_blocks,
+                                                        const int64_t *__restrict__ tile_off, unsigned *__restrict__ bits,
+                                                        int *__restrict__ duplicates)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    for (int rr = (blockIdx.x * blockDim.x + threadIdx.x) / kWave; rr < rows; rr += gridDim.x * blockDim.x / kWave) {
+        const int tile = rr / kBitTileRows, group = (rr % kBitTileRows) / 32, m = rr % 32;
+        const int blocks = tile_blocks[tile];
+        unsigned *base = bits + 4 * (size_t)tile_off[tile];
+        for (int p = seg_begin[rr] + lane; p < seg_end[rr]; p += kWave) {
+            const int q = col_rank[cols[p]];
+            const int block = q / kBitBlockCols, step = (q % kBitBlockCols) / 16, half = (q % 16) / 8, bit = q % 8;
+            if (block >= blocks) continue;  // cannot happen for a consistent plan; never write outside the tile
+            const size_t word = (((size_t)group * blocks + block) * 64 + half * 32 + m) * 4 + step / 4;
+            const unsigned mask = 1u << ((step % 4) * 8 + bit);
+            if (atomicOr(base + word, mask) & mask) *duplicates = 1;
+        }
+    }
+}
+
+__device__ __forceinline__ unsigned bf16_bits_rne(float x)
+{
+    const unsigned u = __float_as_uint(x);
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+
+// Thread (group of 8 ranked columns, feature column n of the pass): scales, splits and packs 8 values of B.
+__global__ __launch_bounds__(256) void bits_split_kernel(int groups, const unsigned *__restrict__ col_order,
+                                                         const float *__restrict__ col_scale,
+                                                         const float *__restrict__ B, int ldb, int K,
+                                                         uint4 *__restrict__ split)
+{
+    const int kg = blockIdx.x * 2 + threadIdx.x / 128, pass = blockIdx.y;
+    if (kg >= groups) return;
+    const int n = threadIdx.x % 128, k = pass * 128 + n;
+    unsigned part[3][8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const unsigned col = col_order[kg * 8 + j];
+        const float x = k < K ? col_scale[col] * B[(size_t)col * ldb + k] : 0.0f;
+        const unsigned hi = bf16_bits_rne(x);
+        const float r1 = x - __uint_as_float(hi << 16);
+        const unsigned mid = bf16_bits_rne(r1);
+        const float r2 = r1 - __uint_as_float(mid << 16);
+        part[0][j] = hi;
+        part[1][j] = mid;
+        part[2][j] = bf16_bits_rne(r2);
+    }
+    uint4 *dst = split + ((size_t)pass * groups + kg) * kGroupVecs + (n / 32) * 32 + n % 32;
+#pragma unroll
+    for (int t = 0; t < 3; ++t)
+        dst[t * 4 * 32] = make_uint4(part[t][0] | part[t][1] << 16, part[t][2] | part[t][3] << 16,
+                                     part[t][4] | part[t][5] << 16, part[t][6] | part[t][7] << 16);
+}
+
+// 8 cells of one row -> 8 bf16 values 1.0 / 0.0
+__device__ __forceinline__ bf16x8 expand_bits(unsigned byte)
+{
+    u32x4 v;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        unsigned t = (byte >> (2 * j)) & 3u;
+        t = (t | (t << 15)) & 0x00010001u;
+        v[j] = t * 0x3F80u;
+    }
+    return __builtin_bit_cast(bf16x8, v);
+}
+
+// One work-group (8 wavefronts) per unit: T[512 x 64 CT] = bits(512 x [c0, c1)) * split([c0, c1) x 64 CT), the three
+// parts summed.  Wavefront w owns rows 128 (w / 2) .. + 128 and feature tiles CT (w % 2) .. + CT as 4 x CT accumulators
+// of 32 x 32, so a 16-byte LDS read of the split operand feeds four matrix instructions.  The split operand of 32
+// columns (a stage: 4 groups x 3 parts x 2 CT tiles x 512 bytes) goes through LDS, double buffered, fetched one stage
+// ahead; the bits come straight from global memory, one 256-column block ahead.
+// Measured on 1.14 G cells with 128 feature columns (ms): matrix instructions alone 0.46 (1.9 PFLOP/s), with the LDS
+// reads 0.52; work-groups of 4 wavefronts x 64 rows x 128 feature columns, two per CU, took 1.12 with the staging
+// through LDS - 64 bytes read and 32 written per clock and CU are more than the LDS delivers next to the matrix cores.
+template <int CT>
+__global__ __launch_bounds__(512, 1) void bits_mfma_kernel(const int *__restrict__ unit_tile,
+                                                           const int *__restrict__ unit_c0,
+                                                           const int *__restrict__ unit_c1,
+                                                           const int *__restrict__ unit_slot,
+                                                           const int *__restrict__ tile_blocks,
+                                                           const int64_t *__restrict__ tile_off,
+                                                           const uint4 *__restrict__ bits,
+                                                           const uint4 *__restrict__ split, float *__restrict__ partial)
+{
+    constexpr int NT = 2 * CT;
+    constexpr int kStageVecs = 4 * 3 * NT * 32;
+    constexpr int kPre = (kStageVecs + 511) / 512;
+    __shared__ uint4 s_b[2][kStageVecs];
+    const int u = blockIdx.x, tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int wr = wave >> 1, wc = wave & 1;
+    const int tile = unit_tile[u], c0 = unit_c0[u], c1 = unit_c1[u];
+    const int blocks = tile_blocks[tile], nblocks = (c1 - c0) / kBitBlockCols;
+    const uint4 *w0 = bits + tile_off[tile] + ((size_t)(4 * wr) * blocks + c0 / kBitBlockCols) * 64 + lane;
+    const size_t wstep = (size_t)blocks * 64;
+    const uint4 *src = split + (size_t)(c0 / 8) * kGroupVecs;
+    int goff[kPre];
+#pragma unroll
+    for (int i = 0; i < kPre; ++i) {
+        const int v = tid + 512 * i;
+        const int g = v / (3 * NT * 32), rem = v % (3 * NT * 32);
+        goff[i] = g * kGroupVecs + (rem / (NT * 32)) * 4 * 32 + ((rem / 32) % NT) * 32 + rem % 32;
+    }
+    f32x16 acc[4][CT];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < CT; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    uint4 pre[kPre];
+    // The work-groups resident at one time share a column range (launch order) and would walk it in step, all asking
+    // one L2 channel for the same line at the same moment: every tile starts at its own block of the range and wraps.
+    const int rot = (tile * 5) % nblocks;
+    uint4 a[4], an[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a[i] = w0[i * wstep + (size_t)rot * 64];
+    {
+        const uint4 *first = src + (size_t)rot * 32 * kGroupVecs;
+#pragma unroll
+        for (int i = 0; i < kPre; ++i)
+            if (tid + 512 * i < kStageVecs) pre[i] = first[goff[i]];
+#pragma unroll
+        for (int i = 0; i < kPre; ++i)
+            if (tid + 512 * i < kStageVecs) s_b[0][tid + 512 * i] = pre[i];
+    }
+    __syncthreads();
+    for (int kb = 0; kb < nblocks; ++kb) {
+        const int block = kb + rot < nblocks ? kb + rot : kb + rot - nblocks;
+        const int block_next = block + 1 < nblocks ? block + 1 : 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) an[i] = w0[i * wstep + (size_t)block_next * 64];
+        unsigned aw[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            aw[i][0] = a[i].x;
+            aw[i][1] = a[i].y;
+            aw[i][2] = a[i].z;
+            aw[i][3] = a[i].w;
+        }
+#pragma unroll
+        for (int st = 0; st < 8; ++st) {
+            const bool more = kb + 1 < nblocks || st < 7;
+#ifndef BITS_EXP_NOGLOBAL
+            if (more) {
+                const uint4 *next = src + (size_t)(st < 7 ? block * 8 + st + 1 : block_next * 8) * 4 * kGroupVecs;
+#pragma unroll
+                for (int i = 0; i < kPre; ++i)
+                    if (tid + 512 * i < kStageVecs) pre[i] = next[goff[i]];
+            }
+#endif
+            const uint4 *cur = s_b[st & 1];
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                const int idx = st * 2 + ks;
+                bf16x8 A[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) A[i] = expand_bits((aw[i][idx / 4] >> ((idx % 4) * 8)) & 0xFFu);
+#pragma unroll
+                for (int part = 0; part < 3; ++part)
+#pragma unroll
+                    for (int ct = 0; ct < CT; ++ct) {
+                        const uint4 raw = cur[(((2 * ks + (lane >> 5)) * 3 + part) * NT + wc * CT + ct) * 32 + (lane & 31)];
+                        const bf16x8 bv = __builtin_bit_cast(bf16x8, raw);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            acc[i][ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[i], bv, acc[i][ct], 0, 0, 0);
+                    }
+            }
+#ifndef BITS_EXP_NOSTORE
+            if (more) {
+#pragma unroll
+                for (int i = 0; i < kPre; ++i)
+                    if (tid + 512 * i < kStageVecs) s_b[(st & 1) ^ 1][tid + 512 * i] = pre[i];
+            }
+#endif
+#ifndef BITS_EXP_NOSYNC
+            __syncthreads();
+#endif
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a[i] = an[i];
+    }
+    float *out = partial + (size_t)unit_slot[u] * kBitTileRows * kPartialLd;
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = 128 * wr + 32 * rt + (r / 4) * 8 + (lane >> 5) * 4 + (r % 4);
+                out[(size_t)row * kPartialLd + 32 * (wc * CT + ct) + (lane & 31)] = acc[rt][ct][r];
+            }
+}
+
+// One wavefront per ranked row: adds the units' tile sums of the row, scales and adds into C.
+__global__ __launch_bounds__(256) void bits_combine_kernel(int rows, const int *__restrict__ tile_unit0,
+                                                           const float *__restrict__ partial, int num_units, int passes,
+                                                           const int *__restrict__ dense_row,
+                                                           const float *__restrict__ row_scale, float *__restrict__ C,
+                                                           int ldc, int K, float alpha)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    for (int rr = (blockIdx.x * blockDim.x + threadIdx.x) / kWave; rr < rows; rr += gridDim.x * blockDim.x / kWave) {
+        const int tile = rr / kBitTileRows, u0 = tile_unit0[tile], u1 = tile_unit0[tile + 1];
+        const int row = dense_row[rr];
+        const float scale = alpha * row_scale[row];
+        for (int k = lane; k < K; k += kWave) {
+            const float *src = partial + ((size_t)(k / 128) * num_units * kBitTileRows + rr % kBitTileRows) * kPartialLd + k % 128;
+            float sum = 0.0f;
+            for (int u = u0; u < u1; ++u) sum += src[(size_t)u * kBitTileRows * kPartialLd];
+            C[(size_t)row * ldc + k] += scale * sum;
+        }
+    }
+}
+
+}  // namespace
+
+int bit_core_create(BitCore *bc, int rows, const std::vector<int> &width_of_row, const int *seg_begin, const int *seg_end,
+                    const int *cols, const int *col_rank, int max_k, hipStream_t s, bool *has_duplicates)
+{
+    *has_duplicates = false;
+    if (rows <= 0) return DRONE_OK;
+    const int tiles = (int)ceil_div(rows, kBitTileRows);
+    std::vector<int> blocks((size_t)tiles), unit0((size_t)tiles + 1, 0), ut, uc0, uc1;
+    std::vector<int64_t> off((size_t)tiles);
+    int64_t words = 0, cells = 0;
+    int wmax = 0;
+    for (int t = 0; t < tiles; ++t) {
+        const int w = width_of_row[(size_t)t * kBitTileRows];
+        DRONE_REQUIRE(w > 0 && w % kBitBlockCols == 0, "dense width must be a positive multiple of 256");
+        blocks[t] = w / kBitBlockCols;
+        off[t] = words;
+        words += (int64_t)(kBitTileRows / 32) * blocks[t] * 64;
+        cells += (int64_t)kBitTileRows * w;
+        wmax = std::max(wmax, w);
+    }
+    // Units: the columns are cut on one grid for all tiles, so that about 1024 work-groups share the cells (one is
+    // resident per CU), never below 2048 columns (a unit's result is a 256 KB tile that is written and read once).
+    // Launch order is column range first, tile second: the work-groups resident at any moment then read the same few
+    // megabytes of the split operand, which L2 serves; in tile order every work-group streamed its own range from
+    // memory.  A unit's slot (where its sums go) stays tile-major, so that a row's sums are adjacent.
+    int unit_cols = (int)ceil_div(ceil_div(cells, (int64_t)kBitTileRows * 1024), kBitBlockCols) * kBitBlockCols;
+    unit_cols = std::max(unit_cols, 2048);
+    for (int t = 0; t < tiles; ++t) unit0[t + 1] = unit0[t] + (int)ceil_div(blocks[t] * kBitBlockCols, unit_cols);
+    std::vector<int> uslot;
+    for (int j = 0; j * unit_cols < wmax; ++j)
+        for (int t = 0; t < tiles; ++t) {
+            const int w = blocks[t] * kBitBlockCols;
+            if (j * unit_cols >= w) continue;
+            ut.push_back(t);
+            uc0.push_back(j * unit_cols);
+            uc1.push_back(std::min((j + 1) * unit_cols, w));
+            uslot.push_back(unit0[t] + j);
+        }
+    bc->tiles = tiles;
+    bc->rows = rows;
+    bc->wmax = wmax;
+    bc->cells = cells;
+    bc->max_k = max_k;
+    bc->passes = (int)ceil_div(max_k, 128);
+    bc->num_units = (int)ut.size();
+    const size_t nu = ut.size();
+    DRONE_HIP_TRY(hipMalloc(&bc->unit_tile, sizeof(int) * nu));
+    DRONE_HIP_TRY(hipMalloc(&bc->unit_c0, sizeof(int) * nu));
+    DRONE_HIP_TRY(hipMalloc(&bc->unit_c1, sizeof(int) * nu));
+    DRONE_HIP_TRY(hipMalloc(&bc->unit_slot, sizeof(int) * nu));
+    DRONE_HIP_TRY(hipMalloc(&bc->tile_unit0, sizeof(int) * unit0.size()));
+    DRONE_HIP_TRY(hipMalloc(&bc->tile_blocks, sizeof(int) * (size_t)tiles));
+    DRONE_HIP_TRY(hipMalloc(&bc->tile_off, sizeof(int64_t) * (size_t)tiles));
+    DRONE_HIP_TRY(hipMalloc(&bc->bits, sizeof(uint4) * (size_t)words));
+    DRONE_HIP_TRY(hipMalloc(&bc->split, sizeof(uint4) * (size_t)bc->passes * (wmax / 8) * kGroupVecs));
+    DRONE_HIP_TRY(hipMalloc(&bc->partial, sizeof(float) * (size_t)bc->passes * nu * kBitTileRows * kPartialLd));
+    DRONE_HIP_TRY(hipMalloc(&bc->duplicates, sizeof(int)));
+    DRONE_HIP_TRY(hipMemcpyAsync(bc->unit_tile, ut.data(), sizeof(int) * nu, hipMemcpyHostToDevice, s));
+    DRONE_HIP_TRY(hipMemcpyAsync(bc->unit_c0, uc0.data(), sizeof(int) * nu, hipMemcpyHostToDevice, s));
+    DRONE_HIP_TRY(hipMemcpyAsync(bc->unit_c1, uc1.data(), sizeof(int) * nu, hipMemcpyHostToDevice, s));
+    DRONE_HIP_TRY(hipMemcpyAsync(bc->unit_slot, uslot.data(), sizeof(int) * nu, hipMemcpyHostToDevice, s));
+    DRONE_HIP_TRY(hipMemcpyAsync(bc->tile_unit0, unit0.data(), sizeof(int) * unit0.size(), hipMemcpyHostToDevice, s));
+    DRONE_HIP_TRY(hipMemcpyAsync(bc->tile_blocks, blocks.data(), sizeof(int) * (size_t)tiles, hipMemcpyHostToDevice, s));
+    DRONE_HIP_TRY(hipMemcpyAsync(bc->tile_off, off.data(), sizeof(int64_t) * (size_t)tiles, hipMemcpyHostToDevice, s));
+    DRONE_HIP_TRY(hipMemsetAsync(bc->bits, 0, sizeof(uint4) * (size_t)words, s));
+    DRONE_HIP_TRY(hipMemsetAsync(bc->duplicates, 0, sizeof(int), s));
+    int grid = (int)ceil_div(rows, 4);
+    if (grid > 65536) grid = 65536;
+    bits_fill_kernel<<<grid, 256, 0, s>>>(rows, seg_begin, seg_end, cols, col_rank, bc->tile_blocks, bc->tile_off,
+                                          reinterpret_cast<unsigned *>(bc->bits), bc->duplicates);
+    DRONE_HIP_TRY(hipGetLastError());
+    int dup = 0;
+    DRONE_HIP_TRY(hipMemcpyAsync(&dup, bc->duplicates, sizeof(int), hipMemcpyDeviceToHost, s));
+    DRONE_HIP_TRY(hipStreamSynchronize(s));  // also keeps the host vectors alive until their copies are done
+    *has_duplicates = dup != 0;
+    return DRONE_OK;
+}
+
+void bit_core_destroy(BitCore *bc)
+{
+    (void)hipFree(bc->unit_tile);
+    (void)hipFree(bc->unit_c0);
+    (void)hipFree(bc->unit_c1);
+    (void)hipFree(bc->unit_slot);
+    (void)hipFree(bc->tile_unit0);
+    (void)hipFree(bc->tile_blocks);
+    (void)hipFree(bc->tile_off);
+    (void)hipFree(bc->bits);
+    (void)hipFree(bc->split);
+    (void)hipFree(bc->partial);
+    (void)hipFree(bc->duplicates);
+    *bc = BitCore();
+}
+
+int bit_core_multiply(const BitCore *bc, const unsigned *col_order, const float *col_scale, const int *dense_row,
+                      const float *row_scale, const float *B, int ldb, float *C, int ldc, int K, float alpha,
+                      hipStream_t s)
+{
+    if (bc->tiles == 0) return DRONE_OK;
+    DRONE_REQUIRE(K > 0 && K <= bc->max_k, "K exceeds the plan's feature width");
+    const int groups = bc->wmax / 8, passes = (int)ceil_div(K, 128);
+    bits_split_kernel<<<dim3((unsigned)ceil_div(groups, 2), (unsigned)passes), 256, 0, s>>>(groups, col_order, col_scale, B,
+                                                                                           ldb, K, bc->split);
+    for (int pass = 0; pass < passes; ++pass) {
+        const int width = std::min(K - pass * 128, 128);
+        const uint4 *split = bc->split + (size_t)pass * groups * kGroupVecs;
+        float *partial = bc->partial + (size_t)pass * bc->num_units * kBitTileRows * kPartialLd;
+        if (width <= 64)
+            bits_mfma_kernel<1><<<bc->num_units, 512, 0, s>>>(bc->unit_tile, bc->unit_c0, bc->unit_c1, bc->unit_slot,
+                                                             bc->tile_blocks, bc->tile_off, bc->bits, split, partial);
+        else
+            bits_mfma_kernel<2><<<bc->num_units, 512, 0, s>>>(bc->unit_tile, bc->unit_c0, bc->unit_c1, bc->unit_slot,
+                                                             bc->tile_blocks, bc->tile_off, bc->bits, split, partial);
+    }
+    int grid = (int)ceil_div(bc->rows, 4);
+    if (grid > 65536) grid = 65536;
+    bits_combine_kernel<<<grid, 256, 0, s>>>(bc->rows, bc->tile_unit0, bc->partial, bc->num_units, passes, dense_row,
+                                             row_scale, C, ldc, K, alpha);
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
+}  // namespace drone

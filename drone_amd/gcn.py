@@ -34,18 +34,32 @@ def csr_transpose(n_rows, n_cols, rp, ci, val=None, stream=0):
     return rpT, ciT, vT
 
 
+def degree_scales(degree, stream=0):
+    """drone_gcn_degree_scales: 1 / sqrt(degree) as fp32, 0 where the degree is 0."""
+    import torch
+    out = torch.empty(degree.numel(), dtype=torch.float32, device=degree.device)
+    check(lib().drone_gcn_degree_scales(degree.numel(), _ptr(degree), _ptr(out), stream))
+    return out
+
+
 class SpmmPlan:
     """Schedule (and band-sorted copy of the long rows) for the SpMM of one CSR; see drone_spmm_plan_create."""
 
-    def __init__(self, rp, ci, val, n_cols, max_k, stream=0):
+    def __init__(self, rp, ci, val, n_cols, max_k, stream=0, row_scale=None, col_scale=None):
+        """With row_scale / col_scale (val[e] = row_scale[row] * col_scale[col]): drone_spmm_plan_create_scaled."""
         self.n_rows = rp.numel() - 1
         self.n_cols = int(n_cols)
         self.nnz = int(ci.numel())
         self.max_k = int(max_k)
         self._keep = (rp, ci, val)
         h = C.c_void_p()
-        check(lib().drone_spmm_plan_create(C.byref(h), self.n_rows, self.n_cols, self.nnz, _ptr(rp), _ptr(ci), _ptr(val),
-                                           self.max_k, stream))
+        if row_scale is not None:
+            assert row_scale.numel() == self.n_rows and col_scale.numel() == self.n_cols
+            check(lib().drone_spmm_plan_create_scaled(C.byref(h), self.n_rows, self.n_cols, self.nnz, _ptr(rp), _ptr(ci),
+                                                      _ptr(val), _ptr(row_scale), _ptr(col_scale), self.max_k, stream))
+        else:
+            check(lib().drone_spmm_plan_create(C.byref(h), self.n_rows, self.n_cols, self.nnz, _ptr(rp), _ptr(ci),
+                                               _ptr(val), self.max_k, stream))
         self.h = h
 
     def update_values(self, val, stream=0):
@@ -57,6 +71,12 @@ class SpmmPlan:
         d, e = C.c_int(0), C.c_int(0)
         check(lib().drone_spmm_plan_info(self.h, C.byref(a), C.byref(b), C.byref(c), C.byref(d), C.byref(e)))
         return dict(long_nnz=a.value, dense_nnz=b.value, dense_cells=c.value, dense_rows=d.value, dense_cols=e.value)
+
+    def bit_core(self):
+        """drone_spmm_plan_bit_core: cells / ranked rows / ranked columns kept as bits (zeros for an unscaled plan)."""
+        a, d, e = C.c_int64(0), C.c_int(0), C.c_int(0)
+        check(lib().drone_spmm_plan_bit_core(self.h, C.byref(a), C.byref(d), C.byref(e)))
+        return dict(cells=a.value, rows=d.value, cols=e.value)
 
     def close(self):
         if self.h:

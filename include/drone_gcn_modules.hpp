@@ -141,8 +141,17 @@ struct Adjacency {
         DRONE_GCN_HIP(hipMalloc(&valT, sizeof(float) * e));
         DRONE_GCN_CHECK(drone_gcn_edge_values(n, rp, ci, in_degree, out_degree, val, s));
         DRONE_GCN_CHECK(drone_csr_transpose_f32(n, n, nnz, rp, ci, val, rpT, ciT, valT, s));
-        DRONE_GCN_CHECK(drone_spmm_plan_create(&plan, n, n, nnz, rp, ci, val, max_dim, s));
-        DRONE_GCN_CHECK(drone_spmm_plan_create(&planT, n, n, nnz, rpT, ciT, valT, max_dim, s));
+        // The values are 1/sqrt(out_degree[row]) * 1/sqrt(in_degree[col]) up to rounding: telling the plans lets them
+        // keep the dense part of the pattern as bits (drone_spmm_plan_create_scaled checks the claim entry by entry).
+        float *out_scale = nullptr, *in_scale = nullptr;
+        DRONE_GCN_HIP(hipMalloc(&out_scale, sizeof(float) * (size_t)(n ? n : 1)));
+        DRONE_GCN_HIP(hipMalloc(&in_scale, sizeof(float) * (size_t)(n ? n : 1)));
+        DRONE_GCN_CHECK(drone_gcn_degree_scales(n, out_degree, out_scale, s));
+        DRONE_GCN_CHECK(drone_gcn_degree_scales(n, in_degree, in_scale, s));
+        DRONE_GCN_CHECK(drone_spmm_plan_create_scaled(&plan, n, n, nnz, rp, ci, val, out_scale, in_scale, max_dim, s));
+        DRONE_GCN_CHECK(drone_spmm_plan_create_scaled(&planT, n, n, nnz, rpT, ciT, valT, in_scale, out_scale, max_dim, s));
+        (void)hipFree(out_scale);
+        (void)hipFree(in_scale);
     }
     Adjacency(const Adjacency &) = delete;
     ~Adjacency()

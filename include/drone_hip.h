@@ -218,12 +218,29 @@ int drone_csr_transpose_f32(int n_rows, int n_cols, int64_t nnz, const int *rp, 
 typedef struct drone_spmm_plan drone_spmm_plan;
 int drone_spmm_plan_create(drone_spmm_plan **plan, int n_rows, int n_cols, int64_t nnz, const int *rp,
                            const int *ci, const float *v, int max_k, drone_stream_t stream);
+/* The same for a matrix whose values are row_scale[row] * col_scale[col] on a 0/1 pattern - what every normalised
+ * adjacency of cuda_gcn is (cuda_kernel.cu:145-155: 1 / sqrtf(outDegree[u] * in_degree[v]); drone_gcn_degree_scales
+ * makes the two factors).  v is still passed and still used by the band pieces and the short rows; the dense part is
+ * then kept as one BIT per cell over a much larger region (any 4096-row x 2048-column chunk where it pays), and
+ * multiplied on the matrix cores against col_scale .* B written as the exact sum of three bf16 numbers per element, with
+ * fp32 accumulation; rows are scaled by row_scale when the result is added into C.  Creation checks every entry
+ * against the scales (relative 4e-6) and every dense cell for holding one entry only; a matrix that fails either
+ * check gets the plan drone_spmm_plan_create would have built.  drone_spmm_plan_update_values refuses a plan that
+ * holds bits.  No counterpart in the reference: cusparseSpMM does not know the values' structure. */
+int drone_spmm_plan_create_scaled(drone_spmm_plan **plan, int n_rows, int n_cols, int64_t nnz, const int *rp,
+                                  const int *ci, const float *v, const float *row_scale, const float *col_scale,
+                                  int max_k, drone_stream_t stream);
+/* out[i] = 1 / sqrtf(degree[i]) (0 for degree 0): the factors of drone_gcn_edge_values' values. */
+int drone_gcn_degree_scales(int n, const int *degree, float *out, drone_stream_t stream);
 int drone_spmm_plan_update_values(drone_spmm_plan *plan, const float *v, drone_stream_t stream);
 int drone_spmm_plan_destroy(drone_spmm_plan *plan);
 /* What the plan decided: entries in rows longer than 512, entries moved to dense rectangles, the cells of those
  * rectangles, and the rows / columns (in rank order) the rectangles span.  Any output may be NULL. */
 int drone_spmm_plan_info(const drone_spmm_plan *plan, int64_t *long_nnz, int64_t *dense_nnz, int64_t *dense_cells,
                          int *dense_rows, int *dense_cols);
+/* The part of the dense region that a scaled plan keeps as bits: its cells, ranked rows and ranked columns (all 0 for a
+ * plan without one; drone_spmm_plan_info counts the same entries and cells under "dense").  Any output may be NULL. */
+int drone_spmm_plan_bit_core(const drone_spmm_plan *plan, int64_t *cells, int *rows, int *cols);
 /* cusparseSpMM(NON_TRANSPOSE, NON_TRANSPOSE, alpha, A, B, beta, C, ALG_DEFAULT) at cuda_module.cu:245
  * (forward: A = transposed CSR) and :335 (backward: A = original CSR):
  * C[n_rows x K] = alpha * A * B + beta * C. */

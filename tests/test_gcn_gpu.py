@@ -355,6 +355,104 @@ def test_spmm_dense_core_matches_oracle(T, oracle):
     plan.close()
 
 
+def _core_graph(rng, n, core, density, extra, duplicates=0):
+    """A directed pattern: a `core`-vertex block of the given density scattered inside n vertices, `extra` random
+    entries, optionally some entries of the block stored twice.  Returns rp, cols and the in-/out-degrees (counted over
+    the stored entries, as a loader would)."""
+    perm = rng.permutation(n)
+    r, c = np.nonzero(rng.random((core, core)) < density)
+    rs, cs = rng.integers(0, n, extra), rng.integers(0, n, extra)
+    key = np.unique(np.concatenate([perm[r].astype(np.int64) * n + perm[c], rs * n + cs]))
+    if duplicates:
+        key = np.sort(np.concatenate([key, (perm[r[:duplicates]].astype(np.int64) * n + perm[c[:duplicates]])]))
+    rows, cols = (key // n).astype(np.int32), (key % n).astype(np.int32)
+    rp = np.zeros(n + 1, np.int32)
+    rp[1:] = np.cumsum(np.bincount(rows, minlength=n))
+    out_deg = np.diff(rp).astype(np.int32)
+    in_deg = np.bincount(cols, minlength=n).astype(np.int32)
+    return rp, cols, in_deg, out_deg
+
+
+def test_spmm_scaled_pattern_bit_core_matches_oracle(T, oracle):
+    """drone_spmm_plan_create_scaled on a normalised adjacency with a dense core: the core is kept as bits and multiplied
+    on the matrix cores against the scaled operand split into three bf16 parts.  Checked element by element against
+    the fp64-accumulated oracle on the reference's edge values (1e-4 of sum |a||b|), for one and two 128-column
+    passes, widths that do not fill a tile, padded leading dimensions, alpha / beta, and the transposed matrix."""
+    from drone_amd import gcn
+    rng = np.random.default_rng(33)
+    n = 12000
+    rp, cols, in_deg, out_deg = _core_graph(rng, n, 6000, 0.8, 60000)
+    d_rp, d_ci = dev(T, rp), dev(T, cols)
+    d_val = gcn.edge_values(d_rp, d_ci, dev(T, in_deg), dev(T, out_deg))
+    val = d_val.cpu().numpy()
+    np.testing.assert_array_equal(val, oracle.edge_values(rp, cols, in_deg, out_deg))
+    r_scale, c_scale = gcn.degree_scales(dev(T, out_deg)), gcn.degree_scales(dev(T, in_deg))
+    plan = gcn.SpmmPlan(d_rp, d_ci, d_val, n, max_k=200, row_scale=r_scale, col_scale=c_scale)
+    core = plan.bit_core()
+    assert core["rows"] >= 6000 and core["cols"] >= 4096 and core["cells"] >= 6000 * 4096
+    assert plan.info()["dense_nnz"] > 20_000_000 and plan.info()["dense_cells"] == core["cells"]
+    absval = np.abs(val)
+    for K, pad in ((128, 0), (200, 0), (41, 3), (7, 1), (64, 0), (65, 0)):
+        B = rng.uniform(-1, 1, (n, K)).astype(np.float32) * rng.choice([1e-6, 1.0, 1e5], size=(1, K)).astype(np.float32)
+        want = oracle.spmm_f64acc(rp, cols, val, B).astype(np.float64)
+        scale = oracle.spmm_f64acc(rp, cols, absval, np.abs(B)).astype(np.float64)
+        Bd = T.zeros((n, K + pad), dtype=T.float32, device="cuda")
+        Bd[:, :K] = dev(T, B)
+        out = T.full((n, K + pad), 7.0, dtype=T.float32, device="cuda")
+        gcn.spmm(plan, d_rp, d_ci, d_val, Bd[:, :K], K=K, out=out[:, :K])
+        res = out.cpu().numpy()
+        assert rel_err(res[:, :K], want, scale) <= 1e-4
+        if pad:
+            assert np.all(res[:, K:] == 7.0)                       # nothing written past K
+        C0 = rng.uniform(-1, 1, (n, K)).astype(np.float32)
+        out = dev(T, C0)
+        gcn.spmm(plan, d_rp, d_ci, d_val, Bd[:, :K], K=K, out=out, alpha=0.5, beta=-2.0)
+        ref = 0.5 * want - 2.0 * C0
+        assert rel_err(out.cpu().numpy(), ref, 0.5 * scale + 2.0 * np.abs(C0)) <= 1e-4
+    a = gcn.spmm(plan, d_rp, d_ci, d_val, Bd[:, :K], K=K)
+    b = gcn.spmm(plan, d_rp, d_ci, d_val, Bd[:, :K], K=K)
+    assert T.equal(a, b)                                           # repeatable bit for bit
+    with pytest.raises(Exception, match="fixed by the scales"):
+        plan.update_values(d_val)
+    plan.close()
+    # the transposed matrix: rows scale with the in-degree, columns with the out-degree
+    rpT, ciT, vT = gcn.csr_transpose(n, n, d_rp, d_ci, d_val)
+    planT = gcn.SpmmPlan(rpT, ciT, vT, n, max_k=128, row_scale=c_scale, col_scale=r_scale)
+    assert planT.bit_core()["cells"] > 0
+    G = rng.uniform(-1, 1, (n, 128)).astype(np.float32)
+    m = sp.csr_matrix((val.astype(np.float64), cols, rp), shape=(n, n))
+    want = m.T @ G.astype(np.float64)
+    scale = abs(m).T @ np.abs(G).astype(np.float64)
+    got = gcn.spmm(planT, rpT, ciT, vT, dev(T, G)).cpu().numpy()
+    assert rel_err(got, want, scale) <= 1e-4
+    planT.close()
+
+
+def test_spmm_scaled_plan_falls_back(T, oracle):
+    """Scales that do not reproduce the values, or a pattern that stores a dense cell twice, cannot be kept as bits:
+    creation then builds the ordinary plan (fp32 rectangles) and the product is still right."""
+    from drone_amd import gcn
+    rng = np.random.default_rng(34)
+    n = 9000
+    for duplicates in (0, 500):
+        rp, cols, in_deg, out_deg = _core_graph(rng, n, 5000, 0.7, 30000, duplicates=duplicates)
+        d_rp, d_ci = dev(T, rp), dev(T, cols)
+        d_val = gcn.edge_values(d_rp, d_ci, dev(T, in_deg), dev(T, out_deg))
+        r_scale, c_scale = gcn.degree_scales(dev(T, out_deg)), gcn.degree_scales(dev(T, in_deg))
+        if not duplicates:
+            r_scale = r_scale * 1.001                              # off by more than rounding
+        plan = gcn.SpmmPlan(d_rp, d_ci, d_val, n, max_k=128, row_scale=r_scale, col_scale=c_scale)
+        assert plan.bit_core()["cells"] == 0 and plan.info()["dense_nnz"] > 0
+        val = d_val.cpu().numpy()
+        B = rng.uniform(-1, 1, (n, 128)).astype(np.float32)
+        want = oracle.spmm_f64acc(rp, cols, val, B).astype(np.float64)
+        scale = oracle.spmm_f64acc(rp, cols, np.abs(val), np.abs(B)).astype(np.float64)
+        got = gcn.spmm(plan, d_rp, d_ci, d_val, dev(T, B)).cpu().numpy()
+        assert rel_err(got, want, scale) <= 1e-4
+        plan.update_values(d_val)                                  # allowed again: the plan holds no bits
+        plan.close()
+
+
 def _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, row_sums, dense=None):
     """Size-independent checks of C = A * B at a benchmark shape: A * 1 against fp64 row sums, adjointness
     <A X, Y> = <X, A^T Y> with the separately built transpose, agreement with the vendor's sparse product on a
