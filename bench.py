@@ -193,14 +193,19 @@ def bench_gcn_step(steps, warmup, cpu_baseline=False):
     # the four SpMMs of the step, timed alone on operands of the same shape
     rp, ci = g["rp"], g["ci"]
     val = gcn.edge_values(rp, ci, g["deg"], g["deg"])
-    plan = gcn.SpmmPlan(rp, ci, val, N, max_k=HID)
-    kernels = []
+    # as the model builds them: the values are 1/sqrt(deg[row]) * 1/sqrt(deg[col]), so the dense region is kept as bits
+    scale = gcn.degree_scales(g["deg"])
+    plan = gcn.SpmmPlan(rp, ci, val, N, max_k=HID, row_scale=scale, col_scale=scale)
+    plain = gcn.SpmmPlan(rp, ci, val, N, max_k=HID)          # what an arbitrary-valued matrix gets: fp32 rectangles
+    kernels, plain_ms = [], {}
     for K, ld in ((HID, HID), (CLS, 44)):
         B = torch.rand((N, ld), device="cuda") * 2 - 1
         out = torch.empty((N, ld), device="cuda")
         ms = time_call(lambda: gcn.spmm(plan, rp, ci, val, B[:, :K], K=K, out=out[:, :K]), reps=5)
-        kernels.append(spmm_report(f"spmm (rows + band pieces + dense core) K={K} ld={ld}", N, nnz, K, ms))
-    plan_info = plan.info()
+        kernels.append(spmm_report(f"spmm (rows + band pieces + bit core) K={K} ld={ld}", N, nnz, K, ms))
+        plain_ms[f"K={K}"] = time_call(lambda: gcn.spmm(plain, rp, ci, val, B[:, :K], K=K, out=out[:, :K]), reps=5)
+    plan_info = dict(plan.info(), bit_core=plan.bit_core(), unscaled_plan=plain.info(), unscaled_plan_ms=plain_ms)
+    plain.close()
     spmm_ms = 2 * sum(k["ms"] for k in kernels[:2])
     spmm_bytes = 2 * sum(k["algorithmic_bytes"] for k in kernels[:2])
     gemms = []
@@ -263,7 +268,9 @@ def bench_gcn_layer(cpu_baseline=False):
     T1 = torch.empty((N, K), device="cuda")
     out = torch.empty((N, K), device="cuda")
     mask = torch.empty((N, K), dtype=torch.uint8, device="cuda")
-    plan = gcn.SpmmPlan(g["rp"], g["ci"], val, N, max_k=K)
+    scale = gcn.degree_scales(g["deg"])
+    plan = gcn.SpmmPlan(g["rp"], g["ci"], val, N, max_k=K, row_scale=scale, col_scale=scale)
+    plan_info = dict(plan.info(), bit_core=plan.bit_core())
 
     def layer():
         gcn.sgemm(0, 0, H, W, out=T1)
@@ -280,7 +287,8 @@ def bench_gcn_layer(cpu_baseline=False):
     log(f"GCN layer (configs[2]): {ms:.2f} ms, SpMM {ms_spmm:.2f} ms, GEMM {ms_gemm:.2f} ms" +
         (f"; CPU SpMM {cpu['value']:.0f} ms on {cpu['cores']} threads" if cpu else ""))
     return {"workload": f"GCN layer forward (configs[2]): R-MAT scale 20 undirected + self-loops, N={N}, nnz={nnz}, K=128",
-            "layer_ms": ms, "spmm": spmm_report("spmm (rows + band pieces + dense core) K=128", N, nnz, K, ms_spmm),
+            "layer_ms": ms, "spmm": spmm_report("spmm (rows + band pieces + bit core) K=128", N, nnz, K, ms_spmm),
+            "spmm_plan": plan_info,
             "gemm_ms": ms_gemm, "gemm_tflops": 2.0 * N * K * K / (ms_gemm * 1e-3) / 1e12,
             "gemm_frac_of_fp32_mfma_peak": 2.0 * N * K * K / (ms_gemm * 1e-3) / 1e12 / 157.3, "cpu_baseline_spmm": cpu}
 
@@ -297,16 +305,19 @@ def bench_spmm_sweep(cpu_baseline=False):
     deg = (rp[1:] - rp[:-1]).clamp(min=1)
     val = (1.0 / torch.repeat_interleave(deg.float(), (rp[1:] - rp[:-1]).long())).contiguous()
     rpT, ciT, vT = gcn.csr_transpose(N, N, rp, ci, val)
+    inv_deg, ones = (1.0 / deg.float()).contiguous(), torch.ones(N, device="cuda")   # val = inv_deg[row] * 1
     out = {"workload": f"SpMM sweep (configs[4]): R-MAT scale 22 ef 32 skewed, N={N}, nnz={nnz}, max row "
                        f"{int((rp[1:]-rp[:-1]).max())}, max transposed row {int((rpT[1:]-rpT[:-1]).max())}", "kernels": []}
     for K in (16, 64, 256):
         H = torch.rand((N, K), device="cuda") * 2 - 1
         C_ = torch.empty((N, K), device="cuda")
-        for name, (a, b, c) in (("forward A*H", (rp, ci, val)), ("transpose A^T*G", (rpT, ciT, vT))):
-            plan = gcn.SpmmPlan(a, b, c, N, max_k=K)
+        for name, (a, b, c, rs, cs) in (("forward A*H", (rp, ci, val, inv_deg, ones)),
+                                        ("transpose A^T*G", (rpT, ciT, vT, ones, inv_deg))):
+            plan = gcn.SpmmPlan(a, b, c, N, max_k=K, row_scale=rs, col_scale=cs)
             ms = time_call(lambda: gcn.spmm(plan, a, b, c, H, out=C_), reps=5)
+            info = dict(plan.info(), bit_core=plan.bit_core())
             plan.close()
-            out["kernels"].append(spmm_report(f"{name} K={K}", N, nnz, K, ms))
+            out["kernels"].append(dict(spmm_report(f"{name} K={K}", N, nnz, K, ms), plan=info))
             log(f"SpMM sweep (configs[4]) {name} K={K}: {ms:.2f} ms = {out['kernels'][-1]['frac_of_hbm_peak']*100:.1f} % of "
                 f"the HBM roofline")
         del H, C_

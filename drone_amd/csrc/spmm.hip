@@ -101,12 +101,20 @@ constexpr double kGatherMsPerEntry = 0.19e-9;  // band-piece kernel: 24 ps per e
 constexpr double kDenseMsPerCell = 0.025e-9;   // dense product: 3.2 ps per cell at K = 128
 constexpr double kDenseMinGainMs = 0.25;
 // Scaled patterns (bit core): row groups of 4096 ranked long rows each, any leading set of 2048-column chunks.
-// Costs per cell of one 32-wide feature tile and per gathered entry of feature width 1, measured on the 232,965-vertex /
-// 229 M-entry graph.
+// Cost per cell of one 32-wide feature tile, measured on the 232,965-vertex / 229 M-entry graph (0.53 ps per cell at 128
+// feature columns); the gathers it replaces are priced as for the fp32 rectangles.  Pricing a gather at 1.4 / 1.8 / 2.6
+// times that (which grows the bit region from 1.24 to 1.87 / 2.09 / 2.17 G cells and takes 177 -> 190 / 193 / 194 M of
+// the 229 M entries) left the product where it was, 2.9 ms at 128 columns: what remains outside is priced by its number
+// of band pieces rather than by its entries.
 constexpr int kBitMaxChunks = 128;      // columns considered: the 262,144 most frequent
 constexpr int kBitGroupRows = 4096;
 constexpr int kBitMaxGroups = 1024;
-constexpr double kBitMsPerCellTile = 0.15e-9;   // ms: 0.15 ps per cell and 32 feature columns
+// Entries a band piece should hold where a row has few left outside the bits (band_keys_kernel merges such a row's bands).
+// ms for 128 / 41 feature columns on the 229 M-entry graph: 0 (no merging) 2.89 / 1.56, 16: 2.88 / 1.56, 32: 2.90 / 1.44,
+// 64: 3.30 / 1.38, 128: 3.60 / 1.51 - at 128 columns a merged band no longer fits an XCD's L2, and that costs more than
+// the short pieces do.
+constexpr int kBitMinPiece = 32;
+constexpr double kBitMsPerCellTile = 0.135e-9;  // ms: 0.135 ps per cell and 32 feature columns
 static_assert(kDenseMaxCols / kDenseChunk <= kBitMaxChunks, "the density histogram keeps at most 128 chunks per wavefront");
 
 template <int VEC> struct VecT;
@@ -464,16 +472,27 @@ __global__ __launch_bounds__(256) void band_keys_kernel(int num_long, const int 
                                                         const int *__restrict__ ci,
                                                         const unsigned char *__restrict__ band_of_col, int num_bands,
                                                         const int *__restrict__ dense_width_of_long,
-                                                        const int *__restrict__ col_rank,
+                                                        const int *__restrict__ col_rank, int min_piece,
                                                         unsigned *__restrict__ keys, unsigned *__restrict__ idx)
 {
     const int lane = threadIdx.x & (kWave - 1);
     for (int i = (blockIdx.x * blockDim.x + threadIdx.x) / kWave; i < num_long; i += gridDim.x * blockDim.x / kWave) {
         const int r = long_row[i], e0 = rp[r], len = rp[r + 1] - e0, o = long_offset[i];
         const int w = dense_width_of_long[i];
+        // min_piece > 0: a row that keeps few entries outside its dense part has its bands merged in aligned groups of
+        // `merge` (a power of two), so that its pieces hold about min_piece entries or more - a piece is a chain of
+        // dependent round trips however short it is, and what is left of such a row no longer fills 21 of them.
+        unsigned merge = 1;
+        if (min_piece > 0) {
+            int left = 0;
+            for (int k = lane; k < len; k += kWave) left += col_rank[ci[e0 + k]] >= w;
+#pragma unroll
+            for (int off = kWave / 2; off > 0; off >>= 1) left += __shfl_xor(left, off, kWave);
+            while (merge < 32 && (int64_t)left * merge < (int64_t)min_piece * num_bands) merge <<= 1;
+        }
         for (int k = lane; k < len; k += kWave) {
             const int c = ci[e0 + k];
-            const unsigned band = col_rank[c] < w ? (unsigned)num_bands : (unsigned)band_of_col[c];
+            const unsigned band = col_rank[c] < w ? (unsigned)num_bands : (unsigned)band_of_col[c] & ~(merge - 1);
             keys[o + k] = band * (unsigned)num_long + (unsigned)i;
             idx[o + k] = (unsigned)(e0 + k);
         }
@@ -713,7 +732,7 @@ int build_band_pieces(drone_spmm_plan *p, const std::vector<int> &h_rp, const st
         DRONE_HIP_TRY(hipMemcpyAsync(d_dense_width, dense_width_of_long.data(), sizeof(int) * (size_t)num_long, hipMemcpyHostToDevice, s));
         // 2. stable sort of the long rows' entries by (band, row); dense entries sort behind every band
         band_keys_kernel<<<kb, 256, 0, s>>>(num_long, p->long_row, d_long_offset, rp, ci, band_of_col, num_bands,
-                                            d_dense_width, p->col_rank, keys, idx);
+                                            d_dense_width, p->col_rank, p->scaled ? kBitMinPiece : 0, keys, idx);
         DRONE_HIP_TRY(rocprim::radix_sort_pairs(temp, temp_bytes, keys, keys_sorted, idx, p->perm, ln, 0, key_bits, s));
         gather_sorted_kernel<<<4096, 256, 0, s>>>(long_nnz, p->perm, ci, v, p->ci2, p->val2);
         // 3. runs of equal key = (band, row) pieces

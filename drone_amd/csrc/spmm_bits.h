@@ -16,7 +16,7 @@
 
 namespace drone {
 
-constexpr int kBitTileRows = 512;   // rows of one tile (one work-group: 4 x 2 wavefronts of 128 rows x half the feature columns)
+constexpr int kBitTileRows = 512;   // rows of one tile (one work-group: 8 wavefronts x 64 rows)
 constexpr int kBitBlockCols = 256;  // columns per bit block: 16 bytes per lane, 16 steps of 16 columns
 
 struct BitCore {

@@ -97,15 +97,20 @@ __device__ __forceinline__ bf16x8 expand_bits(unsigned byte)
     return __builtin_bit_cast(bf16x8, v);
 }
 
-// One work-group (8 wavefronts) per unit: T[512 x 64 CT] = bits(512 x [c0, c1)) * split([c0, c1) x 64 CT), the three
-// parts summed.  Wavefront w owns rows 128 (w / 2) .. + 128 and feature tiles CT (w % 2) .. + CT as 4 x CT accumulators
-// of 32 x 32, so a 16-byte LDS read of the split operand feeds four matrix instructions.  The split operand of 32
-// columns (a stage: 4 groups x 3 parts x 2 CT tiles x 512 bytes) goes through LDS, double buffered, fetched one stage
-// ahead; the bits come straight from global memory, one 256-column block ahead.
+// One work-group (8 wavefronts) per unit: T[512 x 32 NT] = bits(512 x [c0, c1)) * split([c0, c1) x 32 NT), the three
+// parts summed.  Wavefront w owns rows 64 w .. + 64 and all NT feature tiles as 2 x NT accumulators of 32 x 32.  The
+// split operand of 32 columns (a stage: 4 groups x 3 parts x NT tiles x 512 bytes) goes through LDS, double buffered,
+// fetched one stage ahead; the bits come straight from global memory, one 256-column block ahead.
 // Measured on 1.14 G cells with 128 feature columns (ms): matrix instructions alone 0.46 (1.9 PFLOP/s), with the LDS
-// reads 0.52; work-groups of 4 wavefronts x 64 rows x 128 feature columns, two per CU, took 1.12 with the staging
-// through LDS - 64 bytes read and 32 written per clock and CU are more than the LDS delivers next to the matrix cores.
-template <int CT>
+// reads 0.52.  What it took to get near that:
+//  * work-groups of 512 rows, one per CU: with 256 rows and two per CU the split operand is staged twice as often,
+//    and 64 bytes read plus 32 written per clock and CU are more than the LDS delivers next to the matrix cores (1.12);
+//  * launch order by column range with a per-tile starting block (see bit_core_create and `rot`): 1.00 -> 0.84;
+//  * the stage's global loads issued by hand at the top of the stage (see below): 0.83 -> 0.61;
+//  * a wavefront expands a byte of bits into 8 bf16 values with 16 vector instructions, so every expansion must feed
+//    many matrix instructions: 2 row groups x NT tiles per wavefront (an expansion per 3 NT instructions) instead of
+//    4 x NT / 2 (one per 1.5 NT).
+template <int NT>
 __global__ __launch_bounds__(512, 1) void bits_mfma_kernel(const int *__restrict__ unit_tile,
                                                            const int *__restrict__ unit_c0,
                                                            const int *__restrict__ unit_c1,
@@ -115,15 +120,13 @@ __global__ __launch_bounds__(512, 1) void bits_mfma_kernel(const int *__restrict
                                                            const uint4 *__restrict__ bits,
                                                            const uint4 *__restrict__ split, float *__restrict__ partial)
 {
-    constexpr int NT = 2 * CT;
     constexpr int kStageVecs = 4 * 3 * NT * 32;
     constexpr int kPre = (kStageVecs + 511) / 512;
     __shared__ uint4 s_b[2][kStageVecs];
     const int u = blockIdx.x, tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-    const int wr = wave >> 1, wc = wave & 1;
     const int tile = unit_tile[u], c0 = unit_c0[u], c1 = unit_c1[u];
     const int blocks = tile_blocks[tile], nblocks = (c1 - c0) / kBitBlockCols;
-    const uint4 *w0 = bits + tile_off[tile] + ((size_t)(4 * wr) * blocks + c0 / kBitBlockCols) * 64 + lane;
+    const uint4 *w0 = bits + tile_off[tile] + ((size_t)(2 * wave) * blocks + c0 / kBitBlockCols) * 64 + lane;
     const size_t wstep = (size_t)blocks * 64;
     const uint4 *src = split + (size_t)(c0 / 8) * kGroupVecs;
     int goff[kPre];
@@ -133,11 +136,11 @@ __global__ __launch_bounds__(512, 1) void bits_mfma_kernel(const int *__restrict
         const int g = v / (3 * NT * 32), rem = v % (3 * NT * 32);
         goff[i] = g * kGroupVecs + (rem / (NT * 32)) * 4 * 32 + ((rem / 32) % NT) * 32 + rem % 32;
     }
-    f32x16 acc[4][CT];
+    f32x16 acc[2][NT];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < CT; ++j)
+        for (int j = 0; j < NT; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
@@ -145,9 +148,9 @@ __global__ __launch_bounds__(512, 1) void bits_mfma_kernel(const int *__restrict
     // The work-groups resident at one time share a column range (launch order) and would walk it in step, all asking
     // one L2 channel for the same line at the same moment: every tile starts at its own block of the range and wraps.
     const int rot = (tile * 5) % nblocks;
-    uint4 a[4], an[4];
+    uint4 a[2], an[2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) a[i] = w0[i * wstep + (size_t)rot * 64];
+    for (int i = 0; i < 2; ++i) a[i] = w0[i * wstep + (size_t)rot * 64];
     {
         const uint4 *first = src + (size_t)rot * 32 * kGroupVecs;
 #pragma unroll
@@ -162,10 +165,10 @@ __global__ __launch_bounds__(512, 1) void bits_mfma_kernel(const int *__restrict
         const int block = kb + rot < nblocks ? kb + rot : kb + rot - nblocks;
         const int block_next = block + 1 < nblocks ? block + 1 : 0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) an[i] = w0[i * wstep + (size_t)block_next * 64];
-        unsigned aw[4][4];
+        for (int i = 0; i < 2; ++i) an[i] = w0[i * wstep + (size_t)block_next * 64];
+        unsigned aw[2][4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 2; ++i) {
             aw[i][0] = a[i].x;
             aw[i][1] = a[i].y;
             aw[i][2] = a[i].z;
@@ -174,55 +177,52 @@ __global__ __launch_bounds__(512, 1) void bits_mfma_kernel(const int *__restrict
 #pragma unroll
         for (int st = 0; st < 8; ++st) {
             const bool more = kb + 1 < nblocks || st < 7;
-#ifndef BITS_EXP_NOGLOBAL
             if (more) {
+                // Issued by hand: written as plain loads, the compiler sinks them to the LDS stores at the end of the
+                // stage (or loads twice) and the whole memory latency is waited for, stage after stage.  The matching
+                // wait is the s_waitcnt below; extra loads in flight only make the compiler's own waits stricter.
                 const uint4 *next = src + (size_t)(st < 7 ? block * 8 + st + 1 : block_next * 8) * 4 * kGroupVecs;
 #pragma unroll
                 for (int i = 0; i < kPre; ++i)
-                    if (tid + 512 * i < kStageVecs) pre[i] = next[goff[i]];
+                    if (tid + 512 * i < kStageVecs)
+                        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(pre[i]) : "v"(next + goff[i]) : "memory");
             }
-#endif
             const uint4 *cur = s_b[st & 1];
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
                 const int idx = st * 2 + ks;
-                bf16x8 A[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) A[i] = expand_bits((aw[i][idx / 4] >> ((idx % 4) * 8)) & 0xFFu);
+                const bf16x8 A0 = expand_bits((aw[0][idx / 4] >> ((idx % 4) * 8)) & 0xFFu);
+                const bf16x8 A1 = expand_bits((aw[1][idx / 4] >> ((idx % 4) * 8)) & 0xFFu);
 #pragma unroll
                 for (int part = 0; part < 3; ++part)
 #pragma unroll
-                    for (int ct = 0; ct < CT; ++ct) {
-                        const uint4 raw = cur[(((2 * ks + (lane >> 5)) * 3 + part) * NT + wc * CT + ct) * 32 + (lane & 31)];
+                    for (int ct = 0; ct < NT; ++ct) {
+                        const uint4 raw = cur[(((2 * ks + (lane >> 5)) * 3 + part) * NT + ct) * 32 + (lane & 31)];
                         const bf16x8 bv = __builtin_bit_cast(bf16x8, raw);
-#pragma unroll
-                        for (int i = 0; i < 4; ++i)
-                            acc[i][ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[i], bv, acc[i][ct], 0, 0, 0);
+                        acc[0][ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A0, bv, acc[0][ct], 0, 0, 0);
+                        acc[1][ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A1, bv, acc[1][ct], 0, 0, 0);
                     }
             }
-#ifndef BITS_EXP_NOSTORE
             if (more) {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
                 for (int i = 0; i < kPre; ++i)
                     if (tid + 512 * i < kStageVecs) s_b[(st & 1) ^ 1][tid + 512 * i] = pre[i];
             }
-#endif
-#ifndef BITS_EXP_NOSYNC
             __syncthreads();
-#endif
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) a[i] = an[i];
+        for (int i = 0; i < 2; ++i) a[i] = an[i];
     }
     float *out = partial + (size_t)unit_slot[u] * kBitTileRows * kPartialLd;
 #pragma unroll
-    for (int rt = 0; rt < 4; ++rt)
+    for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct)
+        for (int ct = 0; ct < NT; ++ct)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int row = 128 * wr + 32 * rt + (r / 4) * 8 + (lane >> 5) * 4 + (r % 4);
-                out[(size_t)row * kPartialLd + 32 * (wc * CT + ct) + (lane & 31)] = acc[rt][ct][r];
+                const int row = 64 * wave + 32 * rt + (r / 4) * 8 + (lane >> 5) * 4 + (r % 4);
+                out[(size_t)row * kPartialLd + 32 * ct + (lane & 31)] = acc[rt][ct][r];
             }
 }
 
@@ -356,10 +356,10 @@ int bit_core_multiply(const BitCore *bc, const unsigned *col_order, const float 
         const uint4 *split = bc->split + (size_t)pass * groups * kGroupVecs;
         float *partial = bc->partial + (size_t)pass * bc->num_units * kBitTileRows * kPartialLd;
         if (width <= 64)
-            bits_mfma_kernel<1><<<bc->num_units, 512, 0, s>>>(bc->unit_tile, bc->unit_c0, bc->unit_c1, bc->unit_slot,
+            bits_mfma_kernel<2><<<bc->num_units, 512, 0, s>>>(bc->unit_tile, bc->unit_c0, bc->unit_c1, bc->unit_slot,
                                                              bc->tile_blocks, bc->tile_off, bc->bits, split, partial);
         else
-            bits_mfma_kernel<2><<<bc->num_units, 512, 0, s>>>(bc->unit_tile, bc->unit_c0, bc->unit_c1, bc->unit_slot,
+            bits_mfma_kernel<4><<<bc->num_units, 512, 0, s>>>(bc->unit_tile, bc->unit_c0, bc->unit_c1, bc->unit_slot,
                                                              bc->tile_blocks, bc->tile_off, bc->bits, split, partial);
     }
     int grid = (int)ceil_div(bc->rows, 4);

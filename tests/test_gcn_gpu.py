@@ -453,14 +453,18 @@ def test_spmm_scaled_plan_falls_back(T, oracle):
         plan.close()
 
 
-def _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, row_sums, dense=None):
+def _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, row_sums, dense=None, scales=None):
     """Size-independent checks of C = A * B at a benchmark shape: A * 1 against fp64 row sums, adjointness
     <A X, Y> = <X, A^T Y> with the separately built transpose, agreement with the vendor's sparse product on a
-    column sample, and a repeatable result."""
-    plan = gcn.SpmmPlan(rp, ci, val, N, max_k=K)
-    planT = gcn.SpmmPlan(rpT, ciT, vT, N, max_k=K)
-    if dense is not None:                      # whether the plans moved part of the matrix to dense rectangles
+    column sample, and a repeatable result.  scales = (row_scale, col_scale) of A: the plans are then the scaled-pattern
+    plans the module layer builds (bits where the matrix is dense enough), with the factors swapped for A^T."""
+    rs, cs = scales if scales is not None else (None, None)
+    plan = gcn.SpmmPlan(rp, ci, val, N, max_k=K, row_scale=rs, col_scale=cs)
+    planT = gcn.SpmmPlan(rpT, ciT, vT, N, max_k=K, row_scale=cs, col_scale=rs)
+    if dense is not None:                      # whether the plans moved part of the matrix to a dense representation
         assert (plan.info()["dense_nnz"] > 0) == dense and (planT.info()["dense_nnz"] > 0) == dense
+        assert (plan.bit_core()["cells"] > 0) == (dense and scales is not None)
+        assert (planT.bit_core()["cells"] > 0) == (dense and scales is not None)
     ones = torch.ones((N, 4), device="cuda")
     got = gcn.spmm(plan, rp, ci, val, ones)
     assert float(((got[:, 0].double() - row_sums).abs() / row_sums.abs().clamp(min=1e-30)).max()) <= 1e-4
@@ -505,7 +509,10 @@ def test_full_size_properties_config3(T):
     rpT, ciT, vT = gcn.csr_transpose(N, N, rp, ci, val)
     assert torch.equal(rpT, rp) and torch.equal(ciT, ci) and torch.equal(vT, val)      # symmetric
     cs = torch.cat([torch.zeros(1, dtype=torch.float64, device="cuda"), torch.cumsum(val.double(), 0)])
-    _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, 128, cs[rp[1:].long()] - cs[rp[:-1].long()])
+    row_sums = cs[rp[1:].long()] - cs[rp[:-1].long()]
+    _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, 128, row_sums)
+    scale = gcn.degree_scales(deg)
+    _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, 128, row_sums, scales=(scale, scale))
 
 
 @pytest.mark.parametrize("K", [16, 64, 256])
@@ -525,3 +532,7 @@ def test_full_size_properties_config5(T, K):
     rpT, ciT, vT = gcn.csr_transpose(N, N, rp, ci, val)
     assert int(rpT[-1]) == x["nnz"] and int((ciT[1:] < ciT[:-1]).sum()) <= N          # rows ascending inside
     _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, (cnt > 0).double(), dense=(K == 256))
+    if K != 16:                                                     # the same with the plans told that val = 1/count[row] * 1
+        inv = (1.0 / cnt.clamp(min=1).float()).contiguous()
+        _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, (cnt > 0).double(),
+                                   scales=(inv, torch.ones(N, device="cuda")))

@@ -230,23 +230,13 @@ def test_training_reduces_loss_with_adam_and_eval_is_pure(T, oracle):
     m.close()
 
 
-def test_full_size_properties_config4(T):
-    """Fourth configuration at full size (232,965 vertices, ~229 M entries, 602 -> 128 -> 41): properties that
-    need no CPU oracle - A_hat * 1 against fp64 row sums, forward/backward adjointness <A^T X, Y> = <X, A Y>,
-    every element of four columns of the K = 41 and K = 128 products against the vendor's fp64 sparse product,
-    the big GEMMs against torch.matmul in fp32/fp64, and a bitwise repeatable, finite training step."""
-    torch = T
-    from drone_amd import gcn, graphs, rmat
-    N, FIN, HID, CLS = 232965, 602, 128, 41
-    g = graphs.gcn_graph_torch(18, 0, seed=4, n=N, n_edges=221_000_000)
-    rp, ci, deg, nnz = g["rp"], g["ci"], g["deg"], g["nnz"]
-    assert 110e6 < (nnz - N) / 2 < 120e6                      # ~114.6 M undirected edges, as the configuration says
-    val = gcn.edge_values(rp, ci, deg, deg)
-    rpT, ciT, vT = gcn.csr_transpose(N, N, rp, ci, val)
-    assert torch.equal(rpT, rp) and torch.equal(ciT, ci) and torch.equal(vT, val)      # symmetric graph
-    plan = gcn.SpmmPlan(rp, ci, val, N, max_k=HID)
+def _spmm_checks_config4(torch, gcn, N, HID, CLS, rp, ci, val, A64, degree_scale):
+    plan = gcn.SpmmPlan(rp, ci, val, N, max_k=HID, row_scale=degree_scale, col_scale=degree_scale)
     assert plan.info()["dense_nnz"] > 50_000_000           # the products below go through the dense core
-    A64 = torch.sparse_csr_tensor(rp.long(), ci.long(), val.double(), size=(N, N))
+    if degree_scale is not None:
+        assert plan.bit_core()["cells"] > 500_000_000 and plan.info()["dense_nnz"] > 150_000_000
+    else:
+        assert plan.bit_core()["cells"] == 0
     # A * ones == row sums (fp64 prefix sums as the reference value)
     ones = torch.ones((N, 4), device="cuda")
     got = gcn.spmm(plan, rp, ci, val, ones)
@@ -275,8 +265,28 @@ def test_full_size_properties_config4(T):
         ref = torch.sparse.mm(A64, X[:, cols].double().contiguous())
         mag = torch.sparse.mm(A64, X[:, cols].double().abs().contiguous())
         assert float(((AX[:, cols].double() - ref).abs() / mag.clamp(min=1e-30)).max()) <= 1e-4
-    del A64
     plan.close()
+
+
+def test_full_size_properties_config4(T):
+    """Fourth configuration at full size (232,965 vertices, ~229 M entries, 602 -> 128 -> 41): properties that
+    need no CPU oracle - A_hat * 1 against fp64 row sums, forward/backward adjointness <A^T X, Y> = <X, A Y>,
+    every element of four columns of the K = 41 and K = 128 products against the vendor's fp64 sparse product,
+    the big GEMMs against torch.matmul in fp32/fp64, and a bitwise repeatable, finite training step."""
+    torch = T
+    from drone_amd import gcn, graphs, rmat
+    N, FIN, HID, CLS = 232965, 602, 128, 41
+    g = graphs.gcn_graph_torch(18, 0, seed=4, n=N, n_edges=221_000_000)
+    rp, ci, deg, nnz = g["rp"], g["ci"], g["deg"], g["nnz"]
+    assert 110e6 < (nnz - N) / 2 < 120e6                      # ~114.6 M undirected edges, as the configuration says
+    val = gcn.edge_values(rp, ci, deg, deg)
+    rpT, ciT, vT = gcn.csr_transpose(N, N, rp, ci, val)
+    assert torch.equal(rpT, rp) and torch.equal(ciT, ci) and torch.equal(vT, val)      # symmetric graph
+    A64 = torch.sparse_csr_tensor(rp.long(), ci.long(), val.double(), size=(N, N))
+    scale_of = gcn.degree_scales(deg)
+    for scaled in (False, True):                             # fp32 rectangles / bits (what the model's plans hold)
+        _spmm_checks_config4(torch, gcn, N, HID, CLS, rp, ci, val, A64, scale_of if scaled else None)
+    del A64
     # the step's GEMM shapes against torch (fp64 reference on a row sample, fp32 on the whole)
     Xf = torch.from_numpy(rmat.normal_f32((N, FIN), seed=4)).cuda()
     W1 = torch.from_numpy(rmat.uniform_f32((FIN, HID), seed=41, lo=-0.09, hi=0.09)).cuda()
