@@ -179,20 +179,32 @@ __global__ __launch_bounds__(kThreads) void accuracy_kernel(int n, int classes, 
     }
 }
 
-// out[0] = sum of x[i]^2, accumulated in double by one work-group in a fixed order (weights are small)
-__global__ __launch_bounds__(kThreads) void sum_squares_kernel(const float *__restrict__ x, int64_t n,
-                                                               float *__restrict__ out)
+// out[0] = sum of x[i]^2, accumulated in double by one work-group of 1024 in a fixed order (weights are small).  Four
+// independent chains per thread: one chain of dependent loads and fp64 adds took 117 us for the 77,056 weights of a
+// 602 x 128 layer.
+__global__ __launch_bounds__(1024) void sum_squares_kernel(const float *__restrict__ x, int64_t n, float *__restrict__ out)
 {
-    __shared__ double s_part[kThreads];
-    double t = 0.0;
-    for (int64_t i = threadIdx.x; i < n; i += kThreads) t += (double)x[i] * (double)x[i];
-    s_part[threadIdx.x] = t;
-    __syncthreads();
-    for (int m = kThreads / 2; m > 0; m >>= 1) {
-        if (threadIdx.x < m) s_part[threadIdx.x] += s_part[threadIdx.x + m];
-        __syncthreads();
+    __shared__ double s_part[1024 / kWave];
+    double t[4] = {0.0, 0.0, 0.0, 0.0};
+    int64_t i = threadIdx.x;
+    for (; i + 3 * 1024 < n; i += 4 * 1024) {
+        const float a = x[i], b = x[i + 1024], c = x[i + 2 * 1024], d = x[i + 3 * 1024];
+        t[0] += (double)a * (double)a;
+        t[1] += (double)b * (double)b;
+        t[2] += (double)c * (double)c;
+        t[3] += (double)d * (double)d;
     }
-    if (threadIdx.x == 0) out[0] = (float)s_part[0];
+    for (; i < n; i += 1024) t[0] += (double)x[i] * (double)x[i];
+    double v = (t[0] + t[1]) + (t[2] + t[3]);
+#pragma unroll
+    for (int m = kWave / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, kWave);
+    if ((threadIdx.x & (kWave - 1)) == 0) s_part[threadIdx.x / kWave] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double total = 0.0;
+        for (int w = 0; w < 1024 / kWave; ++w) total += s_part[w];
+        out[0] = (float)total;
+    }
 }
 
 __global__ void sgd_kernel(float *__restrict__ w, const float *__restrict__ g, int64_t n, float lr)
@@ -305,7 +317,7 @@ extern "C" int drone_sum_squares_f32(const float *x, int64_t n, float *out, dron
 {
     clear_error();
     DRONE_REQUIRE(n >= 0 && (n == 0 || x) && out, "null operand");
-    sum_squares_kernel<<<1, kThreads, 0, as_stream(stream)>>>(x, n, out);
+    sum_squares_kernel<<<1, 1024, 0, as_stream(stream)>>>(x, n, out);
     DRONE_HIP_TRY(hipGetLastError());
     return DRONE_OK;
 }

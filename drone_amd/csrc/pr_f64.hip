@@ -315,7 +315,7 @@ extern "C" int drone_pr_run_f64(drone_pr_plan *p, double alpha, int iters, doubl
                 p->rows, p->nnz, p->mt.tile_row, p->rl.row_ptr, p->rl.col, epi, carry, p->ms.tile_stat);
         } else {
             pr_rowblock_kernel<PrF64Epi><<<p->rb.num_units, kRbThreads, kRbLdsBytes, s>>>(
-                p->rb.block_row, p->rb.block_nnz, p->rb.col, p->rb.lrow, p->rb.packed, p->rb.batch_base, p->rb.block_batch,
+                p->rb.block_row, p->rb.block_nnz, p->rb.col, p->rb.lrow, p->rb.stream, p->rb.batch_info, p->rb.block_batch,
                 p->rb.block_wide, p->rb.unit_block, p->rb.block_units, p->rb.block_unit0, p->rb.block_partial,
                 p->rb.partial, epi, carry, p->ms.tile_stat);
             if (p->rb.num_split > 0)

@@ -279,7 +279,7 @@ int aggregate_push(Graph *g, PRValues *values, hipStream_t s)
         PushF2 *carry = static_cast<PushF2 *>(x->ms_rb.tile_carry);
         PushF2 *partial = reinterpret_cast<PushF2 *>(rb.partial);
         pr_rowblock_kernel<PushEpi><<<rb.num_units, kRbThreads, kRbLdsBytes, s>>>(
-            rb.block_row, rb.block_nnz, rb.col, rb.lrow, rb.packed, rb.batch_base, rb.block_batch, rb.block_wide,
+            rb.block_row, rb.block_nnz, rb.col, rb.lrow, rb.stream, rb.batch_info, rb.block_batch, rb.block_wide,
             rb.unit_block, rb.block_units, rb.block_unit0, rb.block_partial, partial, epi, carry, x->ms_rb.tile_stat);
         if (rb.num_split > 0)
             pr_rowblock_merge_kernel<PushEpi><<<dim3((unsigned)rb.num_split, (unsigned)(kRbRows / kRbThreads + 1)), kRbThreads, 0, s>>>(

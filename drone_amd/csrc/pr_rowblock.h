@@ -46,11 +46,16 @@ struct RowBlocks {
     int32_t *walk_len = nullptr;    // device [num_blocks]
     int32_t *col = nullptr;         // device [nnz]: sources, ascending inside each block
     uint16_t *lrow = nullptr;       // device [nnz]: row of the entry relative to the block's first row
-    // Packed form, 4 bytes per entry instead of 6: entries of a block are taken 64 at a time (one wavefront
-    // load); batch_base holds the batch's first source and packed[e] = lrow << 16 | (source - base).  A block in
-    // which some batch spans more than 65,535 ids (sparse tail blocks) is flagged wide and read from col / lrow.
-    uint32_t *packed = nullptr;     // device [nnz]
-    int32_t *batch_base = nullptr;  // device [total batches]
+    // Compact form: entries of a block are taken 64 at a time (one wavefront load).  A batch stores its first source
+    // once and, per entry, the row relative to the block (15 bits) above the source's offset from that first source,
+    // in the narrowest of 2, 3 or 4 bytes per entry that holds the batch's largest offset (1, 9 or 17 bits).  The
+    // entries are sorted by source inside a block, so most batches span few sources: on R-MAT scale 24 the stream
+    // shrinks from 4 to about 3 bytes per entry.  batch_info[j] = {first source, (byte offset / 64) << 2 | (bytes per
+    // entry - 2)}; every batch starts on a 64-byte boundary of `stream`.  A block in which some batch spans 131,072 ids
+    // or more (sparse tail blocks) is flagged wide and read from col / lrow.
+    uint8_t *stream = nullptr;      // device: the batches' entries, 4 bytes of slack at the end
+    int2 *batch_info = nullptr;     // device [total batches]
+    int64_t stream_bytes = 0;
     int32_t *block_batch = nullptr; // device [num_blocks + 1]: first batch of the block
     int32_t *block_wide = nullptr;  // device [num_blocks]
     // Work units.  A block with many entries is swept by several work-groups, each taking every shares-th slice of
@@ -91,7 +96,7 @@ __device__ __forceinline__ double block_sum_1024(double v, double *s_red)
     return t;
 }
 
-// Adds the block's entries [e0, e1) into the LDS accumulators.  kWide reads the 6-byte layout, otherwise the packed
+// Adds the block's entries [e0, e1) into the LDS accumulators.  kWide reads the 6-byte layout, otherwise the compact
 // one.  Every wavefront sweeps its own contiguous slice of the (source-sorted) entries, 64 * kRbUnroll at a time.
 // With the 16 wavefronts interleaved at 64-entry granularity instead, neighbouring wavefronts ask for the same
 // popular line while its fill is still pending, and the L1 serialises them behind that fill (counters: the L1
@@ -125,6 +130,9 @@ __device__ __forceinline__ double block_sum_1024(double v, double *s_red)
 // for the whole superstep).
 // `live` is false for the clamped entries past a slice's end, which must add nothing.
 constexpr int kRbSpare = kRbRows + 7;                    // accumulator nobody reads
+constexpr int kRbRowBits = 15;                           // a block-local row is at most kRbRows (the row left open)
+static_assert(kRbRows < (1 << kRbRowBits), "block-local rows must fit the compact entries");
+typedef uint32_t RbUnalignedU32 __attribute__((aligned(1)));
 constexpr int kRbFlagWords = 4096;  // row i's bit: word i % 4096, bit i / 4096 (neighbouring rows in different words)
 __device__ __forceinline__ void rb_add(double *s_acc, uint32_t *, int l, bool live, double v)
 {
@@ -148,7 +156,7 @@ __device__ __forceinline__ void rb_read(const double *s_acc, const uint32_t *s_f
 template <bool kWide, typename Epi>
 __device__ __forceinline__ void rb_accumulate(int64_t block_begin, int64_t block_end, int share, int shares, int tid,
                                               const int32_t *__restrict__ col, const uint16_t *__restrict__ lrow,
-                                              const uint32_t *__restrict__ packed, const int32_t *__restrict__ bases,
+                                              const uint8_t *__restrict__ stream, const int2 *__restrict__ infos,
                                               const Epi &epi, double *s_acc, uint32_t *s_flag)
 {
     using Acc = typename Epi::Acc;
@@ -164,9 +172,28 @@ __device__ __forceinline__ void rb_accumulate(int64_t block_begin, int64_t block
     if (s1 > block_end) s1 = block_end;
     if (s0 >= s1) return;
     const int64_t last = block_end - 1;
-    for (int64_t base = s0; base < s1; base += kWave * kRbUnroll) {
+    // The batches' descriptors are fetched a step ahead (the same for all lanes: scalar loads): an entry's address
+    // depends on its batch's descriptor, and read in the same step that would be a third round trip in the chain
+    // descriptor -> entry -> gathered value.  Batches past the block's last one repeat the last (their entries are
+    // clamped to the block's last entry anyway).
+    const int last_batch = __builtin_amdgcn_readfirstlane((int)((last - block_begin) >> 6));
+    int batch = __builtin_amdgcn_readfirstlane((int)((s0 - block_begin) >> 6));
+    int2 info[kRbUnroll], info_next[kRbUnroll];
+    if (!kWide) {
+#pragma unroll
+        for (int k = 0; k < kRbUnroll; ++k) info[k] = infos[batch + k < last_batch ? batch + k : last_batch];
+    }
+    for (int64_t base = s0; base < s1; base += kWave * kRbUnroll, batch += kRbUnroll) {
         uint32_t a[kRbUnroll];
         int32_t g[kRbUnroll];
+        int bits[kRbUnroll];
+        if (!kWide) {
+#pragma unroll
+            for (int k = 0; k < kRbUnroll; ++k) {
+                const int next = batch + kRbUnroll + k;
+                info_next[k] = infos[next < last_batch ? next : last_batch];
+            }
+        }
 #pragma unroll
         for (int k = 0; k < kRbUnroll; ++k) {
             int64_t e = base + k * kWave + lane;
@@ -175,15 +202,25 @@ __device__ __forceinline__ void rb_accumulate(int64_t block_begin, int64_t block
                 a[k] = (uint32_t)__builtin_nontemporal_load(col + e);
                 g[k] = (int32_t)__builtin_nontemporal_load(lrow + e);
             } else {
-                a[k] = __builtin_nontemporal_load(packed + e);
-                g[k] = bases[(e - block_begin) >> 6];  // same address for all lanes of a wavefront
+                const int bytes = 2 + (info[k].y & 3);
+                const uint8_t *at = stream + ((size_t)((uint32_t)info[k].y >> 2) << 6) + (size_t)((e - block_begin) & 63) * bytes;
+                a[k] = __builtin_nontemporal_load(reinterpret_cast<const RbUnalignedU32 *>(at));
+                g[k] = info[k].x;
+                bits[k] = 8 * bytes;
             }
         }
         int c[kRbUnroll], l[kRbUnroll];
 #pragma unroll
         for (int k = 0; k < kRbUnroll; ++k) {
-            c[k] = kWide ? (int)a[k] : g[k] + (int)(a[k] & 0xFFFFu);
-            l[k] = kWide ? g[k] : (int)(a[k] >> 16);
+            if (kWide) {
+                c[k] = (int)a[k];
+                l[k] = g[k];
+            } else {
+                const uint32_t v = a[k] & (0xFFFFFFFFu >> (32 - bits[k]));
+                const int offset_bits = bits[k] - kRbRowBits;
+                c[k] = g[k] + (int)(v & ((1u << offset_bits) - 1u));
+                l[k] = (int)(v >> offset_bits);
+            }
         }
         Acc v[kRbUnroll];
 #pragma unroll
@@ -191,6 +228,10 @@ __device__ __forceinline__ void rb_accumulate(int64_t block_begin, int64_t block
 #pragma unroll
         for (int k = 0; k < kRbUnroll; ++k)
             rb_add(s_acc, s_flag, l[k], base + k * kWave + lane < s1, v[k]);
+        if (!kWide) {
+#pragma unroll
+            for (int k = 0; k < kRbUnroll; ++k) info[k] = info_next[k];
+        }
     }
 }
 
@@ -199,8 +240,8 @@ __global__ __launch_bounds__(kRbThreads) void pr_rowblock_kernel(const int32_t *
                                                                  const int64_t *__restrict__ block_nnz,
                                                                  const int32_t *__restrict__ col,
                                                                  const uint16_t *__restrict__ lrow,
-                                                                 const uint32_t *__restrict__ packed,
-                                                                 const int32_t *__restrict__ batch_base,
+                                                                 const uint8_t *__restrict__ stream,
+                                                                 const int2 *__restrict__ batch_info,
                                                                  const int32_t *__restrict__ block_batch,
                                                                  const int32_t *__restrict__ block_wide,
                                                                  const int32_t *__restrict__ unit_block,
@@ -223,7 +264,7 @@ __global__ __launch_bounds__(kRbThreads) void pr_rowblock_kernel(const int32_t *
     const int shares = block_units[b];
     const int share = u - block_unit0[b];
     const bool wide = block_wide[b] != 0;
-    const int32_t *bases = batch_base + block_batch[b];
+    const int2 *infos = batch_info + block_batch[b];
     // An unsplit block fetches the epilogue's per-row operand now and lets it wait in registers: read after the
     // sweep, one row at a time, it cost a memory latency per row (a quarter of the time of the blocks that hold
     // many short rows).  Split blocks hold few rows; the work-group that ends up with the epilogue reads them then.
@@ -242,9 +283,9 @@ __global__ __launch_bounds__(kRbThreads) void pr_rowblock_kernel(const int32_t *
     __syncthreads();
 
     if (wide)
-        rb_accumulate<true>(eb, ee, share, shares, tid, col, lrow, packed, bases, epi, s_acc, s_flag);
+        rb_accumulate<true>(eb, ee, share, shares, tid, col, lrow, stream, infos, epi, s_acc, s_flag);
     else
-        rb_accumulate<false>(eb, ee, share, shares, tid, col, lrow, packed, bases, epi, s_acc, s_flag);
+        rb_accumulate<false>(eb, ee, share, shares, tid, col, lrow, stream, infos, epi, s_acc, s_flag);
     __syncthreads();
 
     if (shares > 1) {

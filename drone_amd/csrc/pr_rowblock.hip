@@ -3,6 +3,7 @@
 #include <cstring>
 #include <vector>
 #include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/device/device_scan.hpp>
 
 namespace drone {
 namespace {
@@ -116,18 +117,20 @@ __global__ __launch_bounds__(256) void rb_keys_kernel(const int64_t *__restrict_
 
 // One lane per entry, one wavefront per kPackBatches consecutive 64-entry batches of the blocks' sorted entries (the
 // batches of all blocks are numbered through; a wavefront finds its first batch's block by a search over the blocks'
-// first batches and steps to the next block from there): col = the key's source, base = first source of the batch,
-// packed = lrow << 16 | (source - base); a batch that spans more than 65,535 ids flags its block as wide.  (One
-// work-group per block took 8.4 ms for 263 M entries, a search per batch 2.8 ms.)
+// first batches and steps to the next block from there).  First pass: col = the key's source, the batch's first source
+// and the narrowest entry width (2, 3 or 4 bytes: 15 bits of row plus 1, 9 or 17 bits of offset) that holds the batch's
+// largest offset; a batch that spans 131,072 ids or more flags its block as wide.  (One work-group per block took
+// 8.4 ms for 263 M entries, a search per batch 2.8 ms.)
 constexpr int kPackBatches = 8;
-template <typename Key>
+template <typename Key, bool kWrite>
 __global__ __launch_bounds__(1024) void rb_pack_kernel(int num_blocks, int total_batches,
                                                        const int64_t *__restrict__ block_nnz,
                                                        const int32_t *__restrict__ block_batch, int col_bits,
                                                        const Key *__restrict__ keys_sorted,
                                                        const uint16_t *__restrict__ lrow, int32_t *__restrict__ col,
-                                                       uint32_t *__restrict__ packed, int32_t *__restrict__ batch_base,
-                                                       int32_t *__restrict__ block_wide)
+                                                       int2 *__restrict__ batch_info, uint32_t *__restrict__ batch_size,
+                                                       const uint32_t *__restrict__ batch_pos,
+                                                       uint8_t *__restrict__ stream, int32_t *__restrict__ block_wide)
 {
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t first = (((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave) * kPackBatches;
@@ -146,19 +149,35 @@ __global__ __launch_bounds__(1024) void rb_pack_kernel(int num_blocks, int total
         const int64_t e = block_nnz[b] + (int64_t)(batch - block_batch[b]) * kWave + lane;
         const int32_t c = e < e1 ? (int32_t)((uint32_t)keys_sorted[e] & col_mask) : 0;
         const int32_t base = __shfl(c, 0, kWave);  // sources ascend inside a block
-        bool overflow = false;
-        if (e < e1) {
-            const int32_t off = c - base;
-            overflow = off > 0xFFFF;
-            col[e] = c;
-            packed[e] = ((uint32_t)lrow[e] << 16) | (uint32_t)(off & 0xFFFF);
+        const int32_t off = e < e1 ? c - base : 0;
+        if (!kWrite) {
+            int32_t span = off;
+#pragma unroll
+            for (int m = kWave / 2; m > 0; m >>= 1) {
+                const int32_t other = __shfl_xor(span, m, kWave);
+                span = other > span ? other : span;
+            }
+            const int code = span < (1 << (16 - kRbRowBits)) ? 0 : span < (1 << (24 - kRbRowBits)) ? 1 : 2;
+            if (e < e1) col[e] = c;
+            if (lane == 0) {
+                batch_info[batch] = make_int2(base, code);
+                batch_size[batch] = 2u + (uint32_t)code;  // in 64-byte units
+                if (span >= (1 << (32 - kRbRowBits))) block_wide[b] = 1;  // every writer stores the same value
+            }
+        } else {
+            // second pass: the positions are known (exclusive scan of the sizes); write the entries byte by byte
+            const int code = batch_info[batch].y, bytes = 2 + code;
+            const uint32_t pos = batch_pos[batch];
+            const uint32_t v = e < e1 ? ((uint32_t)lrow[e] << (8 * bytes - kRbRowBits)) | (uint32_t)off : 0u;
+            uint8_t *at = stream + ((size_t)pos << 6) + (size_t)lane * bytes;
+            for (int k = 0; k < bytes; ++k) at[k] = (uint8_t)(v >> (8 * k));
+            __builtin_amdgcn_wave_barrier();
+            if (lane == 0) batch_info[batch].y = (int)((pos << 2) | (uint32_t)code);
         }
-        if (lane == 0) batch_base[batch] = base;
-        if (__any(overflow) && lane == 0) block_wide[b] = 1;  // every writer stores the same value
     }
 }
 
-// Sorts the entries by (block, source) and derives the packed entry format.  The entries arrive grouped by block
+// Sorts the entries by (block, source) and derives the compact entry format.  The entries arrive grouped by block
 // already, so consecutive blocks can be sorted as separate ranges: with `group` (a power of two) blocks per range the
 // key needs col_bits + log2(group) bits, which keeps large matrices on 32-bit keys (R-MAT scale 24, 263 M entries:
 // three ranges of 256 blocks and four 8-bit passes over 6-byte pairs instead of five over 10-byte pairs).
@@ -201,11 +220,39 @@ int rb_sort_and_pack(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_p
         DRONE_HIP_TRY(rocprim::radix_sort_pairs(temp, bytes, keys + first, keys_sorted + first, lrow_in + first,
                                                 rb->lrow + first, count, 0, col_bits + group_bits, stream));
     }
-    rb_pack_kernel<Key><<<(unsigned)ceil_div(ceil_div((int64_t)total_batches, (int64_t)kPackBatches) * kWave, (int64_t)1024), 1024, 0, stream>>>(
-        nb, total_batches, rb->block_nnz, rb->block_batch, col_bits, keys_sorted, rb->lrow, rb->col, rb->packed,
-        rb->batch_base, rb->block_wide);
-    DRONE_HIP_TRY(hipGetLastError());
-    return DRONE_OK;
+    // entry widths per batch, their positions (exclusive scan, in 64-byte units), then the entries themselves
+    uint32_t *batch_size = nullptr, *batch_pos = nullptr;
+    void *scan_temp = nullptr;
+    const auto pack = [&]() -> int {
+        const unsigned grid = (unsigned)ceil_div(ceil_div((int64_t)total_batches, (int64_t)kPackBatches) * kWave, (int64_t)1024);
+        const size_t tb = (size_t)total_batches;
+        DRONE_HIP_TRY(hipMalloc(&batch_size, sizeof(uint32_t) * (tb + 1)));
+        DRONE_HIP_TRY(hipMalloc(&batch_pos, sizeof(uint32_t) * (tb + 1)));
+        DRONE_HIP_TRY(hipMemsetAsync(batch_size + tb, 0, sizeof(uint32_t), stream));
+        rb_pack_kernel<Key, false><<<grid, 1024, 0, stream>>>(nb, total_batches, rb->block_nnz, rb->block_batch, col_bits,
+                                                             keys_sorted, rb->lrow, rb->col, rb->batch_info, batch_size,
+                                                             nullptr, nullptr, rb->block_wide);
+        size_t scan_bytes = 0;
+        DRONE_HIP_TRY(rocprim::exclusive_scan(nullptr, scan_bytes, batch_size, batch_pos, 0u, tb + 1, rocprim::plus<uint32_t>(), stream));
+        DRONE_HIP_TRY(hipMalloc(&scan_temp, scan_bytes ? scan_bytes : 1));
+        DRONE_HIP_TRY(rocprim::exclusive_scan(scan_temp, scan_bytes, batch_size, batch_pos, 0u, tb + 1, rocprim::plus<uint32_t>(), stream));
+        uint32_t total64 = 0;
+        DRONE_HIP_TRY(hipMemcpyAsync(&total64, batch_pos + tb, sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+        DRONE_HIP_TRY(hipStreamSynchronize(stream));
+        rb->stream_bytes = (int64_t)total64 * 64;
+        DRONE_HIP_TRY(hipMalloc(&rb->stream, (size_t)rb->stream_bytes + 64));  // the last entry's 4-byte load may run past it
+        rb_pack_kernel<Key, true><<<grid, 1024, 0, stream>>>(nb, total_batches, rb->block_nnz, rb->block_batch, col_bits,
+                                                            keys_sorted, rb->lrow, rb->col, rb->batch_info, batch_size,
+                                                            batch_pos, rb->stream, rb->block_wide);
+        DRONE_HIP_TRY(hipGetLastError());
+        DRONE_HIP_TRY(hipStreamSynchronize(stream));
+        return DRONE_OK;
+    };
+    const int rc = pack();
+    (void)hipFree(batch_size);
+    (void)hipFree(batch_pos);
+    (void)hipFree(scan_temp);
+    return rc;
 }
 
 }  // namespace
@@ -279,17 +326,16 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
             DRONE_HIP_TRY(hipStreamSynchronize(stream));  // br / bn go out of scope
         }
         rb_walk_len_kernel<<<(int)ceil_div(nb, 256), 256, 0, stream>>>(row_ptr, nb, rb->block_row, rb->block_nnz, rb->walk_len);
-        // packed 4-byte entries: the blocks' 64-entry batches are numbered through
+        // compact entries: the blocks' 64-entry batches are numbered through
         DRONE_HIP_TRY(hipMalloc(&rb->block_batch, sizeof(int32_t) * ((size_t)nb + 1)));
         DRONE_HIP_TRY(hipMalloc(&rb->block_wide, sizeof(int32_t) * (size_t)nb));
-        DRONE_HIP_TRY(hipMalloc(&rb->packed, sizeof(uint32_t) * e));
         DRONE_HIP_TRY(hipMemsetAsync(rb->block_wide, 0, sizeof(int32_t) * (size_t)nb, stream));
         std::vector<int64_t> h_nnz((size_t)nb + 1);
         DRONE_HIP_TRY(hipMemcpyAsync(h_nnz.data(), rb->block_nnz, sizeof(int64_t) * h_nnz.size(), hipMemcpyDeviceToHost, stream));
         DRONE_HIP_TRY(hipStreamSynchronize(stream));
         std::vector<int32_t> h_batch((size_t)nb + 1, 0);
         for (int b = 0; b < nb; ++b) h_batch[b + 1] = h_batch[b] + (int32_t)ceil_div(h_nnz[b + 1] - h_nnz[b], 64);
-        DRONE_HIP_TRY(hipMalloc(&rb->batch_base, sizeof(int32_t) * (size_t)(h_batch[nb] ? h_batch[nb] : 1)));
+        DRONE_HIP_TRY(hipMalloc(&rb->batch_info, sizeof(int2) * (size_t)(h_batch[nb] ? h_batch[nb] : 1)));
         DRONE_HIP_TRY(hipMemcpyAsync(rb->block_batch, h_batch.data(), sizeof(int32_t) * h_batch.size(), hipMemcpyHostToDevice, stream));
         if (nnz > 0) {
             // key = (block within its range << col_bits) | source: 32-bit keys while at most 64 ranges do it
@@ -364,8 +410,8 @@ void row_blocks_destroy(RowBlocks *rb)
     (void)hipFree(rb->walk_len);
     (void)hipFree(rb->col);
     (void)hipFree(rb->lrow);
-    (void)hipFree(rb->packed);
-    (void)hipFree(rb->batch_base);
+    (void)hipFree(rb->stream);
+    (void)hipFree(rb->batch_info);
     (void)hipFree(rb->block_batch);
     (void)hipFree(rb->block_wide);
     (void)hipFree(rb->unit_block);

@@ -218,6 +218,16 @@ def test_sgemm_identity_alpha_beta_ld_and_split_reduction(T):
     assert rel_err(a, ref, np.abs(X.T).astype(np.float64) @ np.abs(G)) <= 1e-4
 
 
+@pytest.mark.parametrize("n", [1, 63, 1024, 4097, 602 * 128, 1_000_003])
+def test_sum_squares(T, n):
+    """drone_sum_squares_f32 (the L2 penalty's reduction, cuda_gcn.cu:254-260) against an fp64 sum; twice the same bits."""
+    from drone_amd import gcn
+    x = np.random.default_rng(n).uniform(-2, 2, n).astype(np.float32)
+    want = float(np.sum(x.astype(np.float64) ** 2))
+    a, b = gcn.sum_squares(dev(T, x)), gcn.sum_squares(dev(T, x))
+    assert abs(float(a) - want) <= 1e-6 * want and T.equal(a, b)
+
+
 def test_relu_dropout(T, oracle):
     from drone_amd import gcn
     rng = np.random.default_rng(0)
