@@ -35,6 +35,9 @@ struct BitCore {
     uint4 *split = nullptr;      // the scaled operand in three bf16 parts, see spmm_bits.hip
     float *partial = nullptr;    // [num_units][512][128]
     int *duplicates = nullptr;   // device flag: an entry met its bit already set
+    // bit_core_products runs here, beside the caller's stream (default priority, ordered by the two events)
+    hipStream_t side = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr;
 };
 
 // width_of_row[rr]: dense width (a multiple of 256, the same for the 512 rows of a tile) of ranked row
@@ -44,10 +47,12 @@ int bit_core_create(BitCore *bc, int rows, const std::vector<int> &width_of_row,
                     const int *cols, const int *col_rank, int max_k, hipStream_t s, bool *has_duplicates);
 void bit_core_destroy(BitCore *bc);
 
-// C[dense_row[rr], 0..K) += alpha * row_scale[dense_row[rr]] * sum over the row's dense cells of
-// col_scale[col] * B[col, 0..K).  col_order: rank -> column.
-int bit_core_multiply(const BitCore *bc, const unsigned *col_order, const float *col_scale, const int *dense_row,
-                      const float *row_scale, const float *B, int ldb, float *C, int ldc, int K, float alpha,
-                      hipStream_t s);
+// Two steps, so that the first can run beside the gathers of the rest of the matrix:
+// bit_core_products: T[rr, 0..K) = sum over ranked row rr's dense cells of col_scale[col] * B[col, 0..K), kept in the core's
+// scratch (col_order: rank -> column); bit_core_add: C[dense_row[rr], 0..K) += alpha * row_scale[dense_row[rr]] * T[rr, :].
+int bit_core_products(const BitCore *bc, const unsigned *col_order, const float *col_scale, const float *B, int ldb,
+                      int K, hipStream_t s);
+int bit_core_add(const BitCore *bc, const int *dense_row, const float *row_scale, float *C, int ldc, int K, float alpha,
+                 hipStream_t s);
 
 }  // namespace drone

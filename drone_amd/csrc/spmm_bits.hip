@@ -305,6 +305,9 @@ int bit_core_create(BitCore *bc, int rows, const std::vector<int> &width_of_row,
     DRONE_HIP_TRY(hipMalloc(&bc->split, sizeof(uint4) * (size_t)bc->passes * (wmax / 8) * kGroupVecs));
     DRONE_HIP_TRY(hipMalloc(&bc->partial, sizeof(float) * (size_t)bc->passes * nu * kBitTileRows * kPartialLd));
     DRONE_HIP_TRY(hipMalloc(&bc->duplicates, sizeof(int)));
+    DRONE_HIP_TRY(hipStreamCreateWithFlags(&bc->side, hipStreamNonBlocking));
+    DRONE_HIP_TRY(hipEventCreateWithFlags(&bc->fork, hipEventDisableTiming));
+    DRONE_HIP_TRY(hipEventCreateWithFlags(&bc->join, hipEventDisableTiming));
     DRONE_HIP_TRY(hipMemcpyAsync(bc->unit_tile, ut.data(), sizeof(int) * nu, hipMemcpyHostToDevice, s));
     DRONE_HIP_TRY(hipMemcpyAsync(bc->unit_c0, uc0.data(), sizeof(int) * nu, hipMemcpyHostToDevice, s));
     DRONE_HIP_TRY(hipMemcpyAsync(bc->unit_c1, uc1.data(), sizeof(int) * nu, hipMemcpyHostToDevice, s));
@@ -339,12 +342,17 @@ void bit_core_destroy(BitCore *bc)
     (void)hipFree(bc->split);
     (void)hipFree(bc->partial);
     (void)hipFree(bc->duplicates);
+    if (bc->side) {
+        (void)hipStreamSynchronize(bc->side);
+        (void)hipStreamDestroy(bc->side);
+    }
+    if (bc->fork) (void)hipEventDestroy(bc->fork);
+    if (bc->join) (void)hipEventDestroy(bc->join);
     *bc = BitCore();
 }
 
-int bit_core_multiply(const BitCore *bc, const unsigned *col_order, const float *col_scale, const int *dense_row,
-                      const float *row_scale, const float *B, int ldb, float *C, int ldc, int K, float alpha,
-                      hipStream_t s)
+int bit_core_products(const BitCore *bc, const unsigned *col_order, const float *col_scale, const float *B, int ldb,
+                      int K, hipStream_t s)
 {
     if (bc->tiles == 0) return DRONE_OK;
     DRONE_REQUIRE(K > 0 && K <= bc->max_k, "K exceeds the plan's feature width");
@@ -362,6 +370,15 @@ int bit_core_multiply(const BitCore *bc, const unsigned *col_order, const float 
             bits_mfma_kernel<4><<<bc->num_units, 512, 0, s>>>(bc->unit_tile, bc->unit_c0, bc->unit_c1, bc->unit_slot,
                                                              bc->tile_blocks, bc->tile_off, bc->bits, split, partial);
     }
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
+int bit_core_add(const BitCore *bc, const int *dense_row, const float *row_scale, float *C, int ldc, int K, float alpha,
+                 hipStream_t s)
+{
+    if (bc->tiles == 0) return DRONE_OK;
+    const int passes = (int)ceil_div(K, 128);
     int grid = (int)ceil_div(bc->rows, 4);
     if (grid > 65536) grid = 65536;
     bits_combine_kernel<<<grid, 256, 0, s>>>(bc->rows, bc->tile_unit0, bc->partial, bc->num_units, passes, dense_row,
