@@ -90,6 +90,8 @@ constexpr size_t kBandBytes = 3u << 20; // feature rows of one band (three quart
 // Band size x hot bands, ms for K = 128 / 41 on the 229 M-entry graph: 1 MB x 48: 4.90 / 3.02; 2 MB x 24: 4.44 / 2.59;
 // 2.5 MB x 19: 4.35 / 2.52; 3 MB x 16: 4.32 / 2.48; 3 MB x 20: 4.33 / 2.49; 3 MB x 24: 4.32 / 2.53; 4 MB x 12: 4.45 / 2.46.
 // With 2 MB bands, 10 / 15 / 24 / 32 hot bands: 5.44 / 4.83 / 4.44 / 4.44 ms (K = 128).
+// With the dense region kept as bits (scaled patterns), 3 MB x 4 / 8 / 12 / 16 / 20 / 28 / 38 / 56 hot bands: 3.45 / 3.00 / 2.85 /
+// 2.75 / 2.80 / 2.95 / 3.07 / 3.05 ms at K = 128 and 1.64 / 1.51 / 1.39 / 1.35 / 1.35 / 1.34 / 1.35 / 1.33 at K = 41.
 constexpr int kBandMaxCols = 8192;      // narrow feature rows: a band is at most this many columns
 constexpr int kRowsPerBlock = 4;        // wavefronts per work-group (2 / 4 / 8: 4.29 / 4.31 / 4.33 ms at K = 128, 2.50 / 2.45 / 2.56 at K = 41)
 constexpr int kDenseChunk = 2048;       // column granularity of the dense rectangles
@@ -104,8 +106,9 @@ constexpr double kDenseMinGainMs = 0.25;
 // Cost per cell of one 32-wide feature tile, measured on the 232,965-vertex / 229 M-entry graph (0.53 ps per cell at 128
 // feature columns); the gathers it replaces are priced as for the fp32 rectangles.  Pricing a gather at 1.4 / 1.8 / 2.6
 // times that (which grows the bit region from 1.24 to 1.87 / 2.09 / 2.17 G cells and takes 177 -> 190 / 193 / 194 M of
-// the 229 M entries) left the product where it was, 2.9 ms at 128 columns: what remains outside is priced by its number
-// of band pieces rather than by its entries.
+// the 229 M entries) left the product where it was, 2.9 ms at 128 columns (2.74 / 2.81 / 2.80 / 2.85 with the bit products
+// running beside the gathers): what remains outside is priced by its number of band pieces rather than by its entries -
+// the piece kernel takes 1.15 ms for 34 M entries and 0.99 ms for 17.5 M.
 constexpr int kBitMaxChunks = 128;      // columns considered: the 262,144 most frequent
 constexpr int kBitGroupRows = 4096;
 constexpr int kBitMaxGroups = 1024;
