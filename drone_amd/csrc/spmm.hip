@@ -102,6 +102,18 @@ constexpr float kDenseThreshold = 0.12f;  // for feature widths that fill 128-co
 constexpr double kGatherMsPerEntry = 0.19e-9;  // band-piece kernel: 24 ps per entry at K = 128
 constexpr double kDenseMsPerCell = 0.025e-9;   // dense product: 3.2 ps per cell at K = 128
 constexpr double kDenseMinGainMs = 0.25;
+// DRONE_SPMM_DENSE_MIN_GAIN_MS in the environment replaces kDenseMinGainMs when a plan is made: 0 lets matrices of a few
+// thousand rows get a dense part too, which is how the tests reach the dense kernels' edge cases at sizes a CPU can check.
+double dense_min_gain_ms()
+{
+    const char *env = getenv("DRONE_SPMM_DENSE_MIN_GAIN_MS");
+    if (env && *env) {
+        char *end = nullptr;
+        const double v = strtod(env, &end);
+        if (end != env && *end == '\0' && v >= 0.0) return v;
+    }
+    return kDenseMinGainMs;
+}
 // Scaled patterns (bit core): row groups of 4096 ranked long rows each, any leading set of 2048-column chunks.
 // Cost per cell of one 32-wide feature tile, measured on the 232,965-vertex / 229 M-entry graph (0.53 ps per cell at 128
 // feature columns); the gathers it replaces are priced as for the fp32 rectangles.  Pricing a gather at 1.4 / 1.8 / 2.6
@@ -727,7 +739,7 @@ int build_band_pieces(drone_spmm_plan *p, const std::vector<int> &h_rp, const st
                 // launches, adding the rows back): measured rates, ms per entry and per cell at feature width 1.
                 gain_ms = dense_entries * p->max_k * kGatherMsPerEntry - dense_cells * (p->max_k / efficiency) * kDenseMsPerCell;
             }
-            if (gain_ms < kDenseMinGainMs) std::fill(group_width.begin(), group_width.end(), 0);
+            if (gain_ms < dense_min_gain_ms()) std::fill(group_width.begin(), group_width.end(), 0);
             for (int g = 0; g < groups && group_width[g] > 0; ++g)
                 for (int r = group_begin[g]; r < group_begin[g + 1]; ++r) dense_width_of_long[by_rank[r]] = group_width[g];
         }

@@ -131,3 +131,57 @@ def test_pull_f64_random(T, case):
     got = plan.run(0.85, iters).cpu().numpy()
     plan.close()
     assert float(np.max(np.abs(got - r) / r)) <= 1e-9
+
+
+@pytest.mark.parametrize("case", range(36))
+def test_scaled_pattern_spmm_random(T, case, monkeypatch):
+    """Scaled 0/1 patterns around the bit core's internal limits (512-row tiles, 4,096-row groups, 2,048-column chunks,
+    256-column blocks, 128-column passes), with the minimum-gain rule switched off so that matrices of a few thousand
+    rows get a bit core: diag(r) P diag(c) B against scipy in fp64, 1e-4 of every element's accumulated |a||b|."""
+    from drone_amd import gcn
+    monkeypatch.setenv("DRONE_SPMM_DENSE_MIN_GAIN_MS", "0")
+    rng = np.random.default_rng(5000 + case)
+    n_rows = int(rng.choice([600, 1100, 4096, 4100, 5000, 9000]))
+    n_cols = int(rng.choice([2048, 2049, 4095, 4100, 6500, 9000]))
+    K = int(rng.choice([1, 7, 32, 33, 41, 64, 65, 100, 128, 129, 200, 256]))
+    ld_pad = int(rng.choice([0, 0, 3, 4]))
+    long_rows = int(rng.choice([1, 40, 511, 512, 513, 700, 3000])) if n_rows > 700 else int(rng.choice([1, 40, 300]))
+    long_rows = min(long_rows, n_rows)
+    density = float(rng.choice([0.3, 0.6, 0.95]))
+    hot_cols = int(rng.choice([2048, 2100, 4096])) if n_cols >= 4096 else 2048
+    # long rows: dense over the hot columns, sparse elsewhere; the other rows sparse everywhere
+    rows_perm, cols_perm = rng.permutation(n_rows), rng.permutation(n_cols)
+    r, c = np.nonzero(rng.random((long_rows, hot_cols)) < density)
+    extra = int(0.002 * n_rows * n_cols)
+    rr = np.concatenate([rows_perm[r], rng.integers(0, n_rows, extra)])
+    cc = np.concatenate([cols_perm[c], rng.integers(0, n_cols, extra)])
+    pat = sp.csr_matrix((np.ones(rr.size, np.float32), (rr, cc)), shape=(n_rows, n_cols))
+    pat.sum_duplicates()
+    pat.sort_indices()
+    pat.data[:] = 1.0
+    row_scale = rng.uniform(0.05, 1.0, n_rows).astype(np.float32)
+    col_scale = rng.uniform(0.05, 1.0, n_cols).astype(np.float32)
+    val = (row_scale[np.repeat(np.arange(n_rows), np.diff(pat.indptr))] * col_scale[pat.indices]).astype(np.float32)
+    m = sp.csr_matrix((val, pat.indices, pat.indptr), shape=(n_rows, n_cols))
+    B = rng.uniform(-1, 1, (n_cols, K)).astype(np.float32)
+    alpha, beta = (1.0, 0.0) if rng.random() < 0.5 else (float(rng.uniform(-2, 2)), float(rng.choice([0.0, 1.0, -0.5])))
+    C0 = rng.uniform(-1, 1, (n_rows, K)).astype(np.float32)
+    rp, ci, v = dev(T, m.indptr.astype(np.int32)), dev(T, m.indices.astype(np.int32)), dev(T, val)
+    Bd = T.zeros((n_cols, K + ld_pad), dtype=T.float32, device="cuda")
+    Bd[:, :K] = dev(T, B)
+    out = T.full((n_rows, K + ld_pad), 7.0, dtype=T.float32, device="cuda")
+    out[:, :K] = dev(T, C0)
+    plan = gcn.SpmmPlan(rp, ci, v, n_cols, max_k=K, row_scale=dev(T, row_scale), col_scale=dev(T, col_scale))
+    has_long = int((np.diff(m.indptr) > 512).sum())
+    if has_long and long_rows >= 511 and K >= 32:                  # 40 rows in a 512-row tile are too sparse to pay
+        assert plan.bit_core()["cells"] > 0, (n_rows, n_cols, K, long_rows, hot_cols, density)
+    gcn.spmm(plan, rp, ci, v, Bd[:, :K], K=K, out=out[:, :K], alpha=alpha, beta=beta)
+    T.cuda.synchronize()
+    plan.close()
+    got = out.cpu().numpy()
+    m64 = m.astype(np.float64)
+    want = alpha * (m64 @ B.astype(np.float64)) + beta * C0
+    scale = abs(alpha) * (abs(m64) @ np.abs(B).astype(np.float64)) + abs(beta) * np.abs(C0)
+    assert np.max(np.abs(got[:, :K] - want) / np.maximum(scale, 1e-30)) <= 1e-4
+    if ld_pad:
+        assert np.all(got[:, K:] == 7.0)
