@@ -33,7 +33,7 @@ constexpr int kRbThreads = 1024;
 // 0.573 ms per fp64 iteration and 0.77 against 0.69 ms per float superstep with the current shared blocks.
 constexpr int kRbRows = 16384;       // most rows ending in one block (LDS accumulators: 128 KB)
 constexpr int kRbMaxItems = 1 << 20; // most entries in one block (the plan picks a power of two up to this)
-constexpr int kRbUnroll = 4;
+constexpr int kRbUnroll = 4;    // batches in flight per wavefront; with the compact entries 2 / 3 / 4 / 6 / 8: 0.679 / 0.577 / 0.552 / 0.544 / 0.554 ms
 constexpr int kRbSplit = 8;         // most work-groups that share one block of a large matrix
 constexpr int kRbLdsBytes = (kRbRows + 8) * (int)sizeof(double);  // rows ending in a block <= kRbRows + 1, + the open row
 
