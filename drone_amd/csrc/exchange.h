@@ -8,8 +8,9 @@
 //
 // What is different here:
 //  * The send lists are static properties of the partition.  They are built once (mirrors grouped by master
-//    worker; (master, mirror worker) pairs grouped by worker; ascending local id inside a group), so a step is
-//    flag -> exclusive scan -> scatter, with no atomics, and the send buffers come out in a reproducible order.
+//    worker; (master, mirror worker) pairs grouped by worker; ascending local id inside a group) and cut into chunks
+//    of at most 1,024 items, so a step is two launches - count the senders of every chunk, then pack every chunk behind
+//    the earlier chunks' counts - with no atomics, and the send buffers come out in list order, the same every time.
 //  * Received segments are applied one source worker at a time.  A worker sends a vertex at most once per phase,
 //    so a segment never names a vertex twice and the float additions at a master happen in worker order.
 //  * The wire is a function table (drone_transport) reached through Comm::comm, so the same code runs over the

@@ -1,6 +1,7 @@
 // Replica exchange: static send lists, pack / apply kernels, the in-process loopback transport.
 #include "exchange.h"
 
+#include <algorithm>
 #include <chrono>
 #include <condition_variable>
 #include <mutex>
@@ -21,41 +22,75 @@ template <typename T> T *to_device_vec(const std::vector<T> &h)
     return d;
 }
 
-// flag[i] = 1 iff item i of the static list sends this step; flag[items] = 0 so that the exclusive scan over
-// items + 1 elements ends with the total.
 template <typename Policy>
-__global__ void exchange_flag_kernel(int phase, int items, const int *__restrict__ item_vertex,
-                                     const int *__restrict__ active, const int *__restrict__ ubm,
-                                     int *__restrict__ flag)
+__device__ __forceinline__ bool exchange_sends(int phase, int v, const int *__restrict__ active, const int *__restrict__ ubm)
 {
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i <= items; i += gridDim.x * blockDim.x) {
-        int f = 0;
-        if (i < items) {
-            const int v = item_vertex[i];
-            f = phase == kMirrorToMaster ? Policy::send_mirror(active[v]) : Policy::send_master(active[v], ubm[v]);
+    return phase == kMirrorToMaster ? Policy::send_mirror(active[v]) : Policy::send_master(active[v], ubm[v]);
+}
+
+// Sum of `v` over the 256 threads of the work-group, in every thread.  s_red: 4 ints of LDS.
+__device__ __forceinline__ int block_sum_256_int(int v, int *s_red)
+{
+#pragma unroll
+    for (int m = kWave / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, kWave);
+    __syncthreads();  // s_red may still be read from an earlier call
+    if ((threadIdx.x & (kWave - 1)) == 0) s_red[threadIdx.x / kWave] = v;
+    __syncthreads();
+    return s_red[0] + s_red[1] + s_red[2] + s_red[3];
+}
+
+// One work-group per chunk of the static list: chunk_count[c] = how many of its items send this step.
+template <typename Policy>
+__global__ __launch_bounds__(256) void exchange_count_kernel(int phase, const int *__restrict__ chunk_begin,
+                                                             const int *__restrict__ chunk_end,
+                                                             const int *__restrict__ item_vertex,
+                                                             const int *__restrict__ active, const int *__restrict__ ubm,
+                                                             int *__restrict__ chunk_count)
+{
+    __shared__ int s_red[4];
+    const int c = blockIdx.x;
+    int mine = 0;
+    for (int i = chunk_begin[c] + threadIdx.x; i < chunk_end[c]; i += 256)
+        mine += exchange_sends<Policy>(phase, item_vertex[i], active, ubm) ? 1 : 0;
+    const int total = block_sum_256_int(mine, s_red);
+    if (threadIdx.x == 0) chunk_count[c] = total;
+}
+
+// One work-group per chunk: the chunk's sending items go to send_*[sum of the earlier chunks' counts ...), in list
+// order - the result of a flag / exclusive scan / scatter over the whole list, in two launches and without a scan
+// library's passes (the counts of at most a few thousand chunks are summed again by every work-group).
+template <typename Policy>
+__global__ __launch_bounds__(256) void exchange_pack_kernel(int phase, const int *__restrict__ chunk_begin,
+                                                            const int *__restrict__ chunk_end,
+                                                            const int *__restrict__ item_vertex,
+                                                            const int *__restrict__ active, const int *__restrict__ ubm,
+                                                            const int *__restrict__ chunk_count,
+                                                            const int *__restrict__ l2g,
+                                                            const typename Policy::T *__restrict__ vals,
+                                                            int *__restrict__ send_id,
+                                                            typename Policy::T *__restrict__ send_val)
+{
+    __shared__ int s_red[4], s_wave[4];
+    const int c = blockIdx.x, lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    if (chunk_count[c] == 0) return;  // the same for the whole work-group
+    int before = 0;
+    for (int k = threadIdx.x; k < c; k += 256) before += chunk_count[k];
+    int base = block_sum_256_int(before, s_red);
+    for (int i0 = chunk_begin[c]; i0 < chunk_end[c]; i0 += 256) {
+        const int i = i0 + threadIdx.x;
+        const int v = i < chunk_end[c] ? item_vertex[i] : 0;
+        const bool f = i < chunk_end[c] && exchange_sends<Policy>(phase, v, active, ubm);
+        const unsigned long long votes = __ballot(f);
+        __syncthreads();  // s_wave of the previous round has been read
+        if (lane == 0) s_wave[wave] = __popcll(votes);
+        __syncthreads();
+        int p = base + __popcll(votes & ((1ull << lane) - 1ull));
+        for (int w = 0; w < wave; ++w) p += s_wave[w];
+        if (f) {
+            send_id[p] = l2g[v];
+            send_val[p] = vals[v];
         }
-        flag[i] = f;
-    }
-}
-
-// send_index[w] = pos[group_off[w]]: where worker w's segment starts in the send buffers
-__global__ void exchange_index_kernel(int workers, const int *__restrict__ group_off, const int *__restrict__ pos,
-                                      int *__restrict__ send_index)
-{
-    const int w = blockIdx.x * blockDim.x + threadIdx.x;
-    if (w <= workers) send_index[w] = pos[group_off[w]];
-}
-
-template <typename T>
-__global__ void exchange_pack_kernel(int items, const int *__restrict__ item_vertex, const int *__restrict__ flag,
-                                     const int *__restrict__ pos, const int *__restrict__ l2g,
-                                     const T *__restrict__ vals, int *__restrict__ send_id, T *__restrict__ send_val)
-{
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < items; i += gridDim.x * blockDim.x) {
-        if (!flag[i]) continue;
-        const int v = item_vertex[i], p = pos[i];
-        send_id[p] = l2g[v];
-        send_val[p] = vals[v];
+        base += s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
     }
 }
 
@@ -109,6 +144,12 @@ void drone::routes_release(RouteLists *r)
     if (r->send_index_h) (void)hipHostFree(r->send_index_h);
     if (r->unknown) (void)hipFree(r->unknown);
     if (r->unknown_h) (void)hipHostFree(r->unknown_h);
+    for (int d = 0; d < 2; ++d) {
+        if (r->chunk_begin[d]) (void)hipFree(r->chunk_begin[d]);
+        if (r->chunk_end[d]) (void)hipFree(r->chunk_end[d]);
+    }
+    if (r->chunk_count) (void)hipFree(r->chunk_count);
+    if (r->chunk_count_h) (void)hipHostFree(r->chunk_count_h);
     *r = RouteLists{};
 }
 
@@ -174,6 +215,28 @@ int drone::routes_prepare(Graph *g, int workerNum)
     DRONE_HIP_TRY(hipHostMalloc(&r.send_index_h, sizeof(int) * ((size_t)workerNum + 1)));
     DRONE_HIP_TRY(hipMalloc(&r.unknown, sizeof(int)));
     DRONE_HIP_TRY(hipHostMalloc(&r.unknown_h, sizeof(int)));
+    // chunks of the two lists for the (id, value) exchange
+    int most_chunks = 0;
+    for (int d = 0; d < 2; ++d) {
+        const std::vector<int> &off = d == 0 ? r.mirror_off : r.master_off;
+        std::vector<int> begin, end;
+        r.chunk_worker[d].clear();
+        for (int w = 0; w < workerNum; ++w)
+            for (int b = off[w]; b < off[w + 1]; b += kExchangeChunk) {
+                begin.push_back(b);
+                end.push_back(b + kExchangeChunk < off[w + 1] ? b + kExchangeChunk : off[w + 1]);
+                r.chunk_worker[d].push_back(w);
+            }
+        r.num_chunks[d] = (int)begin.size();
+        r.chunk_begin[d] = to_device_vec(begin);
+        r.chunk_end[d] = to_device_vec(end);
+        DRONE_REQUIRE(r.chunk_begin[d] && r.chunk_end[d], "device allocation of the send chunks failed");
+        if (r.num_chunks[d] > most_chunks) most_chunks = r.num_chunks[d];
+    }
+    DRONE_HIP_TRY(hipMalloc(&r.chunk_count, sizeof(int) * ((size_t)most_chunks + 1)));
+    DRONE_HIP_TRY(hipHostMalloc(&r.chunk_count_h, sizeof(int) * ((size_t)most_chunks + 1)));
+    DRONE_HIP_TRY(hipMemset(r.chunk_count, 0, sizeof(int) * ((size_t)most_chunks + 1)));
+    r.unknown_reported = 0;
     r.workers = workerNum;
     r.ready = true;
     return DRONE_OK;
@@ -208,34 +271,39 @@ int drone::exchange_phase(Graph *g, int phase, typename Policy::T *vals, int *se
     RouteLists &r = x->routes;
     hipStream_t s = static_cast<hipStream_t>(comm->s);
     const bool up = phase == kMirrorToMaster;
-    const int items = up ? r.mirror_items : r.master_items;
+    const int dir = up ? 0 : 1;
     const int *item_vertex = up ? r.mirror_vertex : r.master_vertex;
-    const int *group_off = r.group_off + (up ? 0 : workerNum + 1);
-
-    exchange_flag_kernel<Policy><<<grid_for(items + 1), 256, 0, s>>>(phase, items, item_vertex, g->active,
-                                                                     g->updateByMessage, r.flag);
-    size_t tmp = r.scan_tmp_bytes;
-    DRONE_HIP_TRY(rocprim::exclusive_scan(r.scan_tmp, tmp, r.flag, r.pos, 0, (size_t)items + 1, rocprim::plus<int>(), s));
-    exchange_index_kernel<<<(int)ceil_div(workerNum + 1, 64), 64, 0, s>>>(workerNum, group_off, r.pos, r.send_index_d);
-    exchange_pack_kernel<T><<<grid_for(items), 256, 0, s>>>(items, item_vertex, r.flag, r.pos, g->Local2Global, vals,
-                                                            send_id, send_val);
-    DRONE_HIP_TRY(hipGetLastError());
-    DRONE_HIP_TRY(hipMemcpyAsync(r.send_index_h, r.send_index_d, sizeof(int) * ((size_t)workerNum + 1),
-                                 hipMemcpyDeviceToHost, s));
+    const int chunks = r.num_chunks[dir];
+    // the slot after the chunks' counts holds the unknown ids received so far: it comes back with the counts, so an
+    // id that is not on this worker is reported one phase late, but the phase needs no second synchronisation for it
+    int *unknown = r.chunk_count + std::max(r.num_chunks[0], r.num_chunks[1]);
+    if (chunks > 0) {
+        exchange_count_kernel<Policy><<<chunks, 256, 0, s>>>(phase, r.chunk_begin[dir], r.chunk_end[dir], item_vertex,
+                                                             g->active, g->updateByMessage, r.chunk_count);
+        exchange_pack_kernel<Policy><<<chunks, 256, 0, s>>>(phase, r.chunk_begin[dir], r.chunk_end[dir], item_vertex,
+                                                            g->active, g->updateByMessage, r.chunk_count,
+                                                            g->Local2Global, vals, send_id, send_val);
+        DRONE_HIP_TRY(hipGetLastError());
+    }
+    const size_t most = (size_t)std::max(r.num_chunks[0], r.num_chunks[1]);
+    DRONE_HIP_TRY(hipMemcpyAsync(r.chunk_count_h, r.chunk_count, sizeof(int) * (most + 1), hipMemcpyDeviceToHost, s));
     DRONE_HIP_TRY(hipStreamSynchronize(s));
+    if (r.chunk_count_h[most] > r.unknown_reported) {
+        printf("error global id: %d received ids are not on worker %d\n", r.chunk_count_h[most] - r.unknown_reported, workerId);
+        r.unknown_reported = r.chunk_count_h[most];
+    }
 
-    std::vector<int> send_len((size_t)workerNum), recv_len((size_t)workerNum, 0);
-    for (int w = 0; w < workerNum; ++w) send_len[w] = r.send_index_h[w + 1] - r.send_index_h[w];
+    std::vector<int> send_len((size_t)workerNum, 0), send_index((size_t)workerNum + 1, 0), recv_len((size_t)workerNum, 0);
+    for (int c = 0; c < chunks; ++c) send_len[(size_t)r.chunk_worker[dir][(size_t)c]] += r.chunk_count_h[c];
+    for (int w = 0; w < workerNum; ++w) send_index[(size_t)w + 1] = send_index[(size_t)w] + send_len[(size_t)w];
     DRONE_REQUIRE(send_len[workerId] == 0, "the routing tables name this worker as its own peer");
     const void *send[2] = {send_id, send_val};
     void *recv[2] = {recv_id, recv_val};
     const size_t elem[2] = {sizeof(int), sizeof(T)};
-    rc = tr->exchange(tr->ctx, workerId, workerNum, send_len.data(), r.send_index_h, 2, send, recv, elem,
+    rc = tr->exchange(tr->ctx, workerId, workerNum, send_len.data(), send_index.data(), 2, send, recv, elem,
                       recv_len.data(), r.capacity, comm->s);
     if (rc != DRONE_OK) return rc;
 
-    int *unknown = r.unknown;
-    DRONE_HIP_TRY(hipMemsetAsync(unknown, 0, sizeof(int), s));
     int total = 0;
     for (int w = 0; w < workerNum; ++w) {
         const int len = recv_len[w];
@@ -246,10 +314,7 @@ int drone::exchange_phase(Graph *g, int phase, typename Policy::T *vals, int *se
         total += len;
     }
     DRONE_HIP_TRY(hipGetLastError());
-    DRONE_HIP_TRY(hipMemcpyAsync(r.unknown_h, unknown, sizeof(int), hipMemcpyDeviceToHost, s));
-    DRONE_HIP_TRY(hipStreamSynchronize(s));
-    if (*r.unknown_h > 0) printf("error global id: %d received ids are not on worker %d\n", *r.unknown_h, workerId);
-    *sent = r.send_index_h[workerNum];
+    *sent = send_index[(size_t)workerNum];
     *received = total;
     return DRONE_OK;
 }

@@ -29,7 +29,17 @@ struct RouteLists {
     int *send_index_h = nullptr;   // pinned [workers + 1]
     int *unknown = nullptr;        // device scalar: received ids that are not on this worker
     int *unknown_h = nullptr;      // pinned landing place of that scalar
+    // The (id, value) exchange packs in chunks: a chunk is at most kExchangeChunk consecutive items of one worker's
+    // group.  [0] the mirror list's chunks, [1] the master list's.
+    int num_chunks[2] = {0, 0};
+    int *chunk_begin[2] = {nullptr, nullptr};  // device [num_chunks]
+    int *chunk_end[2] = {nullptr, nullptr};
+    std::vector<int> chunk_worker[2];          // host [num_chunks]
+    int *chunk_count = nullptr;    // device [max chunks + 1]: items each chunk sends this step; last: unknown ids so far
+    int *chunk_count_h = nullptr;  // pinned copy
+    int unknown_reported = 0;      // how many of the unknown ids have been printed
 };
+constexpr int kExchangeChunk = 1024;
 
 // Staging of the K-wide row synchronisation (grow-only).
 struct RowSync {
