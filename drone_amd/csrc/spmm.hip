@@ -9,7 +9,8 @@
 // read), U rows deep, so P*U feature-row loads are in flight per wave.  (col,val) pairs are read 64 at a time,
 // one per lane, and handed to the groups by cross-lane reads.
 //
-// Schedule: rows of at most kSplitRow non-zeros get one wavefront each, in row order.  Longer rows carry
+// Schedule: rows of at most kSplitRow non-zeros are taken in row order, a wavefront per chunk of consecutive rows
+// that hold at most 64 entries together (spmm_chunks_kernel).  Longer rows carry
 // most of the non-zeros of power-law graphs and gather from all over B; run row by row their accesses miss
 // L2 (B is hundreds of MB, an XCD's L2 is 4 MB).  They are therefore cut by COLUMN BAND: columns are ranked by
 // how often they occur, a band is the set of columns whose feature rows fill about 3 MB (kBandBytes), the first
@@ -48,6 +49,9 @@ struct drone_spmm_plan {
     int n_rows = 0, n_cols = 0;
     int64_t nnz = 0;
     int max_k = 0;
+    // short rows in chunks: consecutive rows of at most 64 entries together (or one row of any length up to the split)
+    int num_chunks = 0;
+    int *chunk_r0 = nullptr, *chunk_r1 = nullptr;  // device [num_chunks]
     // long rows, cut into band pieces
     int num_long = 0, num_pieces = 0;
     int64_t long_nnz = 0;
@@ -217,93 +221,139 @@ __device__ __forceinline__ void store_row(float *__restrict__ dst, int kbase, in
         }
 }
 
-// One wavefront per row; rows longer than kSplitRow are left to the piece kernels.
-template <int G, int VEC>
-__global__ __launch_bounds__(kWave * kRowsPerBlock) void spmm_rows_kernel(
-    int n_rows, const int *__restrict__ rp, const int *__restrict__ ci, const float *__restrict__ val,
-    const float *__restrict__ B, int ldb, float *__restrict__ C, int ldc, int K, float alpha, float beta)
+// One wavefront per CHUNK of short rows: consecutive rows whose entries, at most 64 together, are fetched with one
+// coalesced load (a row of more than 64 entries is a chunk of its own and runs the single-row schedule).  One
+// wavefront per row spends a short row's time on its chain of round trips - bounds, pairs, feature rows, store - with
+// a handful of feature-row loads in flight at the end of it; a chunk pays the first two round trips once for ten rows
+// or so and then keeps U feature-row loads per lane group in flight across the row boundaries.  The P lane groups
+// take contiguous row ranges of the chunk (cut where the entries divide evenly); a group walks its entries in order
+// and stores a row whenever the next entry belongs to another one.  Control flow is kept uniform over the wavefront
+// (the cross-lane reads must see every lane), the groups differ in predicates only.
+// Where a chunk's segments (rows of the matrix) begin and end, and where their sums go.  (The band pieces were run
+// through the same kernel, consecutive pieces of the work list with at most 64 entries together: no gain, 9.85 against
+// 9.79 ms per training step on the 229 M-entry graph - what is left in pieces waits for the fabric, not for round trips.)
+struct RowSegments {
+    const int *__restrict__ rp;
+    float *__restrict__ C;
+    int ldc;
+    float alpha, beta;
+    __device__ __forceinline__ int start(int first, int j, int) const { return rp[first + j]; }  // j <= count
+    __device__ __forceinline__ float *out(int first, int j) const { return C + (size_t)(first + j) * ldc; }
+};
+template <int G, int VEC, typename Segments>
+__global__ __launch_bounds__(kWave * kRowsPerBlock) void spmm_chunks_kernel(
+    int num_chunks, const int *__restrict__ chunk_first, const int *__restrict__ chunk_last, Segments seg,
+    const int *__restrict__ ci, const float *__restrict__ val, const float *__restrict__ B, int ldb, int K)
 {
-    const int r = blockIdx.x * kRowsPerBlock + threadIdx.x / kWave;
-    if (r >= n_rows) return;
-    const int e0 = rp[r], e1 = rp[r + 1];
-    if (e1 - e0 > kSplitRow) return;
+    constexpr int P = kWave / G;
+    constexpr int U = 8;  // feature-row loads in flight per lane group (4 / 6 / 8 measured the same)
+    const int c = blockIdx.x * kRowsPerBlock + threadIdx.x / kWave;
+    if (c >= num_chunks) return;
     const int lane = threadIdx.x & (kWave - 1);
     const int li = lane % G, sub = lane / G;
-    for (int k0 = 0; k0 < K; k0 += G * VEC) {
-        const int kbase = k0 + li * VEC;
-        const bool active = kbase < K;
-        float acc[VEC];
-        row_segment<G, VEC>(e0, e1, ci, val, B, ldb, kbase, active, acc);
-        if (sub == 0 && active) store_row<VEC>(C + (size_t)r * ldc, kbase, K, acc, alpha, beta);
+    const int r0 = chunk_first[c], nrows = chunk_last[c] - r0;
+    const float alpha = seg.alpha, beta = seg.beta;
+    if (nrows == 1) {
+        const int e0 = seg.start(r0, 0, 1), e1 = seg.start(r0, 1, 1);
+        float *dst = seg.out(r0, 0);
+        for (int k0 = 0; k0 < K; k0 += G * VEC) {
+            const int kbase = k0 + li * VEC;
+            const bool active = kbase < K;
+            float acc[VEC];
+            row_segment<G, VEC>(e0, e1, ci, val, B, ldb, kbase, active, acc);
+            if (sub == 0 && active) store_row<VEC>(dst, kbase, K, acc, alpha, beta);
+        }
+        return;
     }
-}
-
-// Narrow feature rows (K <= 32) leave a wavefront with 8 or 16 lane groups, and a short row cannot feed them: one
-// wavefront per row spends its time on the row's chain of round trips (bounds, pairs, feature rows, store).  Here a
-// wavefront takes R consecutive rows, W = 64 / R lanes each: every row has its own batch of W (col, val) pairs and
-// its own P = W / G lane groups; the loop runs as long as the longest of the R rows.
-template <int G, int VEC, int R>
-__global__ __launch_bounds__(kWave * kRowsPerBlock) void spmm_rows_multi_kernel(
-    int n_rows, const int *__restrict__ rp, const int *__restrict__ ci, const float *__restrict__ val,
-    const float *__restrict__ B, int ldb, float *__restrict__ C, int ldc, int K, float alpha, float beta)
-{
-    constexpr int W = kWave / R, P = W / G, U = G < 8 ? G : 8, S = P * U;
-    static_assert(P >= 1 && W % S == 0, "a step never straddles two batches");
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wl = lane % W, w0 = lane - wl, li = wl % G, sub = wl / G;
-    const int r = (blockIdx.x * kRowsPerBlock + threadIdx.x / kWave) * R + lane / W;
-    int e0 = 0, len = 0;
-    if (r < n_rows) {
-        e0 = rp[r];
-        len = rp[r + 1] - e0;
-        if (len > kSplitRow) len = 0;  // left to the piece kernels
-    }
-    int longest = len;
+    // lane j holds where segment r0 + j starts; lanes nrows .. 63 hold where the chunk ends
+    const int start = seg.start(r0, lane < nrows ? lane : nrows, nrows);
+    const int e0 = __shfl(start, 0, kWave), n = __shfl(start, nrows, kWave) - e0;
+    const int col = lane < n ? ci[e0 + lane] : 0;
+    const float a = lane < n ? val[e0 + lane] : 0.0f;
+    // the segment of entry `lane`: the last one that starts at or before it
+    int row_of = 0;
+    {
+        int lo = 0, hi = nrows - 1;
 #pragma unroll
-    for (int off = W; off < kWave; off <<= 1) {
-        const int other = __shfl_xor(longest, off, kWave);
-        longest = other > longest ? other : longest;
+        for (int it = 0; it < 6; ++it) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (__shfl(start, mid, kWave) <= e0 + lane) lo = mid; else hi = mid - 1;
+        }
+        row_of = lo;
     }
+    // group `sub` takes the segments from the first one that starts at or after its share of the entries
+    const auto first_row_at = [&](int target) {  // smallest j in [0, nrows] with start_j >= target (start_nrows = end)
+        int lo = 0, hi = nrows;
+#pragma unroll
+        for (int it = 0; it < 7; ++it) {
+            const int mid = (lo + hi) >> 1;
+            const int at = __shfl(start, mid, kWave);  // by every lane, whatever its own search still needs
+            if (lo < hi) {
+                if (at >= target) hi = mid; else lo = mid + 1;
+            }
+        }
+        return lo;
+    };
+    // (both searches by every lane: the starts they read sit in the first lanes, which must not be masked off)
+    const int ra = first_row_at(e0 + (n * sub + P - 1) / P);
+    const int rb_search = first_row_at(e0 + (n * (sub + 1) + P - 1) / P);
+    const int rb = sub == P - 1 ? nrows : rb_search;
+    const int qa = __shfl(start, ra, kWave) - e0, qb = __shfl(start, rb, kWave) - e0;
+    int steps = (qb - qa + U - 1) / U;
+#pragma unroll
+    for (int off = G; off < kWave; off <<= 1) {
+        const int other = __shfl_xor(steps, off, kWave);
+        steps = other > steps ? other : steps;
+    }
+    // segments without entries: out = beta * out, by the first lane group
+    const int next_start = __shfl_down(start, 1, kWave);
+    const unsigned long long empty = __ballot(lane < nrows && next_start == start);
     for (int k0 = 0; k0 < K; k0 += G * VEC) {
         const int kbase = k0 + li * VEC;
         const bool active = kbase < K;
         float acc[VEC];
 #pragma unroll
         for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
-        for (int base = 0; base < longest; base += W) {
-            const bool mine = base + wl < len;
-            const int c = mine ? ci[e0 + base + wl] : 0;
-            const float a = mine ? val[e0 + base + wl] : 0.0f;
-            const int cnt = len - base;  // entries of this row left in the batch (may be <= 0 or > W)
-            for (int q = 0; q < W; q += S) {
-                int cc[U];
-                float aa[U];
+        int cur = -1;
+        for (int step = 0; step < steps; ++step) {
+            const int q0 = qa + step * U;
+            int cc[U], rr[U];
+            float aa[U];
 #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    cc[u] = __shfl(c, w0 + q + u * P + sub, kWave);
-                    aa[u] = __shfl(a, w0 + q + u * P + sub, kWave);
-                }
-                if (active) {
-                    float b[U][VEC];
+            for (int u = 0; u < U; ++u) {
+                const int q = q0 + u < qb ? q0 + u : 0;
+                cc[u] = __shfl(col, q, kWave);
+                aa[u] = __shfl(a, q, kWave);
+                rr[u] = __shfl(row_of, q, kWave);
+            }
+            float b[U][VEC];
 #pragma unroll
-                    for (int u = 0; u < U; ++u) {
+            for (int u = 0; u < U; ++u) {
 #pragma unroll
-                        for (int v = 0; v < VEC; ++v) b[u][v] = 0.0f;
-                        if (q + u * P + sub < cnt) load_vec<VEC>(B + (size_t)cc[u] * ldb + kbase, b[u]);
+                for (int v = 0; v < VEC; ++v) b[u][v] = 0.0f;
+                if (active && q0 + u < qb) load_vec<VEC>(B + (size_t)cc[u] * ldb + kbase, b[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (q0 + u < qb) {
+                    if (rr[u] != cur) {
+                        if (cur >= 0 && active) store_row<VEC>(seg.out(r0, cur), kbase, K, acc, alpha, beta);
+                        cur = rr[u];
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
                     }
 #pragma unroll
-                    for (int u = 0; u < U; ++u)
-#pragma unroll
-                        for (int v = 0; v < VEC; ++v) acc[v] = fmaf(aa[u], b[u][v], acc[v]);
+                    for (int v = 0; v < VEC; ++v) acc[v] = fmaf(aa[u], b[u][v], acc[v]);
                 }
             }
         }
+        if (cur >= 0 && active) store_row<VEC>(seg.out(r0, cur), kbase, K, acc, alpha, beta);
+        for (unsigned long long left = empty; left; left &= left - 1) {
+            const int j = __ffsll((long long)left) - 1;
 #pragma unroll
-        for (int off = G; off < W; off <<= 1)
-#pragma unroll
-            for (int v = 0; v < VEC; ++v) acc[v] += __shfl_xor(acc[v], off, kWave);
-        if (sub == 0 && active && r < n_rows && rp[r + 1] - rp[r] <= kSplitRow)
-            store_row<VEC>(C + (size_t)r * ldc, kbase, K, acc, alpha, beta);
+            for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
+            if (sub == 0 && active) store_row<VEC>(seg.out(r0, j), kbase, K, acc, alpha, beta);
+        }
     }
 }
 
@@ -569,18 +619,9 @@ void launch_spmm(const drone_spmm_plan *plan, const int *rp, const int *ci, cons
             plan->num_pieces, plan->piece_begin, plan->piece_end, plan->piece_slot, plan->ci2, plan->val2, B, ldb,
             plan->partial, plan->max_k, K);
     }
-    // rows per wavefront of the short-row kernel.  R-MAT scale 22, 90 M entries, K = 16 (lane groups of 4): 1 / 4 / 8
-    // rows 2.10 / 1.86 / 1.92 ms; two rows for lane groups of 16 lost: K = 64 4.03 against 3.65 ms, K = 41 2.57 against 2.45.
-    constexpr int R = G <= 4 ? 4 : G <= 8 ? 2 : 1;
-    const int blocks = (int)ceil_div(plan->n_rows, kRowsPerBlock * R);
-    if (blocks > 0) {
-        if constexpr (R > 1)
-            spmm_rows_multi_kernel<G, VEC, R><<<blocks, kWave * kRowsPerBlock, 0, s>>>(plan->n_rows, rp, ci, v, B, ldb, C,
-                                                                                      ldc, K, alpha, beta);
-        else
-            spmm_rows_kernel<G, VEC><<<blocks, kWave * kRowsPerBlock, 0, s>>>(plan->n_rows, rp, ci, v, B, ldb, C, ldc, K,
-                                                                             alpha, beta);
-    }
+    if (plan->num_chunks > 0)
+        spmm_chunks_kernel<G, VEC, RowSegments><<<(int)ceil_div(plan->num_chunks, kRowsPerBlock), kWave * kRowsPerBlock, 0, s>>>(
+            plan->num_chunks, plan->chunk_r0, plan->chunk_r1, RowSegments{rp, C, ldc, alpha, beta}, ci, v, B, ldb, K);
     if (plan->num_long > 0)  // also when every entry of the long rows went to the dense part: C = beta * C there
         spmm_combine_kernel<<<plan->num_long, 128, 0, s>>>(plan->num_long, plan->long_row, plan->first_slot,
                                                           plan->partial, plan->max_k, C, ldc, K, alpha, beta);
@@ -912,6 +953,34 @@ int plan_create(drone_spmm_plan **out, int n_rows, int n_cols, int64_t nnz, cons
         DRONE_REQUIRE(len >= 0, "row_ptr must be non-decreasing");
         if (len > kSplitRow) long_row.push_back(r);
     }
+    // chunks of the short rows
+    std::vector<int> h_c0, h_c1;
+    {
+        int first = -1, entries = 0;
+        const auto close = [&](int end) {
+            if (first >= 0) {
+                h_c0.push_back(first);
+                h_c1.push_back(end);
+            }
+            first = -1;
+            entries = 0;
+        };
+        for (int r = 0; r < n_rows; ++r) {
+            const int len = h_rp[r + 1] - h_rp[r];
+            if (len > kSplitRow) {  // a long row: not ours, and it ends the run
+                close(r);
+            } else if (len > kWave) {  // more than one load of pairs: a chunk of its own
+                close(r);
+                h_c0.push_back(r);
+                h_c1.push_back(r + 1);
+            } else {
+                if (first >= 0 && (entries + len > kWave || r - first >= kWave - 1)) close(r);
+                if (first < 0) first = r;
+                entries += len;
+            }
+        }
+        close(n_rows);
+    }
     bool scaled = row_scale != nullptr && col_scale != nullptr && !long_row.empty();
     if (scaled) {  // the bit core stands on value = row_scale * col_scale: check it, entry by entry
         unsigned *d_bad = nullptr, bad = 0;
@@ -934,6 +1003,18 @@ int plan_create(drone_spmm_plan **out, int n_rows, int n_cols, int64_t nnz, cons
         p->nnz = nnz;
         p->max_k = max_k;
         p->scaled = scaled;
+        p->num_chunks = (int)h_c0.size();
+        if (p->num_chunks > 0) {
+            const auto upload = [&]() -> int {
+                DRONE_HIP_TRY(hipMalloc(&p->chunk_r0, sizeof(int) * h_c0.size()));
+                DRONE_HIP_TRY(hipMalloc(&p->chunk_r1, sizeof(int) * h_c1.size()));
+                DRONE_HIP_TRY(hipMemcpy(p->chunk_r0, h_c0.data(), sizeof(int) * h_c0.size(), hipMemcpyHostToDevice));
+                DRONE_HIP_TRY(hipMemcpy(p->chunk_r1, h_c1.data(), sizeof(int) * h_c1.size(), hipMemcpyHostToDevice));
+                return DRONE_OK;
+            };
+            const int urc = upload();
+            if (urc != DRONE_OK) { drone_spmm_plan_destroy(p); return urc; }
+        }
         bool duplicates = false;
         int rc = DRONE_OK;
         if (scaled) {
@@ -998,6 +1079,8 @@ extern "C" int drone_spmm_plan_update_values(drone_spmm_plan *p, const float *v,
 extern "C" int drone_spmm_plan_destroy(drone_spmm_plan *p)
 {
     if (!p) return DRONE_OK;
+    (void)hipFree(p->chunk_r0);
+    (void)hipFree(p->chunk_r1);
     (void)hipFree(p->long_row);
     (void)hipFree(p->first_slot);
     (void)hipFree(p->piece_begin);

@@ -81,6 +81,32 @@ def test_spmm_against_oracle(T, oracle, K, ld_pad):
     assert np.all(got[np.diff(m.indptr) == 0] == 0.0)             # empty rows are written as zero (beta = 0)
 
 
+@pytest.mark.parametrize("K,ld_pad", [(5, 0), (16, 0), (41, 3), (64, 0), (128, 0), (300, 0)])
+def test_spmm_short_row_chunks(T, oracle, K, ld_pad):
+    """Row-length patterns around the limits of the short-row chunks (at most 64 entries and 63 rows per wavefront, a
+    row of more than 64 entries alone, long rows in between): runs of empty rows longer than a chunk, rows of exactly
+    64 / 65 entries, 63 and 64 one-entry rows in a row, a long row between short ones; beta != 0 so that empty rows
+    must come out as beta * C."""
+    lens = ([0] * 70 + [64, 65, 0, 64] + [1] * 63 + [2] + [1] * 64 + [32, 32, 1, 0, 0, 3] + [600] + [0, 5, 59, 1, 0] +
+            [512, 513, 7] + [0] * 130 + [63, 1, 1] + [10] * 20)
+    rng = np.random.default_rng(K)
+    n_cols = 700
+    rp = np.zeros(len(lens) + 1, np.int32)
+    rp[1:] = np.cumsum(lens)
+    ci = np.concatenate([np.sort(rng.choice(n_cols, size=l, replace=False)) for l in lens if l]).astype(np.int32)
+    val = rng.uniform(-1, 1, ci.size).astype(np.float32)
+    m = sp.csr_matrix((val, ci, rp), shape=(len(lens), n_cols))
+    B = rng.uniform(-1, 1, (n_cols, K)).astype(np.float32)
+    C0 = rng.uniform(-1, 1, (len(lens), K)).astype(np.float32)
+    for alpha, beta in ((1.0, 0.0), (0.5, -2.0)):
+        got = run_spmm(T, m, B, ld_pad=ld_pad, alpha=alpha, beta=beta, C0=C0)
+        ref = alpha * oracle.spmm_f64acc(rp, ci, val, B) + beta * C0
+        scale = abs(alpha) * oracle.spmm_f64acc(rp, ci, np.abs(val), np.abs(B)) + abs(beta) * np.abs(C0)
+        assert rel_err(got, ref, scale) <= 1e-4
+        empty = np.array(lens) == 0
+        np.testing.assert_array_equal(got[empty], (beta * C0[empty]).astype(np.float32))
+
+
 @pytest.mark.parametrize("K", [8, 16, 41, 64, 128, 256])
 def test_spmm_long_rows_split_and_alpha_beta(T, oracle, K):
     """Rows above 512 entries take the band path: several of them, several column bands (a band holds
