@@ -206,8 +206,8 @@ int drone_gcn_edge_values(int n, const int *rp, const int *ci, const int *in_deg
  * ascend within each output row.  v / vT may both be NULL (pattern only).  Synchronises `stream`. */
 int drone_csr_transpose_f32(int n_rows, int n_cols, int64_t nnz, const int *rp, const int *ci,
                             const float *v, int *rpT, int *ciT, float *vT, drone_stream_t stream);
-/* Schedule for the SpMM of one CSR with feature widths up to max_k.  Rows of at most 512 entries run one
- * wavefront each.  Longer rows are cut by column band (columns ranked by frequency; a band's feature rows fill
+/* Schedule for the SpMM of one CSR with feature widths up to max_k.  Rows of at most 512 entries run in row
+ * order, one wavefront per chunk of consecutive rows that hold at most 64 entries together.  Longer rows are cut by column band (columns ranked by frequency; a band's feature rows fill
  * about 2 MB of L2) and the plan keeps a (band,row)-sorted copy of their entries - columns AND values as
  * passed here - plus the scratch for their partial rows.  Where the longest rows meet the most frequent
  * columns densely enough (at least 12 % of the cells of a 2048-column chunk), those entries are stored as dense
