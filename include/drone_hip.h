@@ -214,7 +214,10 @@ int drone_csr_transpose_f32(int n_rows, int n_cols, int64_t nnz, const int *rp, 
  * fp32 rectangles instead and multiplied on the matrix cores (drone_spmm_plan_info reports how much).  The rp / ci / v later passed to
  * drone_spmm_csr_f32 must be the arrays the plan was built from; after changing values in place call
  * drone_spmm_plan_update_values.  Set-up step (the counterpart of cusparseSpMM_bufferSize + the
- * preprocessing cuSPARSE hides, cuda_module.cu:232-243); synchronises `stream`. */
+ * preprocessing cuSPARSE hides, cuda_module.cu:232-243); synchronises `stream`.
+ * One difference from a purely sparse product: inside a dense region every cell is multiplied, empty ones by 0, so a
+ * NaN or an infinity in a row of B reaches every row of C that the region spans, not only the rows that hold an entry
+ * in that column (finite inputs are not affected; values within 0.4 % of FLT_MAX count as infinite for a scaled plan). */
 typedef struct drone_spmm_plan drone_spmm_plan;
 int drone_spmm_plan_create(drone_spmm_plan **plan, int n_rows, int n_cols, int64_t nnz, const int *rp,
                            const int *ci, const float *v, int max_k, drone_stream_t stream);
