@@ -109,7 +109,8 @@ __device__ __forceinline__ bf16x8 expand_bits(unsigned byte)
 //  * the stage's global loads issued by hand at the top of the stage (see below): 0.83 -> 0.61;
 //  * a wavefront expands a byte of bits into 8 bf16 values with 16 vector instructions, so every expansion must feed
 //    many matrix instructions: 2 row groups x NT tiles per wavefront (an expansion per 3 NT instructions) instead of
-//    4 x NT / 2 (one per 1.5 NT).
+//    4 x NT / 2 (one per 1.5 NT).  A 256-entry table of expanded bytes in LDS instead of the 16 instructions measured 0.573
+//    against 0.595 ms with every lane reading the same entry (no bank conflicts), too little to carry real patterns.
 template <int NT>
 __global__ __launch_bounds__(512, 1) void bits_mfma_kernel(const int *__restrict__ unit_tile,
                                                            const int *__restrict__ unit_c0,
