@@ -196,7 +196,8 @@ int drone_pr_run_workers_f64(Graph *g, PRValues *values, int workerId, int worke
  * int32 offsets / int32 columns / fp32 values, base 0 - the descriptors of cuda_module.cu:166-194.
  * Calls are asynchronous on `stream`.  Apart from plan creation, the transpose (a set-up step) and
  * grow-only scratch kept per (device, stream) by drone_sgemm_rm_f32 (split reductions) and
- * drone_cross_entropy_f32, nothing allocates; calls on different streams may overlap. */
+ * drone_cross_entropy_f32, nothing allocates; calls on different streams may overlap, except that two products with
+ * the SAME plan share the plan's partial-row scratch and must not run at the same time. */
 
 /* cuda_gcn/src/cuda/cuda_kernel.cu:145-155 (launched at cuda_module.cu:163):
  * v[e(u->col)] = 1 / sqrtf(1.0 * out_deg[u] * in_deg[col]) for every entry of row u. */
@@ -208,10 +209,12 @@ int drone_csr_transpose_f32(int n_rows, int n_cols, int64_t nnz, const int *rp, 
                             const float *v, int *rpT, int *ciT, float *vT, drone_stream_t stream);
 /* Schedule for the SpMM of one CSR with feature widths up to max_k.  Rows of at most 512 entries run in row
  * order, one wavefront per chunk of consecutive rows that hold at most 64 entries together.  Longer rows are cut by column band (columns ranked by frequency; a band's feature rows fill
- * about 2 MB of L2) and the plan keeps a (band,row)-sorted copy of their entries - columns AND values as
+ * about 3 MB of L2) and the plan keeps a (band,row)-sorted copy of their entries - columns AND values as
  * passed here - plus the scratch for their partial rows.  Where the longest rows meet the most frequent
  * columns densely enough (at least 12 % of the cells of a 2048-column chunk), those entries are stored as dense
- * fp32 rectangles instead and multiplied on the matrix cores (drone_spmm_plan_info reports how much).  The rp / ci / v later passed to
+ * fp32 rectangles instead and multiplied on the matrix cores (drone_spmm_plan_info reports how much; a dense part is
+ * only made when its estimated gain exceeds 0.25 ms per product, DRONE_SPMM_DENSE_MIN_GAIN_MS=<ms> in the environment
+ * at creation replaces that figure).  The rp / ci / v later passed to
  * drone_spmm_csr_f32 must be the arrays the plan was built from; after changing values in place call
  * drone_spmm_plan_update_values.  Set-up step (the counterpart of cusparseSpMM_bufferSize + the
  * preprocessing cuSPARSE hides, cuda_module.cu:232-243); synchronises `stream`.
