@@ -583,7 +583,7 @@ def main():
                      "traffic": pr_traffic_from_profile() if (args.scale == 24 and n == 16777216) else None,
                      "traffic_source": "profiles/pr_rowblock_pagerank_c2.hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / "
                                        "WRITE_SIZE of this command, scaled by the 1 GiB copy kernel)",
-                     "kernel": "one iteration: " + " + ".join(PR_KERNELS) + " + row fix-up + dangling-mass reduction",
+                     "kernel": "one iteration: " + " + ".join(PR_KERNELS) + " + row fix-up (whose last work-group reduces the dangling mass)",
                      "algorithmic_bytes_per_launch": bytes_iter, "mean_launch_ms": prof["mean_ms"],
                      "launches_timed": prof["launches"]},
         "plan_ms_one_off": plan_s * 1e3,

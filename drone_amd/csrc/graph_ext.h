@@ -88,6 +88,8 @@ void ensure_aggregation_ready(Graph *g);
 struct PRExt {
     float *push = nullptr;        // device [n]: value each vertex pushes along its out-edges this step
     double *stat = nullptr;       // device scalar: statistic of the last launch
+    double *stat_host = nullptr;  // pinned host word that the aggregation's last work-group writes the same value to
+    unsigned int *ticket = nullptr;  // device counter of the vertex kernel's last_block_done
     double *block_part = nullptr; // device [vertex_blocks]
     int vertex_blocks = 0;
 };

@@ -79,17 +79,17 @@ __global__ __launch_bounds__(kSpmvBlock) void pr_f64_count_idle_dangling_kernel(
     if (threadIdx.x == 0) block_count[blockIdx.x] = total;  // summed by reduce_stat_kernel
 }
 
-// dang[0] = sum of the blocks' statistics + idle[0] * base_k (dang[0] still holds dang_{k-1} when this runs).
-__global__ __launch_bounds__(kSpmvBlock) void pr_f64_reduce_dangling_kernel(const double *__restrict__ in, int count,
-                                                                            const double *__restrict__ idle, double alpha,
-                                                                            double inv_n, double *__restrict__ dang)
-{
-    __shared__ double s_red[kSpmvBlock / kWave];
-    double v = 0.0;
-    for (int k = threadIdx.x; k < count; k += kSpmvBlock) v += in[k];
-    const double total = block_sum_256(v, s_red);
-    if (threadIdx.x == 0) dang[0] = total + idle[0] * ((1.0 - alpha) * inv_n + alpha * dang[0] * inv_n);
-}
+// What the fix-up's last work-group does with the sweep's dangling mass: dang[0] = total + idle[0] * base_k (dang[0]
+// still holds dang_{k-1} at that point: every work-group has finished reading it).
+struct DanglingFinish {
+    const double *idle;
+    double alpha, inv_n;
+    double *dang;
+    __device__ __forceinline__ void operator()(double total) const
+    {
+        dang[0] = total + idle[0] * ((1.0 - alpha) * inv_n + alpha * dang[0] * inv_n);
+    }
+};
 
 // Last iteration: the isolated vertices' ranks, r_out[order[i]] = base_k for i in [live, n).
 __global__ void pr_f64_idle_ranks_kernel(int64_t live, int64_t n, const int32_t *__restrict__ order,
@@ -323,13 +323,12 @@ extern "C" int drone_pr_run_f64(drone_pr_plan *p, double alpha, int iters, doubl
                     p->rb.split_block, p->rb.block_row, p->rb.block_units, p->rb.block_partial, p->rb.partial, epi, carry,
                     p->ms.tile_stat);
         }
-        spmv_fixup_kernel<double, PrF64Epi><<<fb, kSpmvBlock, 0, s>>>(
-            p->units, p->deterministic ? p->mt.tile_row : p->rb.block_row,
-            p->deterministic ? p->mt.walk_len : p->rb.walk_len, carry, p->ms.tile_stat, epi, p->ms.block_stat);
-        if (epi.r_out && p->rows < p->n)
+        if (epi.r_out && p->rows < p->n)  // reads dang_{k-1}, which the fix-up's last work-group replaces
             pr_f64_idle_ranks_kernel<<<1024, 256, 0, s>>>(p->rows, p->n, p->rl.order, p->dang, alpha, inv_n, rank_out);
-        // dang is read by the kernels above and overwritten here, in stream order
-        pr_f64_reduce_dangling_kernel<<<1, kSpmvBlock, 0, s>>>(p->ms.block_stat, fb, p->idle, alpha, inv_n, p->dang);
+        spmv_fixup_kernel<double, PrF64Epi, DanglingFinish><<<fb, kSpmvBlock, 0, s>>>(
+            p->units, p->deterministic ? p->mt.tile_row : p->rb.block_row,
+            p->deterministic ? p->mt.walk_len : p->rb.walk_len, carry, p->ms.tile_stat, epi, p->ms.block_stat,
+            p->ms.ticket, DanglingFinish{p->idle, alpha, inv_n, p->dang});
         if (prof) DRONE_HIP_TRY(hipEventRecord(p->ev1[p->prof_n++], s));  // the whole iteration, small kernels included
     }
     DRONE_HIP_TRY(hipGetLastError());

@@ -82,24 +82,18 @@ __global__ __launch_bounds__(kSpmvBlock) void pr_init_vertex_kernel(
     if (threadIdx.x == 0) block_part[blockIdx.x] = total;
 }
 
-// pr.cu:430-448 (thread 0): globalAcc += globalDiff; globalDiff = 0
-__global__ void pr_fold_global_kernel(float *global_acc, float *global_diff)
-{
-    if (blockIdx.x == 0 && threadIdx.x == 0) {
-        *global_acc += *global_diff;
-        *global_diff = 0.0f;
-    }
-}
-
-// pr.cu:430-448 (per vertex) fused with pr.cu:51-87 without the edge loop.
+// pr.cu:430-448 fused with pr.cu:51-87 without the edge loop.  The reference's thread 0 folds the global diff
+// (globalAcc += globalDiff; globalDiff = 0) while the other threads already read globalAcc; here every work-group
+// computes the folded value itself and the last one to finish stores it, together with the new global diff: the sum of
+// the work-groups' dangling mass, added in index order.
 __global__ __launch_bounds__(kSpmvBlock) void pr_increment_vertex_kernel(
     int n, int nglobal, const int *__restrict__ outdeg, const int *__restrict__ m2w, float *__restrict__ pr,
-    float *__restrict__ acc, const float *__restrict__ diff, const float *__restrict__ global_acc,
+    float *__restrict__ acc, const float *__restrict__ diff, float *global_acc, float *global_diff,
     float *__restrict__ push, const int32_t *__restrict__ push_slot, int *__restrict__ update_by_message,
-    double *__restrict__ block_part)
+    double *block_part, unsigned int *ticket)
 {
     __shared__ double s_red[kSpmvBlock / kWave];
-    const float ga = *global_acc;
+    const float ga = *global_acc + *global_diff;
     double part = 0.0;
     for (int id = blockIdx.x * kSpmvBlock + threadIdx.x; id < n; id += gridDim.x * kSpmvBlock) {
         update_by_message[id] = 0;
@@ -122,7 +116,14 @@ __global__ __launch_bounds__(kSpmvBlock) void pr_increment_vertex_kernel(
         push[push_slot ? push_slot[id] : id] = out;
     }
     const double total = block_sum_256(part, s_red);
-    if (threadIdx.x == 0) block_part[blockIdx.x] = total;
+    unsigned int one = 0;
+    if (threadIdx.x == 0) one = publish_part(block_part + blockIdx.x, total);
+    if (!last_block_done(ticket, one)) return;
+    const double all = block_sum_of_parts(block_part, (int)gridDim.x, s_red);
+    if (threadIdx.x == 0) {
+        *global_acc = ga;
+        *global_diff = (float)all;
+    }
 }
 
 // globalDiff += (float) sum of block partials, fixed order
@@ -182,13 +183,13 @@ void exchange_push(Graph *g, PRValues *values, int workerId, int workerNum, Comm
 }
 
 // Subgraphs with at least this many edges get source-sorted row blocks for the aggregation.  One superstep at
-// R-MAT scale 20 / 21 / 22 / 23 / 24 (16 ... 263 M edges) takes 0.13 / 0.17 / 0.24 / 0.38 / 0.70 ms with them and
-// 0.12 / 0.20 / 0.39 / 0.78 / 1.65 ms on the merge path; building them at the first PR_PEVal costs 8 / 12 / 18 ms
-// at scale 22 / 23 / 24 (and 15 ms more in a process that has not run these kernels yet), i.e. 55 / 30 / 23
-// supersteps' worth of the saving.  The default keeps the merge path (whose sums are also added in a fixed order)
-// until a PageRank run of fifty to a hundred supersteps gets the build back; DRONE_PR_ROWBLOCK_MIN_EDGES in the
-// environment moves the limit for jobs that run longer or shorter.
-constexpr int64_t kRowBlockMinEdges = 64ll << 20;
+// R-MAT scale 20 / 21 / 22 / 23 / 24 (16 ... 263 M edges) takes 0.087 / 0.125 / 0.20 / 0.36 / 0.68 ms with them and
+// 0.107 / 0.187 / 0.37 / 0.78 / 1.65 ms on the merge path; building them at the first PR_PEVal costs 8 / 12 / 18 ms
+// at scale 22 / 23 / 24 (and 15 ms more in a process that has not run these kernels yet), i.e. 46 / 29 / 19
+// supersteps' worth of the saving, and about 90 at scale 21.  The default keeps the merge path (whose sums are also
+// added in a fixed order) until a PageRank run of about fifty supersteps gets the build back;
+// DRONE_PR_ROWBLOCK_MIN_EDGES in the environment moves the limit for jobs that run longer or shorter.
+constexpr int64_t kRowBlockMinEdges = 48ll << 20;
 
 int64_t row_block_min_edges()
 {
@@ -285,17 +286,16 @@ int aggregate_push(Graph *g, PRValues *values, hipStream_t s)
             pr_rowblock_merge_kernel<PushEpi><<<dim3((unsigned)rb.num_split, (unsigned)(kRbRows / kRbThreads + 1)), kRbThreads, 0, s>>>(
                 rb.split_block, rb.block_row, rb.block_units, rb.block_partial, partial, epi, carry, x->ms_rb.tile_stat);
         const int fb = fixup_blocks(rb.num_blocks);
-        spmv_fixup_kernel<PushF2, PushEpi><<<fb, kSpmvBlock, 0, s>>>(rb.num_blocks, rb.block_row, rb.walk_len, carry,
-                                                                    x->ms_rb.tile_stat, epi, x->ms_rb.block_stat);
-        reduce_stat_kernel<0><<<1, kSpmvBlock, 0, s>>>(x->ms_rb.block_stat, fb, px->stat);
+        spmv_fixup_kernel<PushF2, PushEpi, StoreStat><<<fb, kSpmvBlock, 0, s>>>(
+            rb.num_blocks, rb.block_row, rb.walk_len, carry, x->ms_rb.tile_stat, epi, x->ms_rb.block_stat,
+            x->ms_rb.ticket, StoreStat{px->stat, px->stat_host});
     } else {
-        spmv_merge_launch<PushF2, int, kPushIpt, PushEpi>(x->mt, x->ms, x->in_index, x->in_src, epi, px->stat, s);
+        spmv_merge_launch<PushF2, int, kPushIpt, PushEpi>(x->mt, x->ms, x->in_index, x->in_src, epi, px->stat, s,
+                                                          px->stat_host);
     }
     DRONE_HIP_OR_DIE(hipGetLastError());
-    double visited = 0.0;
-    DRONE_HIP_OR_DIE(hipMemcpyAsync(&visited, px->stat, sizeof(double), hipMemcpyDeviceToHost, s));
-    DRONE_HIP_OR_DIE(hipStreamSynchronize(s));
-    return (int)visited;
+    DRONE_HIP_OR_DIE(hipStreamSynchronize(s));  // the fix-up's last work-group has written the count to the host
+    return (int)*px->stat_host;
 }
 
 }  // namespace
@@ -362,9 +362,12 @@ extern "C" Response PR_PEVal(Graph *g, PRValues *values, int workerId, int worke
         PRExt *px = new PRExt();
         DRONE_HIP_OR_DIE(hipMalloc(&px->push, sizeof(float) * cnt));
         DRONE_HIP_OR_DIE(hipMalloc(&px->stat, sizeof(double)));
+        DRONE_HIP_OR_DIE(hipHostMalloc(&px->stat_host, sizeof(double)));
         px->vertex_blocks = (int)ceil_div(cnt, kSpmvBlock * 4);
         if (px->vertex_blocks > 4096) px->vertex_blocks = 4096;
         DRONE_HIP_OR_DIE(hipMalloc(&px->block_part, sizeof(double) * (size_t)px->vertex_blocks));
+        DRONE_HIP_OR_DIE(hipMalloc(&px->ticket, sizeof(unsigned int) * ticket_words(px->vertex_blocks)));
+        DRONE_HIP_OR_DIE(hipMemsetAsync(px->ticket, 0, sizeof(unsigned int) * ticket_words(px->vertex_blocks), s));
         values->ext = px;
         // exchange staging (pr.cu:402-405) is allocated by the first exchange; with one subgraph it stays null
     }
@@ -403,11 +406,10 @@ extern "C" Response PR_IncEVal(Graph *g, PRValues *values, int workerId, int wor
     }
     PRExt *px = static_cast<PRExt *>(values->ext);
     const int n = getLocalVertexSize(g), nglobal = getGlobalVertexSize(g);
-    pr_fold_global_kernel<<<1, 64, 0, s>>>(values->globalAcc, values->globalDiff);
     pr_increment_vertex_kernel<<<px->vertex_blocks, kSpmvBlock, 0, s>>>(
         n, nglobal, values->outDegree, g->Mirror2Worker, values->prValue, values->accValue, values->diffValue,
-        values->globalAcc, px->push, push_slot_of(g), g->updateByMessage, px->block_part);
-    pr_add_global_diff_kernel<<<1, kSpmvBlock, 0, s>>>(px->block_part, px->vertex_blocks, values->globalDiff);
+        values->globalAcc, values->globalDiff, px->push, push_slot_of(g), g->updateByMessage, px->block_part,
+        px->ticket);
     res.VisitedSize = aggregate_push(g, values, s);
     res.LocalVertexSize = n;
     res.CalTime = (float)seconds_since(t0);
@@ -425,6 +427,8 @@ extern "C" void drone_pr_values_destroy(Graph *g, PRValues *values)
     if (px) {
         (void)hipFree(px->push);
         (void)hipFree(px->stat);
+        if (px->stat_host) (void)hipHostFree(px->stat_host);
+        (void)hipFree(px->ticket);
         (void)hipFree(px->block_part);
         delete px;
     }

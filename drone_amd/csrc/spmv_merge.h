@@ -252,13 +252,88 @@ __global__ __launch_bounds__(kSpmvBlock) void spmv_merge_kernel(
     if (tid == 0) tile_stat[t] = total;
 }
 
+// Hand-over of per-work-group partial results to the last work-group of the same launch, without a device-wide fence
+// (on this GPU a fence at device scope writes back a whole L2, once per work-group that executes it: a vertex kernel of
+// 4096 work-groups took twice its time).  Thread 0 of every work-group stores its part with publish_part - an atomic
+// exchange at device scope, performed where all XCDs see it, whose return value is waited for - and then takes a
+// ticket; the work-group that draws the last ticket reads the parts with load_agent.  Nothing else the other
+// work-groups wrote is guaranteed to be visible to it.
+__device__ __forceinline__ unsigned int publish_part(double *slot, double v)
+{
+    const unsigned long long old =
+        __hip_atomic_exchange(reinterpret_cast<unsigned long long *>(slot), (unsigned long long)__double_as_longlong(v),
+                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    unsigned int one = 1u;
+    asm volatile("" : "+v"(one) : "v"((unsigned int)old));  // the ticket's increment exists once the exchange has returned
+    return one;
+}
+
+// True in every thread of the work-group whose thread 0 draws the last ticket of the launch.  Tickets are drawn in
+// two levels - 64 work-groups share a counter, the last of each 64 draws from the launch's counter - because atomics on
+// ONE address take about 5 ns each here (4096 work-groups on a single counter doubled a 20 us kernel).  `ticket`:
+// ticket_words(work-groups of the launch) device words, zero before the launch; the last drawers set them back, so
+// consecutive launches on one stream can share them.  `one`: what publish_part returned to thread 0.
+constexpr int kTicketGroup = 64;   // work-groups per first-level counter
+constexpr int kTicketStride = 32;  // words between counters: a cache line each
+inline size_t ticket_words(int64_t max_blocks)
+{
+    return (size_t)(ceil_div(max_blocks > 0 ? max_blocks : 1, kTicketGroup) + 1) * kTicketStride;
+}
+__device__ __forceinline__ bool last_block_done(unsigned int *ticket, unsigned int one)
+{
+    __shared__ int s_last;
+    if (threadIdx.x == 0) {
+        const unsigned int blocks = gridDim.x * gridDim.y * gridDim.z;
+        const unsigned int b = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+        const unsigned int group = b / kTicketGroup, groups = (blocks + kTicketGroup - 1) / kTicketGroup;
+        const unsigned int in_group = group + 1 < groups ? kTicketGroup : blocks - group * kTicketGroup;
+        unsigned int *mine = ticket + (size_t)(group + 1) * kTicketStride;
+        bool last = false;
+        if (atomicAdd(mine, one) == in_group - 1) {  // returns before the next draw is issued
+            atomicExch(mine, 0u);
+            last = atomicAdd(ticket, 1u) == groups - 1;
+            if (last) atomicExch(ticket, 0u);
+        }
+        s_last = last;
+    }
+    __syncthreads();
+    return s_last != 0;
+}
+
+// A load that does not take its value from this CU's L1 or this XCD's L2 (another work-group published it).
+__device__ __forceinline__ double load_agent(const double *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Sum of in[0..count) over the block in a fixed order (thread k takes k, k + 256, ...), valid in thread 0.
+__device__ __forceinline__ double block_sum_of_parts(const double *in, int count, double *s_red)
+{
+    double v = 0.0;
+    for (int k = threadIdx.x; k < count; k += kSpmvBlock) v += load_agent(in + k);
+    return block_sum_256(v, s_red);
+}
+
+// What the last work-group of spmv_fixup_kernel does with the launch's statistic: store it on the device and, when
+// `host` is set, in pinned host memory as well (the caller then only has to wait for the stream).
+struct StoreStat {
+    double *out;
+    double *host;
+    __device__ __forceinline__ void operator()(double total) const
+    {
+        out[0] = total;
+        if (host) host[0] = total;
+    }
+};
+
 // Completes rows that cross tile boundaries and folds the per-tile statistics:
-// block_stat[b] = sum over the block's tiles of (tile_stat + what Epi::fix added).
-template <typename V, typename Epi>
+// block_stat[b] = sum over the block's tiles of (tile_stat + what Epi::fix added); the last work-group to finish adds
+// the blocks' statistics in index order and hands the sum to `finish` (thread 0).
+template <typename V, typename Epi, typename Finish>
 __global__ __launch_bounds__(kSpmvBlock) void spmv_fixup_kernel(
     int num_tiles, const int32_t *__restrict__ tile_row, const int32_t *__restrict__ walk_len,
-    const V *__restrict__ tile_carry, const double *__restrict__ tile_stat, Epi epi,
-    double *__restrict__ block_stat)
+    const V *__restrict__ tile_carry, const double *__restrict__ tile_stat, Epi epi, double *block_stat,
+    unsigned int *ticket, Finish finish)
 {
     __shared__ double s_red[kSpmvBlock / kWave];
     const int t = (blockIdx.x * kSpmvBlock + threadIdx.x) / kFixGroup;
@@ -277,7 +352,11 @@ __global__ __launch_bounds__(kSpmvBlock) void spmv_fixup_kernel(
         stat += tile_stat[t];
     }
     const double total = block_sum_256(stat, s_red);
-    if (threadIdx.x == 0) block_stat[blockIdx.x] = total;
+    unsigned int one = 0;
+    if (threadIdx.x == 0) one = publish_part(block_stat + blockIdx.x, total);
+    if (!last_block_done(ticket, one)) return;
+    const double all = block_sum_of_parts(block_stat, (int)gridDim.x, s_red);
+    if (threadIdx.x == 0) finish(all);
 }
 
 // out[0] = sum of in[0..count) by one block, fixed order.
@@ -331,6 +410,7 @@ struct MergeScratch {
     void *tile_carry = nullptr;    // V [num_tiles]
     double *tile_stat = nullptr;   // [num_tiles]
     double *block_stat = nullptr;  // [fixup_blocks]
+    unsigned int *ticket = nullptr;  // [ticket_words(fixup_blocks)] counters of last_block_done, zero between launches
 };
 
 inline int merge_scratch_create(MergeScratch *ms, const MergeTiling &mt, size_t value_bytes)
@@ -338,6 +418,10 @@ inline int merge_scratch_create(MergeScratch *ms, const MergeTiling &mt, size_t 
     DRONE_HIP_TRY(hipMalloc(&ms->tile_carry, value_bytes * (size_t)mt.num_tiles));
     DRONE_HIP_TRY(hipMalloc(&ms->tile_stat, sizeof(double) * (size_t)mt.num_tiles));
     DRONE_HIP_TRY(hipMalloc(&ms->block_stat, sizeof(double) * (size_t)fixup_blocks(mt.num_tiles)));
+    const size_t words = ticket_words(fixup_blocks(mt.num_tiles));
+    DRONE_HIP_TRY(hipMalloc(&ms->ticket, sizeof(unsigned int) * words));
+    DRONE_HIP_TRY(hipMemset(ms->ticket, 0, sizeof(unsigned int) * words));
+    DRONE_HIP_TRY(hipStreamSynchronize(nullptr));  // the first launch may be on any stream
     return DRONE_OK;
 }
 
@@ -346,21 +430,24 @@ inline void merge_scratch_destroy(MergeScratch *ms)
     if (ms->tile_carry) (void)hipFree(ms->tile_carry);
     if (ms->tile_stat) (void)hipFree(ms->tile_stat);
     if (ms->block_stat) (void)hipFree(ms->block_stat);
+    if (ms->ticket) (void)hipFree(ms->ticket);
     *ms = MergeScratch{};
 }
 
-// One aggregation: main kernel, boundary fix-up, statistic reduction into stat_out[0] (device).
+// One aggregation: main kernel and boundary fix-up, whose last work-group leaves the statistic in stat_out[0] (device)
+// and, when stat_host is given, in that pinned host word too.
 template <typename V, typename OffT, int IPT, typename Epi>
 void spmv_merge_launch(const MergeTiling &mt, const MergeScratch &ms, const OffT *row_ptr,
-                       const int32_t *col, const Epi &epi, double *stat_out, hipStream_t stream)
+                       const int32_t *col, const Epi &epi, double *stat_out, hipStream_t stream,
+                       double *stat_host = nullptr)
 {
     V *carry = static_cast<V *>(ms.tile_carry);
     spmv_merge_kernel<V, OffT, IPT, Epi><<<mt.num_tiles, kSpmvBlock, 0, stream>>>(
         mt.n, mt.nnz, mt.tile_row, row_ptr, col, epi, carry, ms.tile_stat);
     const int fb = fixup_blocks(mt.num_tiles);
-    spmv_fixup_kernel<V, Epi><<<fb, kSpmvBlock, 0, stream>>>(mt.num_tiles, mt.tile_row, mt.walk_len, carry,
-                                                            ms.tile_stat, epi, ms.block_stat);
-    reduce_stat_kernel<0><<<1, kSpmvBlock, 0, stream>>>(ms.block_stat, fb, stat_out);
+    spmv_fixup_kernel<V, Epi, StoreStat><<<fb, kSpmvBlock, 0, stream>>>(
+        mt.num_tiles, mt.tile_row, mt.walk_len, carry, ms.tile_stat, epi, ms.block_stat, ms.ticket,
+        StoreStat{stat_out, stat_host});
 }
 
 }  // namespace drone

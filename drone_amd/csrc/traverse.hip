@@ -128,11 +128,6 @@ __global__ __launch_bounds__(kSpmvBlock) void count_active_kernel(int n, const i
     if (threadIdx.x == 0) block_part[blockIdx.x] = total;
 }
 
-__global__ void clear_counters_kernel(unsigned long long *c)
-{
-    if (threadIdx.x < 2 && blockIdx.x == 0) c[threadIdx.x] = 0ull;
-}
-
 __global__ void iota_kernel(int *out, int n)
 {
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) out[i] = i;
@@ -159,14 +154,19 @@ __global__ void gather_len_kernel(int n, const int *__restrict__ eid, const floa
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) out[i] = len[eid[i]];
 }
 
+// Launches of at most this many work-groups hand their counters to the host themselves (publish_counters); larger
+// ones - push rounds over a long list of hubs - leave them to a copy.
+constexpr int kPublishMaxBlocks = 16384;
+
 // Per-call scratch of the traversals, hung off CCValues::ext / SSSPValues::ext.
 struct TraverseExt {
     double *stat = nullptr;        // device scalar
     double *block_part = nullptr;  // device [blocks]
     int blocks = 0;
     int *frontier[2] = {nullptr, nullptr};  // device [n] each: vertex lists of the push rounds
-    unsigned long long *counters = nullptr; // device [2]: {vertices << 32 | out-edges, largest out-degree} of the list being built
-    unsigned long long *host = nullptr;     // pinned [2]: landing place of the statistic and of the counters
+    unsigned long long *counters = nullptr; // device [2]: {vertices << 32 | out-edges, largest out-degree} of the list being built; zero between launches
+    unsigned int *ticket = nullptr;         // device [ticket_words(kPublishMaxBlocks)]: counters of last_block_done, zero between launches
+    unsigned long long *host = nullptr;     // pinned [2]: where the kernels' last work-groups leave the statistic / the counters
 };
 
 double seconds_since(std::chrono::steady_clock::time_point t0)
@@ -190,6 +190,10 @@ TraverseExt *traverse_ext_create(int n)
     DRONE_HIP_OR_DIE(hipMalloc(&t->frontier[0], sizeof(int) * (size_t)(n > 0 ? n : 1)));
     DRONE_HIP_OR_DIE(hipMalloc(&t->frontier[1], sizeof(int) * (size_t)(n > 0 ? n : 1)));
     DRONE_HIP_OR_DIE(hipMalloc(&t->counters, sizeof(unsigned long long) * 2));
+    DRONE_HIP_OR_DIE(hipMemset(t->counters, 0, sizeof(unsigned long long) * 2));
+    DRONE_HIP_OR_DIE(hipMalloc(&t->ticket, sizeof(unsigned int) * ticket_words(kPublishMaxBlocks)));
+    DRONE_HIP_OR_DIE(hipMemset(t->ticket, 0, sizeof(unsigned int) * ticket_words(kPublishMaxBlocks)));
+    DRONE_HIP_OR_DIE(hipStreamSynchronize(nullptr));  // the kernels that count may run on any stream
     DRONE_HIP_OR_DIE(hipHostMalloc(&t->host, sizeof(unsigned long long) * 2));
     return t;
 }
@@ -203,21 +207,24 @@ void traverse_ext_destroy(void *ext)
     (void)hipFree(t->frontier[0]);
     (void)hipFree(t->frontier[1]);
     (void)hipFree(t->counters);
+    (void)hipFree(t->ticket);
     (void)hipHostFree(t->host);
     delete t;
 }
 
+// Where a sweep's fix-up leaves its statistic for the host.
+double *stat_landing(TraverseExt *t) { return reinterpret_cast<double *>(t->host); }
+
+// The statistic of the last sweep (or of reduce_parts): its kernel wrote it to pinned memory, so waiting is enough.
 double read_stat(TraverseExt *t, hipStream_t s)
 {
-    double *landing = reinterpret_cast<double *>(t->host);  // pinned: the copy does not go through a staging buffer
-    DRONE_HIP_OR_DIE(hipMemcpyAsync(landing, t->stat, sizeof(double), hipMemcpyDeviceToHost, s));
     DRONE_HIP_OR_DIE(hipStreamSynchronize(s));
-    return *landing;
+    return *stat_landing(t);
 }
 
 double reduce_parts(TraverseExt *t, hipStream_t s)
 {
-    reduce_stat_kernel<0><<<1, kSpmvBlock, 0, s>>>(t->block_part, t->blocks, t->stat);
+    reduce_stat_kernel<0><<<1, kSpmvBlock, 0, s>>>(t->block_part, t->blocks, stat_landing(t));
     return read_stat(t, s);
 }
 
@@ -280,18 +287,34 @@ __device__ __forceinline__ void frontier_append(bool take, int v, int degree, in
     unsigned long long base = 0;
     if (lane == leader) {
         base = atomicAdd(counters, ((unsigned long long)__popcll(mask) << 32) + sum) >> 32;
-        if ((unsigned long long)mx > __atomic_load_n(counters + 1, __ATOMIC_RELAXED))
-            atomicMax(counters + 1, (unsigned long long)mx);
+        if ((unsigned long long)mx > __atomic_load_n(counters + 1, __ATOMIC_RELAXED)) {
+            // waited for, like the add above: publish_counters reads the word once every work-group has its ticket
+            const unsigned long long seen = atomicMax(counters + 1, (unsigned long long)mx);
+            asm volatile("" ::"v"((unsigned int)seen));
+        }
     }
     base = __shfl(base, leader, kWave);
     if (take) list[base + __popcll(mask & ((1ull << lane) - 1ull))] = v;
+}
+
+// The last work-group of a launch that built a list hands {count << 32 | edges, largest degree} to the host (pinned
+// memory) and clears the counters for the next launch.  ticket == nullptr: the host copies and clears them.
+__device__ __forceinline__ void publish_counters(unsigned long long *counters, unsigned int *ticket,
+                                                 unsigned long long *host)
+{
+    if (ticket == nullptr) return;
+    __syncthreads();  // every wavefront of the work-group has issued its appends (their atomics return before they go on)
+    if (!last_block_done(ticket, 1u) || threadIdx.x != 0) return;
+    host[0] = __hip_atomic_exchange(counters, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    host[1] = __hip_atomic_exchange(counters + 1, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // list <- vertices whose active flag equals `value`.  A work-group first compacts its matches in LDS, then the
 // first wavefront appends them, so the shared counter sees one atomic per 256 vertices that hold a match.
 __global__ __launch_bounds__(kSpmvBlock) void collect_frontier_kernel(int n, const int *__restrict__ active, int value,
                                                                       const int *__restrict__ index, int *__restrict__ list,
-                                                                      unsigned long long *__restrict__ counters)
+                                                                      unsigned long long *counters, unsigned int *ticket,
+                                                                      unsigned long long *host)
 {
     __shared__ int s_v[kSpmvBlock];
     __shared__ int s_count;
@@ -311,6 +334,7 @@ __global__ __launch_bounds__(kSpmvBlock) void collect_frontier_kernel(int n, con
         }
         __syncthreads();
     }
+    publish_counters(counters, ticket, host);
 }
 
 // One wavefront per (frontier vertex, chunk of kPushChunk out-edges); blockIdx.y is the chunk, so a hub's edges are
@@ -323,7 +347,8 @@ template <typename Push>
 __global__ __launch_bounds__(256) void push_round_kernel(int count, const int *__restrict__ frontier,
                                                          const int *__restrict__ index, const int *__restrict__ dst,
                                                          Push push, int *__restrict__ active, int mark,
-                                                         int *__restrict__ next, unsigned long long *__restrict__ counters)
+                                                         int *__restrict__ next, unsigned long long *counters,
+                                                         unsigned int *ticket, unsigned long long *host)
 {
     const int lane = threadIdx.x & (kWave - 1);
     const int waves = gridDim.x * (blockDim.x / kWave);
@@ -345,25 +370,29 @@ __global__ __launch_bounds__(256) void push_round_kernel(int count, const int *_
             frontier_append(take, t, take ? index[t + 1] - index[t] : 0, next, counters);
         }
     }
+    publish_counters(counters, ticket, host);
 }
 
 struct Frontier {
     unsigned long long count = 0, edges = 0, max_degree = 0;
 };
 
-Frontier read_counters(TraverseExt *t, hipStream_t s)
+Frontier read_counters(TraverseExt *t, hipStream_t s, bool published)
 {
-    DRONE_HIP_OR_DIE(hipMemcpyAsync(t->host, t->counters, sizeof(unsigned long long) * 2, hipMemcpyDeviceToHost, s));
-    DRONE_HIP_OR_DIE(hipStreamSynchronize(s));
+    if (!published) {
+        DRONE_HIP_OR_DIE(hipMemcpyAsync(t->host, t->counters, sizeof(unsigned long long) * 2, hipMemcpyDeviceToHost, s));
+        DRONE_HIP_OR_DIE(hipMemsetAsync(t->counters, 0, sizeof(unsigned long long) * 2, s));
+    }
+    DRONE_HIP_OR_DIE(hipStreamSynchronize(s));  // else publish_counters has written them
     return Frontier{t->host[0] >> 32, t->host[0] & 0xFFFFFFFFull, t->host[1]};
 }
 
 Frontier collect_frontier(Graph *g, TraverseExt *t, int value, int *list, hipStream_t s)
 {
     const int n = getLocalVertexSize(g);
-    clear_counters_kernel<<<1, 64, 0, s>>>(t->counters);
-    collect_frontier_kernel<<<t->blocks, kSpmvBlock, 0, s>>>(n, g->active, value, g->index, list, t->counters);
-    return read_counters(t, s);
+    collect_frontier_kernel<<<t->blocks, kSpmvBlock, 0, s>>>(n, g->active, value, g->index, list, t->counters, t->ticket,
+                                                            t->host);
+    return read_counters(t, s, true);
 }
 
 // Runs rounds until nothing changes.  `fr` describes the vertices that still have to propagate and sit in
@@ -384,7 +413,7 @@ int run_to_fixed_point(Graph *g, TraverseExt *t, Epi epi, Push push, Frontier fr
         ++mark;  // cc.cu:37 `active[v] = step + 1`: positive, and different in every round
         if (pull) {
             epi.mark = mark;
-            spmv_merge_launch<V, int, kIpt, Epi>(x->mt, x->ms, x->in_index, x->in_src, epi, t->stat, s);
+            spmv_merge_launch<V, int, kIpt, Epi>(x->mt, x->ms, x->in_index, x->in_src, epi, t->stat, s, stat_landing(t));
             DRONE_HIP_OR_DIE(hipGetLastError());
             const double changed = read_stat(t, s);
             if (changed == 0.0) return rounds;
@@ -394,14 +423,14 @@ int run_to_fixed_point(Graph *g, TraverseExt *t, Epi epi, Push push, Frontier fr
                 pull = fr.edges > push_limit;
             }
         } else {
-            clear_counters_kernel<<<1, 64, 0, s>>>(t->counters);
             const int waves_per_block = 256 / kWave;
             const int gx = (int)(ceil_div((int64_t)fr.count, waves_per_block) < 16384 ? ceil_div((int64_t)fr.count, waves_per_block) : 16384);
             const int gy = (int)ceil_div((int64_t)(fr.max_degree > 0 ? fr.max_degree : 1), kPushChunk);
+            const bool publish = (int64_t)gx * gy <= kPublishMaxBlocks;
             push_round_kernel<Push><<<dim3(gx, gy), 256, 0, s>>>((int)fr.count, t->frontier[cur], g->index, g->dst, push, g->active,
-                                                         mark, t->frontier[cur ^ 1], t->counters);
+                                                         mark, t->frontier[cur ^ 1], t->counters, publish ? t->ticket : nullptr, t->host);
             DRONE_HIP_OR_DIE(hipGetLastError());
-            fr = read_counters(t, s);
+            fr = read_counters(t, s, publish);
             cur ^= 1;
             if (fr.count == 0) return rounds;
             pull = fr.edges > push_limit;  // a sweep covers whatever the listed vertices still had to propagate
