@@ -183,9 +183,9 @@ void exchange_push(Graph *g, PRValues *values, int workerId, int workerNum, Comm
 }
 
 // Subgraphs with at least this many edges get source-sorted row blocks for the aggregation.  One superstep at
-// R-MAT scale 20 / 21 / 22 / 23 / 24 (16 ... 263 M edges) takes 0.087 / 0.125 / 0.20 / 0.36 / 0.68 ms with them and
-// 0.107 / 0.187 / 0.37 / 0.78 / 1.65 ms on the merge path; building them at the first PR_PEVal costs 8 / 12 / 18 ms
-// at scale 22 / 23 / 24 (and 15 ms more in a process that has not run these kernels yet), i.e. 46 / 29 / 19
+// R-MAT scale 20 / 21 / 22 / 23 / 24 (16 ... 263 M edges) takes 0.087 / 0.125 / 0.20 / 0.34 / 0.65 ms with them and
+// 0.107 / 0.187 / 0.37 / 0.77 / 1.64 ms on the merge path; building them at the first PR_PEVal costs 8 / 12 / 18 ms
+// at scale 22 / 23 / 24 (and 15 ms more in a process that has not run these kernels yet), i.e. 46 / 27 / 18
 // supersteps' worth of the saving, and about 90 at scale 21.  The default keeps the merge path (whose sums are also
 // added in a fixed order) until a PageRank run of about fifty supersteps gets the build back;
 // DRONE_PR_ROWBLOCK_MIN_EDGES in the environment moves the limit for jobs that run longer or shorter.

@@ -166,7 +166,7 @@ struct TraverseExt {
     int *frontier[2] = {nullptr, nullptr};  // device [n] each: vertex lists of the push rounds
     unsigned long long *counters = nullptr; // device [2]: {vertices << 32 | out-edges, largest out-degree} of the list being built; zero between launches
     unsigned int *ticket = nullptr;         // device [ticket_words(kPublishMaxBlocks)]: counters of last_block_done, zero between launches
-    unsigned long long *host = nullptr;     // pinned [2]: where the kernels' last work-groups leave the statistic / the counters
+    unsigned long long *host = nullptr;     // pinned [4]: where the kernels' last work-groups leave the statistic / the counters (+ rounds run)
 };
 
 double seconds_since(std::chrono::steady_clock::time_point t0)
@@ -194,7 +194,7 @@ TraverseExt *traverse_ext_create(int n)
     DRONE_HIP_OR_DIE(hipMalloc(&t->ticket, sizeof(unsigned int) * ticket_words(kPublishMaxBlocks)));
     DRONE_HIP_OR_DIE(hipMemset(t->ticket, 0, sizeof(unsigned int) * ticket_words(kPublishMaxBlocks)));
     DRONE_HIP_OR_DIE(hipStreamSynchronize(nullptr));  // the kernels that count may run on any stream
-    DRONE_HIP_OR_DIE(hipHostMalloc(&t->host, sizeof(unsigned long long) * 2));
+    DRONE_HIP_OR_DIE(hipHostMalloc(&t->host, sizeof(unsigned long long) * 4));
     return t;
 }
 
@@ -373,6 +373,64 @@ __global__ __launch_bounds__(256) void push_round_kernel(int count, const int *_
     publish_counters(counters, ticket, host);
 }
 
+// Push rounds of a short list inside ONE launch: a single work-group walks the list, builds the next one (counters in
+// LDS) and goes on with it for as long as it stays short - at most kSmallCount vertices with kSmallEdges out-edges -
+// and is not empty, up to max_rounds rounds.  Round k of the launch marks with mark + k.  A path of 20,000 vertices
+// then costs one launch and a barrier per hop instead of a launch and a host round trip per hop.  The lists alternate
+// between a and b; the host learns the rounds run and the last list's counters from pinned memory:
+// host[0] = count << 32 | out-edges, host[1] = largest out-degree, host[2] = rounds (the list is b after an odd number).
+constexpr int kSmallCount = 256;
+constexpr int kSmallEdges = 8192;
+
+template <typename Push>
+__global__ __launch_bounds__(256) void push_rounds_small_kernel(int count, int *a, int *b, const int *__restrict__ index,
+                                                                const int *__restrict__ dst, Push push, int *active,
+                                                                int mark, int max_rounds, unsigned long long *host)
+{
+    __shared__ unsigned long long s_counters[2];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int waves = blockDim.x / kWave;
+    int rounds = 0;
+    unsigned long long packed = 0, max_degree = 0;
+    for (;;) {
+        if (threadIdx.x < 2) s_counters[threadIdx.x] = 0ull;
+        __syncthreads();
+        for (int i = threadIdx.x / kWave; i < count; i += waves) {
+            const int v = a[i];
+            const int e0 = index[v], e1 = index[v + 1];
+            const auto val = push.load(v);
+            for (int eb = e0; eb < e1; eb += kWave) {
+                const int e = eb + lane;
+                bool take = false;
+                int t = 0;
+                if (e < e1) {
+                    t = dst[e];
+                    take = push.lower(t, push.relax(val, e)) && atomicExch(active + t, mark) != mark;
+                }
+                frontier_append(take, t, take ? index[t + 1] - index[t] : 0, b, s_counters);
+            }
+        }
+        __syncthreads();  // the next list and its counters are complete (the work-group's own writes are visible to it)
+        ++rounds;
+        packed = s_counters[0];
+        max_degree = s_counters[1];
+        count = (int)(packed >> 32);
+        int *const swap = a;
+        a = b;
+        b = swap;
+        if (count == 0 || count > kSmallCount || (packed & 0xFFFFFFFFull) > (unsigned long long)kSmallEdges ||
+            rounds == max_rounds)
+            break;
+        ++mark;
+        __syncthreads();  // everyone has read the counters before they are cleared
+    }
+    if (threadIdx.x == 0) {
+        host[0] = packed;
+        host[1] = max_degree;
+        host[2] = (unsigned long long)rounds;
+    }
+}
+
 struct Frontier {
     unsigned long long count = 0, edges = 0, max_degree = 0;
 };
@@ -422,6 +480,19 @@ int run_to_fixed_point(Graph *g, TraverseExt *t, Epi epi, Push push, Frontier fr
                 fr = collect_frontier(g, t, mark, t->frontier[0], s);
                 pull = fr.edges > push_limit;
             }
+        } else if (fr.count <= (unsigned long long)kSmallCount && fr.edges <= (unsigned long long)kSmallEdges) {
+            const int left = n + 3 - rounds;  // rounds this launch may run: the bound of n + 1 trips at the next check
+            push_rounds_small_kernel<Push><<<1, 256, 0, s>>>((int)fr.count, t->frontier[cur], t->frontier[cur ^ 1], g->index, g->dst,
+                                                           push, g->active, mark, left, t->host);
+            DRONE_HIP_OR_DIE(hipGetLastError());
+            DRONE_HIP_OR_DIE(hipStreamSynchronize(s));
+            const int ran = (int)t->host[2];
+            fr = Frontier{t->host[0] >> 32, t->host[0] & 0xFFFFFFFFull, t->host[1]};
+            rounds += ran - 1;
+            mark += ran - 1;
+            cur ^= ran & 1;
+            if (fr.count == 0) return rounds;
+            pull = fr.edges > push_limit;
         } else {
             const int waves_per_block = 256 / kWave;
             const int gx = (int)(ceil_div((int64_t)fr.count, waves_per_block) < 16384 ? ceil_div((int64_t)fr.count, waves_per_block) : 16384);

@@ -245,6 +245,48 @@ def test_long_chain_uses_sparse_rounds(oracle):
         w.close()
 
 
+def test_short_and_long_lists_alternate(oracle):
+    """A path, then a hub with 20,000 out-neighbours that each start a path of their own which all meet again in one
+    vertex, then another path: the list of lowered vertices is one vertex, then 20,000, then one again, so the rounds
+    that stay inside one launch (short lists) hand over to the wide push rounds and back, after an odd and an even
+    number of rounds.  Distances, labels and flags as the oracle's."""
+    from drone_amd.traverse import CCWorkerCUDA, SSSPWorkerCUDA
+    for lead in (37, 38):
+        fan, tail = 20000, 301
+        hub = lead
+        first = np.arange(lead, dtype=np.int64)
+        mid0 = hub + 1 + np.arange(fan, dtype=np.int64)              # out-neighbours of the hub
+        mid1 = mid0 + fan                                            # one more hop each
+        sink = hub + 1 + 2 * fan
+        last = sink + np.arange(tail, dtype=np.int64)
+        u = np.concatenate([first, np.full(fan, hub), mid0, mid1, last]).astype(np.int32)
+        v = np.concatenate([first + 1, mid0, mid1, np.full(fan, sink), last + 1]).astype(np.int32)
+        n = int(last[-1]) + 2
+        perm = np.random.default_rng(lead).permutation(n).astype(np.int32)
+        u, v = perm[u], perm[v]
+        nl, g2l, l2g, index, dst = oracle.build_graph(n, u, v)
+        st = oracle.SSSPState(index, dst)
+        st.peval(int(g2l[perm[0]]))
+        w = SSSPWorkerCUDA(n, u, v, startId=int(perm[0]))
+        try:
+            res = w.peval()
+            np.testing.assert_array_equal(w.read(), st.val)
+            np.testing.assert_array_equal(_sign(w.flags()["active"]), _sign(st.active))
+            assert res.VisitedSize == st.visited()
+            assert float(st.val.max()) == lead + 3 + tail
+        finally:
+            w.close()
+        sc = oracle.CCState(index, dst)
+        sc.peval()
+        w = CCWorkerCUDA(n, u, v)
+        try:
+            res = w.peval()
+            np.testing.assert_array_equal(w.read(), sc.val)
+            assert res.VisitedSize == sc.visited()
+        finally:
+            w.close()
+
+
 def test_graph_without_edges(oracle):
     from drone_amd.traverse import CCWorkerCUDA, SSSPWorkerCUDA
     e = np.zeros(0, np.int32)
