@@ -5,6 +5,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <vector>
 
 #include "../../include/drone_hip.h"
 
@@ -19,6 +20,46 @@ inline hipStream_t as_stream(drone_stream_t s) { return reinterpret_cast<hipStre
 constexpr int kWave = 64;
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// One device allocation handed out in 256-byte-aligned pieces.  Set-up code that needs a dozen arrays names them first
+// (want), pays for one hipMalloc (commit, which fills in the pointers) and later for one hipFree (release): a hipMalloc
+// or hipFree of a large buffer costs 0.1 ... 1.5 ms here, and a plan built from forty of them spent most of its time
+// there.  The pieces follow each other in the order they were asked for.
+struct DeviceArena {
+    char *base = nullptr;
+    size_t bytes = 0;
+
+    template <typename T> void want(T **p, size_t count)
+    {
+        wants_.push_back(Want{reinterpret_cast<void **>(p), bytes});
+        bytes += (count * sizeof(T) + 255) & ~(size_t)255;
+    }
+    hipError_t commit()
+    {
+        const hipError_t e = hipMalloc(reinterpret_cast<void **>(&base), bytes ? bytes : 256);
+        if (e != hipSuccess) {
+            base = nullptr;
+            return e;
+        }
+        for (const Want &w : wants_) *w.p = base + w.offset;
+        wants_.clear();
+        return hipSuccess;
+    }
+    void release()
+    {
+        if (base) (void)hipFree(base);
+        base = nullptr;
+        bytes = 0;
+        wants_.clear();
+    }
+
+private:
+    struct Want {
+        void **p;
+        size_t offset;
+    };
+    std::vector<Want> wants_;
+};
 
 }  // namespace drone
 

@@ -175,10 +175,7 @@ extern "C" int drone_pr_plan_create_ex(drone_pr_plan **out, int64_t n, int64_t n
             if (rc != DRONE_OK) return rc;
             p->units = p->rb.num_blocks;
             // the row-ordered copy is only needed to build the blocks
-            (void)hipFree(p->rl.row_ptr);
-            (void)hipFree(p->rl.col);
-            p->rl.row_ptr = nullptr;
-            p->rl.col = nullptr;
+            relabel_release_csr(&p->rl);
             DRONE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&pr_rowblock_kernel<PrF64Epi>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, kRbLdsBytes));
         }

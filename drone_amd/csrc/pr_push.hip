@@ -184,12 +184,12 @@ void exchange_push(Graph *g, PRValues *values, int workerId, int workerNum, Comm
 
 // Subgraphs with at least this many edges get source-sorted row blocks for the aggregation.  One superstep at
 // R-MAT scale 20 / 21 / 22 / 23 / 24 (16 ... 263 M edges) takes 0.087 / 0.125 / 0.20 / 0.34 / 0.65 ms with them and
-// 0.107 / 0.187 / 0.37 / 0.77 / 1.64 ms on the merge path; building them at the first PR_PEVal costs 8 / 12 / 18 ms
-// at scale 22 / 23 / 24 (and 15 ms more in a process that has not run these kernels yet), i.e. 46 / 27 / 18
-// supersteps' worth of the saving, and about 90 at scale 21.  The default keeps the merge path (whose sums are also
-// added in a fixed order) until a PageRank run of about fifty supersteps gets the build back;
+// 0.107 / 0.187 / 0.37 / 0.77 / 1.64 ms on the merge path; building them at the first PR_PEVal costs 2.9 / 3.8 /
+// 5.3 / 9.3 / 15.6 ms at scale 20 ... 24 (and 15 ms more in a process that has not run these kernels yet), i.e. 145 /
+// 61 / 31 / 21 / 16 supersteps' worth of the saving.  A run to the reference's eps of 1e-6 takes some 85 supersteps (0.85^85 = 1e-6),
+// so the default keeps the merge path (whose sums are also added in a fixed order) below 24 Mi edges;
 // DRONE_PR_ROWBLOCK_MIN_EDGES in the environment moves the limit for jobs that run longer or shorter.
-constexpr int64_t kRowBlockMinEdges = 48ll << 20;
+constexpr int64_t kRowBlockMinEdges = 24ll << 20;
 
 int64_t row_block_min_edges()
 {

@@ -71,6 +71,7 @@ struct RowBlocks {
     int num_split = 0;
     int32_t *split_block = nullptr;  // device [num_split]: the blocks with more than one unit
     double *partial = nullptr;       // device: per split block, block_units x (rows + 1) row sums (8-byte values)
+    DeviceArena arena;               // every array above except `stream` is a piece of this one allocation
 };
 
 // Builds the blocks for a CSR with device row_ptr / col (already in the plan's internal id space).

@@ -177,81 +177,87 @@ __global__ __launch_bounds__(1024) void rb_pack_kernel(int num_blocks, int total
     }
 }
 
+// Temporaries of the sort and of the packing, pieces of one allocation.
+template <typename Key> struct RbTemps {
+    Key *keys = nullptr, *keys_sorted = nullptr;
+    uint16_t *lrow_in = nullptr;
+    void *sort_temp = nullptr, *scan_temp = nullptr;
+    size_t sort_bytes = 0, scan_bytes = 0;
+    uint32_t *batch_size = nullptr, *batch_pos = nullptr;
+};
+
 // Sorts the entries by (block, source) and derives the compact entry format.  The entries arrive grouped by block
 // already, so consecutive blocks can be sorted as separate ranges: with `group` (a power of two) blocks per range the
 // key needs col_bits + log2(group) bits, which keeps large matrices on 32-bit keys (R-MAT scale 24, 263 M entries:
 // three ranges of 256 blocks and four 8-bit passes over 6-byte pairs instead of five over 10-byte pairs).
+// `landing`: a pinned word for the size of the entry stream.  Everything the sort needs comes from one allocation
+// that is released before returning; the entry stream is the one array whose size is only known half-way.
 template <typename Key>
 int rb_sort_and_pack(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_ptr, const int32_t *col, int nb,
-                     int col_bits, int group, const std::vector<int64_t> &h_nnz, int total_batches, void **scratch,
-                     hipStream_t stream)
+                     int col_bits, int group, const std::vector<int64_t> &h_nnz, int total_batches,
+                     uint32_t *landing, hipStream_t stream)
 {
-    // scratch[0..3]: keys, sorted keys, unsorted local rows, the sort's workspace (freed by the caller)
-    Key *keys = nullptr, *keys_sorted = nullptr;
-    uint16_t *lrow_in = nullptr;
-    void *temp = nullptr;
-    const size_t e = (size_t)nnz;
-    DRONE_HIP_TRY(hipMalloc(&keys, sizeof(Key) * e));
-    scratch[0] = keys;
-    DRONE_HIP_TRY(hipMalloc(&keys_sorted, sizeof(Key) * e));
-    scratch[1] = keys_sorted;
-    DRONE_HIP_TRY(hipMalloc(&lrow_in, sizeof(uint16_t) * e));
-    scratch[2] = lrow_in;
-    rb_keys_kernel<Key><<<(unsigned)ceil_div(nnz, (int64_t)kKeysChunk), 256, 0, stream>>>(
-        row_ptr, col, n, nnz, nb, rb->block_row, rb->block_nnz, col_bits, group - 1, keys, lrow_in);
-    int group_bits = 0;
-    while ((1 << group_bits) < group) ++group_bits;
-    size_t temp_bytes = 0;
-    for (int b0 = 0; b0 < nb; b0 += group) {  // the workspace of the largest range serves all
-        const int b1 = b0 + group < nb ? b0 + group : nb;
-        const size_t count = (size_t)(h_nnz[(size_t)b1] - h_nnz[(size_t)b0]);
-        size_t need = 0;
-        DRONE_HIP_TRY(rocprim::radix_sort_pairs(nullptr, need, keys, keys_sorted, lrow_in, rb->lrow, count, 0,
-                                                col_bits + group_bits, stream));
-        if (need > temp_bytes) temp_bytes = need;
-    }
-    DRONE_HIP_TRY(hipMalloc(&temp, temp_bytes ? temp_bytes : 1));
-    scratch[3] = temp;
-    for (int b0 = 0; b0 < nb; b0 += group) {
-        const int b1 = b0 + group < nb ? b0 + group : nb;
-        const size_t first = (size_t)h_nnz[(size_t)b0], count = (size_t)(h_nnz[(size_t)b1] - h_nnz[(size_t)b0]);
-        if (count == 0) continue;
-        size_t bytes = temp_bytes;
-        DRONE_HIP_TRY(rocprim::radix_sort_pairs(temp, bytes, keys + first, keys_sorted + first, lrow_in + first,
-                                                rb->lrow + first, count, 0, col_bits + group_bits, stream));
-    }
-    // entry widths per batch, their positions (exclusive scan, in 64-byte units), then the entries themselves
-    uint32_t *batch_size = nullptr, *batch_pos = nullptr;
-    void *scan_temp = nullptr;
-    const auto pack = [&]() -> int {
+    RbTemps<Key> t;
+    DeviceArena temps;
+    const auto body = [&]() -> int {
+        const size_t e = (size_t)nnz, tb = (size_t)total_batches;
+        int group_bits = 0;
+        while ((1 << group_bits) < group) ++group_bits;
+        for (int b0 = 0; b0 < nb; b0 += group) {  // the workspace of the largest range serves all
+            const int b1 = b0 + group < nb ? b0 + group : nb;
+            const size_t count = (size_t)(h_nnz[(size_t)b1] - h_nnz[(size_t)b0]);
+            size_t need = 0;
+            // stand-in addresses (never read): the arrays do not exist yet, and the sort sizes its workspace
+            // differently when input and output are the same array
+            DRONE_HIP_TRY(rocprim::radix_sort_pairs(nullptr, need, reinterpret_cast<Key *>(0x1000),
+                                                    reinterpret_cast<Key *>(0x2000), reinterpret_cast<uint16_t *>(0x3000),
+                                                    rb->lrow, count, 0, col_bits + group_bits, stream));
+            if (need > t.sort_bytes) t.sort_bytes = need;
+        }
+        DRONE_HIP_TRY(rocprim::exclusive_scan(nullptr, t.scan_bytes, reinterpret_cast<uint32_t *>(0x1000),
+                                              reinterpret_cast<uint32_t *>(0x2000), 0u, tb + 1,
+                                              rocprim::plus<uint32_t>(), stream));
+        temps.want(&t.keys, e);
+        temps.want(&t.keys_sorted, e);
+        temps.want(&t.lrow_in, e);
+        temps.want(reinterpret_cast<char **>(&t.sort_temp), t.sort_bytes);
+        temps.want(reinterpret_cast<char **>(&t.scan_temp), t.scan_bytes);
+        temps.want(&t.batch_size, tb + 1);
+        temps.want(&t.batch_pos, tb + 1);
+        DRONE_HIP_TRY(temps.commit());
+        rb_keys_kernel<Key><<<(unsigned)ceil_div(nnz, (int64_t)kKeysChunk), 256, 0, stream>>>(
+            row_ptr, col, n, nnz, nb, rb->block_row, rb->block_nnz, col_bits, group - 1, t.keys, t.lrow_in);
+        for (int b0 = 0; b0 < nb; b0 += group) {
+            const int b1 = b0 + group < nb ? b0 + group : nb;
+            const size_t first = (size_t)h_nnz[(size_t)b0], count = (size_t)(h_nnz[(size_t)b1] - h_nnz[(size_t)b0]);
+            if (count == 0) continue;
+            size_t bytes = t.sort_bytes;
+            DRONE_HIP_TRY(rocprim::radix_sort_pairs(t.sort_temp, bytes, t.keys + first, t.keys_sorted + first,
+                                                    t.lrow_in + first, rb->lrow + first, count, 0, col_bits + group_bits,
+                                                    stream));
+        }
+        // entry widths per batch, their positions (exclusive scan, in 64-byte units), then the entries themselves
         const unsigned grid = (unsigned)ceil_div(ceil_div((int64_t)total_batches, (int64_t)kPackBatches) * kWave, (int64_t)1024);
-        const size_t tb = (size_t)total_batches;
-        DRONE_HIP_TRY(hipMalloc(&batch_size, sizeof(uint32_t) * (tb + 1)));
-        DRONE_HIP_TRY(hipMalloc(&batch_pos, sizeof(uint32_t) * (tb + 1)));
-        DRONE_HIP_TRY(hipMemsetAsync(batch_size + tb, 0, sizeof(uint32_t), stream));
+        DRONE_HIP_TRY(hipMemsetAsync(t.batch_size + tb, 0, sizeof(uint32_t), stream));
         rb_pack_kernel<Key, false><<<grid, 1024, 0, stream>>>(nb, total_batches, rb->block_nnz, rb->block_batch, col_bits,
-                                                             keys_sorted, rb->lrow, rb->col, rb->batch_info, batch_size,
+                                                             t.keys_sorted, rb->lrow, rb->col, rb->batch_info, t.batch_size,
                                                              nullptr, nullptr, rb->block_wide);
-        size_t scan_bytes = 0;
-        DRONE_HIP_TRY(rocprim::exclusive_scan(nullptr, scan_bytes, batch_size, batch_pos, 0u, tb + 1, rocprim::plus<uint32_t>(), stream));
-        DRONE_HIP_TRY(hipMalloc(&scan_temp, scan_bytes ? scan_bytes : 1));
-        DRONE_HIP_TRY(rocprim::exclusive_scan(scan_temp, scan_bytes, batch_size, batch_pos, 0u, tb + 1, rocprim::plus<uint32_t>(), stream));
-        uint32_t total64 = 0;
-        DRONE_HIP_TRY(hipMemcpyAsync(&total64, batch_pos + tb, sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+        size_t scan_bytes = t.scan_bytes;
+        DRONE_HIP_TRY(rocprim::exclusive_scan(t.scan_temp, scan_bytes, t.batch_size, t.batch_pos, 0u, tb + 1,
+                                              rocprim::plus<uint32_t>(), stream));
+        DRONE_HIP_TRY(hipMemcpyAsync(landing, t.batch_pos + tb, sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
         DRONE_HIP_TRY(hipStreamSynchronize(stream));
-        rb->stream_bytes = (int64_t)total64 * 64;
+        rb->stream_bytes = (int64_t)*landing * 64;
         DRONE_HIP_TRY(hipMalloc(&rb->stream, (size_t)rb->stream_bytes + 64));  // the last entry's 4-byte load may run past it
         rb_pack_kernel<Key, true><<<grid, 1024, 0, stream>>>(nb, total_batches, rb->block_nnz, rb->block_batch, col_bits,
-                                                            keys_sorted, rb->lrow, rb->col, rb->batch_info, batch_size,
-                                                            batch_pos, rb->stream, rb->block_wide);
+                                                            t.keys_sorted, rb->lrow, rb->col, rb->batch_info, t.batch_size,
+                                                            t.batch_pos, rb->stream, rb->block_wide);
         DRONE_HIP_TRY(hipGetLastError());
-        DRONE_HIP_TRY(hipStreamSynchronize(stream));
+        DRONE_HIP_TRY(hipStreamSynchronize(stream));  // the temporaries go next
         return DRONE_OK;
     };
-    const int rc = pack();
-    (void)hipFree(batch_size);
-    (void)hipFree(batch_pos);
-    (void)hipFree(scan_temp);
+    const int rc = body();
+    temps.release();
     return rc;
 }
 
@@ -286,79 +292,57 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
     rb->items = items * split;             // entries one block holds at most
     const int weight = items / kRbRows;
     const int64_t total = (int64_t)weight * n + nnz;
-    int nb = (int)ceil_div(total, items);  // blocks of the weighted split; fewer once neighbours are merged
-    rb->num_blocks = nb;
-    void *scratch[4] = {nullptr, nullptr, nullptr, nullptr};  // temporaries of the sort
-    auto body = [&]() -> int {
-        const size_t e = (size_t)(nnz ? nnz : 1);
-        DRONE_HIP_TRY(hipMalloc(&rb->block_row, sizeof(int32_t) * ((size_t)nb + 1)));
-        DRONE_HIP_TRY(hipMalloc(&rb->block_nnz, sizeof(int64_t) * ((size_t)nb + 1)));
-        DRONE_HIP_TRY(hipMalloc(&rb->walk_len, sizeof(int32_t) * (size_t)nb));
-        DRONE_HIP_TRY(hipMalloc(&rb->col, sizeof(int32_t) * e));
-        DRONE_HIP_TRY(hipMalloc(&rb->lrow, sizeof(uint16_t) * e));
-        rb_search_kernel<<<(int)ceil_div(nb + 1, 256), 256, 0, stream>>>(row_ptr, n, nnz, nb, items, weight, rb->block_row, rb->block_nnz);
+    const int nb0 = (int)ceil_div(total, items);  // blocks of the weighted split; fewer once neighbours are merged
+    // The build makes two round trips to the host: the block boundaries come back once (the host merges neighbours,
+    // numbers the 64-entry batches and lays out the work units, and sends all the per-block tables back in one copy),
+    // and the size of the entry stream once.  Device memory: the boundaries of the first split, one allocation for
+    // everything the plan keeps except the entry stream, one for the sort's temporaries, the stream.
+    int64_t *bounds = nullptr;          // device [nb0 + 1] entries, then [nb0 + 1] rows (as int32)
+    unsigned char *pinned = nullptr;    // host staging of the same and of the per-block tables
+    const auto body = [&]() -> int {
+        const size_t nb0p = (size_t)nb0 + 1;
+        DRONE_HIP_TRY(hipMalloc(&bounds, sizeof(int64_t) * nb0p + sizeof(int32_t) * nb0p));
+        int32_t *bounds_row = reinterpret_cast<int32_t *>(bounds + nb0p);
+        rb_search_kernel<<<(int)ceil_div(nb0 + 1, 256), 256, 0, stream>>>(row_ptr, n, nnz, nb0, items, weight, bounds_row, bounds);
+        // staging: the boundaries on the way back, the tables on the way out (sized below, never more than this)
+        const size_t units_max = (size_t)ceil_div(nnz, unit_items) + nb0p;
+        const size_t stage_bytes = 256 * 11 + nb0p * (8 + 4 + 4 + 4 + 4 + 8 + 4) + units_max * 4;  // the last 256 bytes: a landing word
+        DRONE_HIP_TRY(hipHostMalloc(&pinned, stage_bytes));
+        DRONE_HIP_TRY(hipMemcpyAsync(pinned, bounds, sizeof(int64_t) * nb0p + sizeof(int32_t) * nb0p, hipMemcpyDeviceToHost, stream));
+        DRONE_HIP_TRY(hipStreamSynchronize(stream));
+        std::vector<int64_t> h_nnz(nb0p);
+        std::vector<int32_t> h_row(nb0p);
+        memcpy(h_nnz.data(), pinned, sizeof(int64_t) * nb0p);
+        memcpy(h_row.data(), pinned + sizeof(int64_t) * nb0p, sizeof(int32_t) * nb0p);
+        int nb = nb0;
         if (split > 1) {
             // Shared blocks: the weighted split trades rows against entries, so its blocks reach neither limit.
             // Neighbours are merged while the result stays within 16,384 rows and split x items entries.
-            std::vector<int32_t> br((size_t)nb + 1);
-            std::vector<int64_t> bn((size_t)nb + 1);
-            DRONE_HIP_TRY(hipMemcpyAsync(br.data(), rb->block_row, sizeof(int32_t) * br.size(), hipMemcpyDeviceToHost, stream));
-            DRONE_HIP_TRY(hipMemcpyAsync(bn.data(), rb->block_nnz, sizeof(int64_t) * bn.size(), hipMemcpyDeviceToHost, stream));
-            DRONE_HIP_TRY(hipStreamSynchronize(stream));
             int out = 0, first = 0;
-            for (int b = 1; b <= nb; ++b) {
+            for (int b = 1; b <= nb0; ++b) {
                 // close the block [first, b) when taking block b as well would break a limit
-                const bool last_one = b == nb;
-                if (last_one || br[(size_t)b + 1] - br[(size_t)first] > kRbRows ||
-                    bn[(size_t)b + 1] - bn[(size_t)first] > (int64_t)items * split) {
-                    br[(size_t)out] = br[(size_t)first];
-                    bn[(size_t)out] = bn[(size_t)first];
+                const bool last_one = b == nb0;
+                if (last_one || h_row[(size_t)b + 1] - h_row[(size_t)first] > kRbRows ||
+                    h_nnz[(size_t)b + 1] - h_nnz[(size_t)first] > (int64_t)items * split) {
+                    h_row[(size_t)out] = h_row[(size_t)first];
+                    h_nnz[(size_t)out] = h_nnz[(size_t)first];
                     ++out;
                     first = b;
                 }
             }
-            br[(size_t)out] = br[(size_t)nb];
-            bn[(size_t)out] = bn[(size_t)nb];
+            h_row[(size_t)out] = h_row[(size_t)nb0];
+            h_nnz[(size_t)out] = h_nnz[(size_t)nb0];
             nb = out;
-            rb->num_blocks = nb;
-            DRONE_HIP_TRY(hipMemcpyAsync(rb->block_row, br.data(), sizeof(int32_t) * ((size_t)nb + 1), hipMemcpyHostToDevice, stream));
-            DRONE_HIP_TRY(hipMemcpyAsync(rb->block_nnz, bn.data(), sizeof(int64_t) * ((size_t)nb + 1), hipMemcpyHostToDevice, stream));
-            DRONE_HIP_TRY(hipStreamSynchronize(stream));  // br / bn go out of scope
         }
-        rb_walk_len_kernel<<<(int)ceil_div(nb, 256), 256, 0, stream>>>(row_ptr, nb, rb->block_row, rb->block_nnz, rb->walk_len);
+        rb->num_blocks = nb;
         // compact entries: the blocks' 64-entry batches are numbered through
-        DRONE_HIP_TRY(hipMalloc(&rb->block_batch, sizeof(int32_t) * ((size_t)nb + 1)));
-        DRONE_HIP_TRY(hipMalloc(&rb->block_wide, sizeof(int32_t) * (size_t)nb));
-        DRONE_HIP_TRY(hipMemsetAsync(rb->block_wide, 0, sizeof(int32_t) * (size_t)nb, stream));
-        std::vector<int64_t> h_nnz((size_t)nb + 1);
-        DRONE_HIP_TRY(hipMemcpyAsync(h_nnz.data(), rb->block_nnz, sizeof(int64_t) * h_nnz.size(), hipMemcpyDeviceToHost, stream));
-        DRONE_HIP_TRY(hipStreamSynchronize(stream));
         std::vector<int32_t> h_batch((size_t)nb + 1, 0);
         for (int b = 0; b < nb; ++b) h_batch[b + 1] = h_batch[b] + (int32_t)ceil_div(h_nnz[b + 1] - h_nnz[b], 64);
-        DRONE_HIP_TRY(hipMalloc(&rb->batch_info, sizeof(int2) * (size_t)(h_batch[nb] ? h_batch[nb] : 1)));
-        DRONE_HIP_TRY(hipMemcpyAsync(rb->block_batch, h_batch.data(), sizeof(int32_t) * h_batch.size(), hipMemcpyHostToDevice, stream));
-        if (nnz > 0) {
-            // key = (block within its range << col_bits) | source: 32-bit keys while at most 64 ranges do it
-            int col_bits = 1, block_bits = 1;
-            while (col_bits < 32 && (1ll << col_bits) < n) ++col_bits;
-            while (block_bits < 31 && (1ll << block_bits) < nb) ++block_bits;
-            int group_bits = block_bits < 32 - col_bits ? block_bits : 32 - col_bits;
-            if (group_bits < 0) group_bits = 0;
-            const bool narrow = col_bits + group_bits <= 32 && ceil_div(nb, 1 << group_bits) <= 64;
-            const int rc = narrow ? rb_sort_and_pack<uint32_t>(rb, n, nnz, row_ptr, col, nb, col_bits, 1 << group_bits,
-                                                               h_nnz, h_batch[nb], scratch, stream)
-                                  : rb_sort_and_pack<uint64_t>(rb, n, nnz, row_ptr, col, nb, col_bits, 1 << block_bits,
-                                                               h_nnz, h_batch[nb], scratch, stream);
-            if (rc != DRONE_OK) return rc;
-        }
         // work units: a block is shared by as many work-groups as it holds unit_items entries (at most `split`).
         // The units are numbered block by block, so the work-groups of one block spread over the XCDs (work-groups go
         // to the XCDs round-robin); numbering eight blocks share-major, which puts a block's work-groups on one XCD
         // where they could find each other's source lines in L2, measured 0.590 against 0.572 ms per iteration.
-        std::vector<int32_t> h_row((size_t)nb + 1);
-        DRONE_HIP_TRY(hipMemcpyAsync(h_row.data(), rb->block_row, sizeof(int32_t) * h_row.size(), hipMemcpyDeviceToHost, stream));
-        DRONE_HIP_TRY(hipStreamSynchronize(stream));
-        std::vector<int32_t> h_unit_block, h_units((size_t)nb), h_unit0((size_t)nb);
+        std::vector<int32_t> h_unit_block, h_units((size_t)nb), h_unit0((size_t)nb), h_split;
         std::vector<int64_t> h_partial((size_t)nb, 0);
         int64_t partial_doubles = 0;
         for (int b = 0; b < nb; ++b) {
@@ -374,52 +358,78 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
             if (shares > 1) {
                 h_partial[b] = partial_doubles;
                 partial_doubles += (int64_t)shares * (h_row[b + 1] - h_row[b] + 1);
+                h_split.push_back(b);
             }
         }
         rb->num_units = (int)h_unit_block.size();
-        DRONE_HIP_TRY(hipMalloc(&rb->unit_block, sizeof(int32_t) * h_unit_block.size()));
-        DRONE_HIP_TRY(hipMalloc(&rb->block_units, sizeof(int32_t) * (size_t)nb));
-        DRONE_HIP_TRY(hipMalloc(&rb->block_unit0, sizeof(int32_t) * (size_t)nb));
-        DRONE_HIP_TRY(hipMalloc(&rb->block_partial, sizeof(int64_t) * (size_t)nb));
-        DRONE_HIP_TRY(hipMalloc(&rb->partial, sizeof(double) * (size_t)(partial_doubles ? partial_doubles : 1)));
-        DRONE_HIP_TRY(hipMemcpyAsync(rb->unit_block, h_unit_block.data(), sizeof(int32_t) * h_unit_block.size(), hipMemcpyHostToDevice, stream));
-        DRONE_HIP_TRY(hipMemcpyAsync(rb->block_units, h_units.data(), sizeof(int32_t) * (size_t)nb, hipMemcpyHostToDevice, stream));
-        DRONE_HIP_TRY(hipMemcpyAsync(rb->block_unit0, h_unit0.data(), sizeof(int32_t) * (size_t)nb, hipMemcpyHostToDevice, stream));
-        DRONE_HIP_TRY(hipMemcpyAsync(rb->block_partial, h_partial.data(), sizeof(int64_t) * (size_t)nb, hipMemcpyHostToDevice, stream));
-        std::vector<int32_t> h_split;
-        for (int b = 0; b < nb; ++b)
-            if (h_units[b] > 1) h_split.push_back(b);
         rb->num_split = (int)h_split.size();
-        DRONE_HIP_TRY(hipMalloc(&rb->split_block, sizeof(int32_t) * (h_split.size() ? h_split.size() : 1)));
-        if (!h_split.empty())
-            DRONE_HIP_TRY(hipMemcpyAsync(rb->split_block, h_split.data(), sizeof(int32_t) * h_split.size(), hipMemcpyHostToDevice, stream));
+        // what the plan keeps: the tables the host just made first, in the order they are staged
+        const size_t e = (size_t)(nnz ? nnz : 1), nbp = (size_t)nb + 1, nbs = (size_t)(nb ? nb : 1);
+        DeviceArena &ar = rb->arena;
+        ar.want(&rb->block_nnz, nbp);
+        ar.want(&rb->block_partial, nbs);
+        ar.want(&rb->block_row, nbp);
+        ar.want(&rb->block_batch, nbp);
+        ar.want(&rb->block_units, nbs);
+        ar.want(&rb->block_unit0, nbs);
+        ar.want(&rb->unit_block, h_unit_block.size() ? h_unit_block.size() : 1);
+        ar.want(&rb->split_block, h_split.size() ? h_split.size() : 1);
+        const size_t tables_bytes = ar.bytes;
+        ar.want(&rb->walk_len, nbs);
+        ar.want(&rb->block_wide, nbs);
+        ar.want(&rb->batch_info, (size_t)(h_batch[nb] ? h_batch[nb] : 1));
+        ar.want(&rb->col, e);
+        ar.want(&rb->lrow, e);
+        ar.want(&rb->partial, (size_t)(partial_doubles ? partial_doubles : 1));
+        DRONE_HIP_TRY(ar.commit());
+        if (tables_bytes > stage_bytes - 256) {
+            set_error(DRONE_ERR_INVALID, "row blocks: staging buffer too small (%zu > %zu)", tables_bytes, stage_bytes);
+            return DRONE_ERR_INVALID;
+        }
+        const auto stage = [&](const void *device_piece, const void *src, size_t bytes) {
+            memcpy(pinned + (reinterpret_cast<const char *>(device_piece) - ar.base), src, bytes);
+        };
+        stage(rb->block_nnz, h_nnz.data(), sizeof(int64_t) * nbp);
+        stage(rb->block_partial, h_partial.data(), sizeof(int64_t) * (size_t)nb);
+        stage(rb->block_row, h_row.data(), sizeof(int32_t) * nbp);
+        stage(rb->block_batch, h_batch.data(), sizeof(int32_t) * nbp);
+        stage(rb->block_units, h_units.data(), sizeof(int32_t) * (size_t)nb);
+        stage(rb->block_unit0, h_unit0.data(), sizeof(int32_t) * (size_t)nb);
+        stage(rb->unit_block, h_unit_block.data(), sizeof(int32_t) * h_unit_block.size());
+        stage(rb->split_block, h_split.data(), sizeof(int32_t) * h_split.size());
+        DRONE_HIP_TRY(hipMemcpyAsync(ar.base, pinned, tables_bytes, hipMemcpyHostToDevice, stream));
+        DRONE_HIP_TRY(hipMemsetAsync(rb->block_wide, 0, sizeof(int32_t) * nbs, stream));
+        rb_walk_len_kernel<<<(int)ceil_div(nb, 256), 256, 0, stream>>>(row_ptr, nb, rb->block_row, rb->block_nnz, rb->walk_len);
+        if (nnz > 0) {
+            // key = (block within its range << col_bits) | source: 32-bit keys while at most 64 ranges do it
+            int col_bits = 1, block_bits = 1;
+            while (col_bits < 32 && (1ll << col_bits) < n) ++col_bits;
+            while (block_bits < 31 && (1ll << block_bits) < nb) ++block_bits;
+            int group_bits = block_bits < 32 - col_bits ? block_bits : 32 - col_bits;
+            if (group_bits < 0) group_bits = 0;
+            const bool narrow = col_bits + group_bits <= 32 && ceil_div(nb, 1 << group_bits) <= 64;
+            uint32_t *landing = reinterpret_cast<uint32_t *>(pinned + stage_bytes - 256);
+            const int rc = narrow ? rb_sort_and_pack<uint32_t>(rb, n, nnz, row_ptr, col, nb, col_bits, 1 << group_bits,
+                                                               h_nnz, h_batch[nb], landing, stream)
+                                  : rb_sort_and_pack<uint64_t>(rb, n, nnz, row_ptr, col, nb, col_bits, 1 << block_bits,
+                                                               h_nnz, h_batch[nb], landing, stream);
+            if (rc != DRONE_OK) return rc;
+        }
         DRONE_HIP_TRY(hipGetLastError());
         DRONE_HIP_TRY(hipStreamSynchronize(stream));
         return DRONE_OK;
     };
     const int rc = body();
-    for (void *p : scratch) (void)hipFree(p);
+    (void)hipFree(bounds);
+    if (pinned) (void)hipHostFree(pinned);
     if (rc != DRONE_OK) row_blocks_destroy(rb);
     return rc;
 }
 
 void row_blocks_destroy(RowBlocks *rb)
 {
-    (void)hipFree(rb->block_row);
-    (void)hipFree(rb->block_nnz);
-    (void)hipFree(rb->walk_len);
-    (void)hipFree(rb->col);
-    (void)hipFree(rb->lrow);
+    rb->arena.release();
     (void)hipFree(rb->stream);
-    (void)hipFree(rb->batch_info);
-    (void)hipFree(rb->block_batch);
-    (void)hipFree(rb->block_wide);
-    (void)hipFree(rb->unit_block);
-    (void)hipFree(rb->block_units);
-    (void)hipFree(rb->block_unit0);
-    (void)hipFree(rb->block_partial);
-    (void)hipFree(rb->split_block);
-    (void)hipFree(rb->partial);
     *rb = RowBlocks{};
 }
 

@@ -19,6 +19,7 @@ struct Relabel {
     int32_t *order = nullptr;    // device [n]: new id -> old id
     int64_t *row_ptr = nullptr;  // device [n+1]: relabelled CSR offsets
     int32_t *col = nullptr;      // device [nnz]: relabelled sources, row order kept
+    DeviceArena arena;           // row_ptr and col are pieces of this one allocation; order is on its own
 };
 
 // Builds the relabelled CSR from (row_ptr, col) on `stream`.  inv_outdeg (device [n], may be null): the vertices'
@@ -31,6 +32,8 @@ int relabel_create(Relabel *rl, int64_t n, int64_t nnz, const int64_t *row_ptr, 
                    const double *inv_outdeg, hipStream_t stream, bool keep_rows = false,
                    const int *transposed_offsets = nullptr);
 void relabel_destroy(Relabel *rl);
+// Releases row_ptr and col (for callers that only needed them to build something else) and keeps order.
+void relabel_release_csr(Relabel *rl);
 
 // out[i] = in[order[i]]
 int relabel_gather_f64(const Relabel &rl, const double *in, double *out, hipStream_t stream);

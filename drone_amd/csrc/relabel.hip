@@ -168,23 +168,37 @@ int relabel_create(Relabel *rl, int64_t n, int64_t nnz, const int64_t *row_ptr, 
     unsigned *count = nullptr, *count_sorted = nullptr;
     int32_t *ids = nullptr, *new_id = nullptr;
     int64_t *len = nullptr;
-    void *temp = nullptr;
+    char *temp = nullptr;
     unsigned long long *live = nullptr;  // device: [0] vertices that are not isolated, [1] (as int) largest gathered new id
-    unsigned long long h_live[2] = {0, 0};
+    unsigned long long *h_live = nullptr;  // pinned landing place of the two
     size_t temp_bytes = 0, need = 0;
     const int blocks = 2048, threads = 256;
+    DeviceArena temps;  // one allocation for what the plan keeps (rl->arena), one for the temporaries
     rl->n = n;
     rl->nnz = nnz;
     rl->live = n;
+    rl->arena.want(&rl->row_ptr, (size_t)n + 1);
+    rl->arena.want(&rl->col, (size_t)(nnz ? nnz : 1));
+    RL_TRY(rl->arena.commit());
     RL_TRY(hipMalloc(&rl->order, sizeof(int32_t) * (size_t)n));
-    RL_TRY(hipMalloc(&rl->row_ptr, sizeof(int64_t) * ((size_t)n + 1)));
-    RL_TRY(hipMalloc(&rl->col, sizeof(int32_t) * (size_t)(nnz ? nnz : 1)));
-    RL_TRY(hipMalloc(&count, sizeof(unsigned) * (size_t)n));
-    RL_TRY(hipMalloc(&count_sorted, sizeof(unsigned) * (size_t)n));
-    RL_TRY(hipMalloc(&ids, sizeof(int32_t) * (size_t)n));
-    RL_TRY(hipMalloc(&new_id, sizeof(int32_t) * (size_t)n));
-    RL_TRY(hipMalloc(&len, sizeof(int64_t) * ((size_t)n + 1)));
-    RL_TRY(hipMalloc(&live, sizeof(unsigned long long) * 2));
+    // stable descending sort by gather count: order[new] = old.  The size queries come before the arrays exist; they
+    // get distinct stand-in addresses (never read), because the sort sizes its workspace differently when input and
+    // output are the same array.
+    RL_TRY(rocprim::radix_sort_pairs_desc(nullptr, temp_bytes, reinterpret_cast<unsigned *>(0x1000),
+                                          reinterpret_cast<unsigned *>(0x2000), reinterpret_cast<int32_t *>(0x3000),
+                                          rl->order, (size_t)n, 0, 32, stream));
+    RL_TRY(rocprim::exclusive_scan(nullptr, need, reinterpret_cast<int64_t *>(0x1000), rl->row_ptr, (int64_t)0,
+                                   (size_t)n + 1, rocprim::plus<int64_t>(), stream));
+    if (need > temp_bytes) temp_bytes = need;
+    temps.want(&len, (size_t)n + 1);
+    temps.want(&live, 2);
+    temps.want(&count, (size_t)n);
+    temps.want(&count_sorted, (size_t)n);
+    temps.want(&ids, (size_t)n);
+    temps.want(&new_id, (size_t)n);
+    temps.want(&temp, temp_bytes);
+    RL_TRY(temps.commit());
+    RL_TRY(hipHostMalloc(&h_live, sizeof(unsigned long long) * 2));
     RL_TRY(hipMemsetAsync(live, 0, sizeof(unsigned long long), stream));
     RL_TRY(hipMemsetAsync(live + 1, 0xFF, sizeof(unsigned long long), stream));  // -1 as an int
     RL_TRY(hipMemsetAsync(count, 0, sizeof(unsigned) * (size_t)n, stream));
@@ -194,28 +208,22 @@ int relabel_create(Relabel *rl, int64_t n, int64_t nnz, const int64_t *row_ptr, 
     else if (nnz) count_sources_kernel<<<blocks, threads, 0, stream>>>(col, nnz, count);
     if (!keep_rows) order_keys_kernel<<<blocks, threads, 0, stream>>>(row_ptr, n, count, live);
     iota_kernel<<<blocks, threads, 0, stream>>>(ids, n);
-    // stable descending sort by gather count: order[new] = old
-    RL_TRY(rocprim::radix_sort_pairs_desc(nullptr, temp_bytes, count, count_sorted, ids, rl->order, (size_t)n, 0, 32,
-                                          stream));
-    RL_TRY(rocprim::exclusive_scan(nullptr, need, len, rl->row_ptr, (int64_t)0, (size_t)n + 1,
-                                   rocprim::plus<int64_t>(), stream));
-    if (need > temp_bytes) temp_bytes = need;
-    RL_TRY(hipMalloc(&temp, temp_bytes ? temp_bytes : 1));
-    RL_TRY(rocprim::radix_sort_pairs_desc(temp, temp_bytes, count, count_sorted, ids, rl->order, (size_t)n, 0, 32,
-                                          stream));
+    need = temp_bytes;
+    RL_TRY(rocprim::radix_sort_pairs_desc(temp, need, count, count_sorted, ids, rl->order, (size_t)n, 0, 32, stream));
     invert_and_lengths_kernel<<<blocks, threads, 0, stream>>>(rl->order, row_ptr, n, new_id, len);
     if (keep_rows) {
         RL_TRY(hipMemcpyAsync(rl->row_ptr, row_ptr, sizeof(int64_t) * ((size_t)n + 1), hipMemcpyDeviceToDevice, stream));
         if (nnz > 0) remap_cols_kernel<<<blocks, threads, 0, stream>>>(col, new_id, nnz, rl->col);
     } else {
-        RL_TRY(rocprim::exclusive_scan(temp, temp_bytes, len, rl->row_ptr, (int64_t)0, (size_t)n + 1,
+        need = temp_bytes;
+        RL_TRY(rocprim::exclusive_scan(temp, need, len, rl->row_ptr, (int64_t)0, (size_t)n + 1,
                                        rocprim::plus<int64_t>(), stream));
     }
     if (nnz > 0 && !keep_rows)
         remap_rows_kernel<<<(int)ceil_div(nnz, kRemapChunk), 256, 0, stream>>>(rl->order, row_ptr, col, new_id, rl->row_ptr, n,
                                                                               nnz, rl->col, reinterpret_cast<int *>(live + 1));
     RL_TRY(hipGetLastError());
-    RL_TRY(hipMemcpyAsync(h_live, live, sizeof(h_live), hipMemcpyDeviceToHost, stream));
+    RL_TRY(hipMemcpyAsync(h_live, live, sizeof(unsigned long long) * 2, hipMemcpyDeviceToHost, stream));
     RL_TRY(hipStreamSynchronize(stream));
     if (!keep_rows) {
         int max_col = -1;
@@ -224,22 +232,23 @@ int relabel_create(Relabel *rl, int64_t n, int64_t nnz, const int64_t *row_ptr, 
         rl->live = (int64_t)max_col < (int64_t)h_live[0] ? (int64_t)h_live[0] : n;
     }
 done:
-    (void)hipFree(count);
-    (void)hipFree(count_sorted);
-    (void)hipFree(ids);
-    (void)hipFree(new_id);
-    (void)hipFree(len);
-    (void)hipFree(temp);
-    (void)hipFree(live);
+    temps.release();
+    if (h_live) (void)hipHostFree(h_live);
     if (rc != DRONE_OK) relabel_destroy(rl);
     return rc;
 }
 
+void relabel_release_csr(Relabel *rl)
+{
+    rl->arena.release();
+    rl->row_ptr = nullptr;
+    rl->col = nullptr;
+}
+
 void relabel_destroy(Relabel *rl)
 {
+    rl->arena.release();
     if (rl->order) (void)hipFree(rl->order);
-    if (rl->row_ptr) (void)hipFree(rl->row_ptr);
-    if (rl->col) (void)hipFree(rl->col);
     *rl = Relabel{};
 }
 

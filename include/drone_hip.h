@@ -117,8 +117,8 @@ void loadOutDegree(Graph *g, PRValues *values, int *globalOutDegree);
 /* DRONE/src/cuda/algorithm/pr.h:20-21 / pr.cu:375-428, 450-488.  float32 delta-push semantics
  * (alpha 0.85, eps 1e-6), computed as a pull over the in-edge CSR; state is left in PRValues exactly
  * as the reference leaves it (prValue, accValue, diffValue, globalAcc, globalDiff, g->active).
- * A subgraph of 48 Mi edges or more gets a second, source-sorted copy of its in-edges at the first PR_PEVal
- * (about 10 bytes per edge and 8 ... 18 ms for 65 ... 263 M edges), which about halves the time of every superstep
+ * A subgraph of 24 Mi edges or more gets a second, source-sorted copy of its in-edges at the first PR_PEVal
+ * (about 10 bytes per edge and 4 ... 16 ms for 32 ... 263 M edges), which takes a third to a half off every superstep
  * after it; the environment variable DRONE_PR_ROWBLOCK_MIN_EDGES (an edge count, read at the first PR_PEVal of
  * each graph) moves that limit, e.g. 0 for jobs that run many supersteps on smaller subgraphs. */
 Response PR_PEVal(Graph *g, PRValues *values, int workerId, int workerNum, Comm *comm);
