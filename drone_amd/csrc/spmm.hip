@@ -134,6 +134,12 @@ constexpr int kBitMaxGroups = 1024;
 // the short pieces do.
 constexpr int kBitMinPiece = 32;
 constexpr double kBitMsPerCellTile = 0.135e-9;  // ms: 0.135 ps per cell and 32 feature columns
+// A gather from an operand that does not fit the Infinity Cache (256 MB; 192 MB leaves room for everything else) is
+// priced three times higher: its feature rows come from HBM.  On the 4.2 M-vertex / 90 M-entry row-normalised graph
+// this gives the 16-wide product a bit region at all (1.29 -> 1.16 ms) and leaves the 64- and 256-wide ones where they
+// were (1.82, 8.8 -> 8.7 ms; factor 5: 1.99 / 8.97); the 128-wide product of the R-MAT scale-20 layer (1 M vertices) 2.09 -> 1.82 ms.
+constexpr double kFarOperandBytes = 192e6;
+constexpr double kFarGatherFactor = 3.0;
 static_assert(kDenseMaxCols / kDenseChunk <= kBitMaxChunks, "the density histogram keeps at most 128 chunks per wavefront");
 
 template <int VEC> struct VecT;
@@ -754,12 +760,13 @@ int build_band_pieces(drone_spmm_plan *p, const std::vector<int> &h_rp, const st
             if (p->scaled) {
                 // bit core: per group, the leading chunks that maximise (gathers saved) - (cells multiplied)
                 const int feature_tiles = (int)ceil_div(p->max_k, 32);
+                const double gather_ms = kGatherMsPerEntry * ((double)p->n_cols * p->max_k * sizeof(float) > kFarOperandBytes ? kFarGatherFactor : 1.0);
                 for (int g = 0; g < groups; ++g) {
                     const double cells = (double)ceil_div(group_begin[g + 1] - group_begin[g], kBitTileRows) * kBitTileRows * kDenseChunk;
                     double run = 0.0, best = 0.0;
                     int w = 0;
                     for (int c = 0; c < chunks; ++c) {
-                        run += hist[(size_t)g * chunks + c] * p->max_k * kGatherMsPerEntry - cells * feature_tiles * kBitMsPerCellTile;
+                        run += hist[(size_t)g * chunks + c] * p->max_k * gather_ms - cells * feature_tiles * kBitMsPerCellTile;
                         if (run > best) { best = run; w = c + 1; }
                     }
                     if (w == 0) break;  // the dense rows must be a leading run of the ranking
