@@ -123,6 +123,8 @@ SIGNATURES = {
     "drone_relu_backward_f32": (_I, [_P, _P, _I64, _P]),
     "drone_dropout_mask": (_I, [_P, _I64, _U64, _U64, _F, _P]),
     "drone_dropout_apply_f32": (_I, [_P, _P, _I64, _F, _P]),
+    "drone_relu_dropout_forward_f32": (_I, [_P, _P, _P, _I64, _U64, _U64, _F, _P]),
+    "drone_relu_dropout_backward_f32": (_I, [_P, _P, _P, _I64, _F, _P]),
     "drone_cross_entropy_f32": (_I, [_I, _I, _P, _I, _P, _P, _I, _F, _P, _P, _P]),
     "drone_accuracy_f32": (_I, [_I, _I, _P, _I, _P, _P, _P, _P, _P]),
     "drone_sum_squares_f32": (_I, [_P, _I64, _P, _P]),

@@ -235,8 +235,9 @@ extern "C" int drone_gcn_tensor(struct drone_gcn *h, const char *name, void **pt
         if (ld) *ld = l;
         return DRONE_OK;
     };
-    if (!strcmp(name, "relu_mask")) return flat(m->relu->mask_ptr(), N, m->layer1_var2->cols, m->layer1_var2->ld);
-    if (!strcmp(name, "keep1") && m->drop) return flat(m->drop->keep_ptr(), N, m->layer1_var2->cols, m->layer1_var2->ld);
+    if (!strcmp(name, "relu_mask"))
+        return flat(m->relu_drop ? m->relu_drop->mask_ptr() : m->relu->mask_ptr(), N, m->layer1_var2->cols, m->layer1_var2->ld);
+    if (!strcmp(name, "keep1") && m->relu_drop) return flat(m->relu_drop->keep_ptr(), N, m->layer1_var2->cols, m->layer1_var2->ld);
     if (!strcmp(name, "truth")) return flat(m->truth, 1, N, N);
     if (!strcmp(name, "val")) return flat(m->adj->val, 1, (int)nnz, (int)nnz);
     if (!strcmp(name, "valT")) return flat(m->adj->valT, 1, (int)nnz, (int)nnz);

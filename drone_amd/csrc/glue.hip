@@ -59,6 +59,64 @@ __global__ void dropout_apply_kernel(float *__restrict__ x, const uint8_t *__res
         x[i] *= keep[i] ? scale : 0.0f;
 }
 
+// ReLU and the dropout that follows it in one pass over the activations (the two modules apart read and write them
+// twice and the keep-mask three times): element by element the arithmetic of relu_forward_kernel, dropout_mask_kernel
+// and dropout_apply_kernel in that order.  Four elements per lane when the count allows 16-byte accesses.
+template <int V>
+__global__ void relu_dropout_forward_kernel(float *__restrict__ x, uint8_t *__restrict__ mask, uint8_t *__restrict__ keep,
+                                            int64_t n, uint64_t seed, uint64_t step, float p, float scale)
+{
+    const uint64_t key = splitmix64_dev(splitmix64_dev(seed) ^ (step * 0xD1342543DE82EF95ull));
+    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q * V < n; q += (int64_t)gridDim.x * blockDim.x) {
+        float v[V];
+        uint8_t m[V], k[V];
+        if constexpr (V == 4) {
+            const float4 t = reinterpret_cast<const float4 *>(x)[q];
+            v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+        } else {
+            v[0] = x[q];
+        }
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            const int64_t i = q * V + j;
+            m[j] = v[j] > 0;
+            const float u = (float)(splitmix64_dev(key + (uint64_t)i) >> 40) * (1.0f / 16777216.0f);
+            k[j] = u >= p;
+            const float r = m[j] ? v[j] : 0.0f;
+            v[j] = r * (k[j] ? scale : 0.0f);
+        }
+        if constexpr (V == 4) {
+            reinterpret_cast<float4 *>(x)[q] = make_float4(v[0], v[1], v[2], v[3]);
+            reinterpret_cast<uchar4 *>(mask)[q] = make_uchar4(m[0], m[1], m[2], m[3]);
+            reinterpret_cast<uchar4 *>(keep)[q] = make_uchar4(k[0], k[1], k[2], k[3]);
+        } else {
+            x[q] = v[0];
+            mask[q] = m[0];
+            keep[q] = k[0];
+        }
+    }
+}
+
+// The two backward steps in the module list's order: g *= keep ? scale : 0 (dropout), then g = 0 where the ReLU was off.
+template <int V>
+__global__ void relu_dropout_backward_kernel(float *__restrict__ g, const uint8_t *__restrict__ mask,
+                                             const uint8_t *__restrict__ keep, int64_t n, float scale)
+{
+    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q * V < n; q += (int64_t)gridDim.x * blockDim.x) {
+        if constexpr (V == 4) {
+            float4 t = reinterpret_cast<const float4 *>(g)[q];
+            const uchar4 m = reinterpret_cast<const uchar4 *>(mask)[q], k = reinterpret_cast<const uchar4 *>(keep)[q];
+            t.x *= k.x ? scale : 0.0f; t.y *= k.y ? scale : 0.0f; t.z *= k.z ? scale : 0.0f; t.w *= k.w ? scale : 0.0f;
+            if (!m.x) t.x = 0; if (!m.y) t.y = 0; if (!m.z) t.z = 0; if (!m.w) t.w = 0;
+            reinterpret_cast<float4 *>(g)[q] = t;
+        } else {
+            float t = g[q] * (keep[q] ? scale : 0.0f);
+            if (!mask[q]) t = 0;
+            g[q] = t;
+        }
+    }
+}
+
 // L lanes per row, 64 / L rows per wavefront (L = the power of two that gives a lane at most four classes: a whole
 // wavefront per 41-class row left a third of the lanes idle and took 74 us for 232,965 rows).  grad = softmax - onehot on
 // labelled rows, 0 elsewhere; the per-block loss sum and labelled-row count go to block_loss / block_count.
@@ -304,6 +362,38 @@ extern "C" int drone_dropout_apply_f32(float *x, const uint8_t *keep, int64_t n,
     DRONE_REQUIRE(n >= 0 && (n == 0 || (x && keep)) && p >= 0.0f && p < 1.0f, "operand / probability");
     if (n == 0) return DRONE_OK;
     dropout_apply_kernel<<<grid_for(n), kThreads, 0, as_stream(stream)>>>(x, keep, n, 1 / (1 - p));
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
+extern "C" int drone_relu_dropout_forward_f32(float *x, uint8_t *mask, uint8_t *keep, int64_t n, uint64_t seed,
+                                              uint64_t step, float p, drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(n >= 0 && (n == 0 || (x && mask && keep)) && p >= 0.0f && p < 1.0f, "operands / probability");
+    if (n == 0) return DRONE_OK;
+    const bool wide = n % 4 == 0 && (reinterpret_cast<uintptr_t>(x) % 16 == 0) &&
+                      (reinterpret_cast<uintptr_t>(mask) % 4 == 0) && (reinterpret_cast<uintptr_t>(keep) % 4 == 0);
+    if (wide)
+        relu_dropout_forward_kernel<4><<<grid_for(n / 4, 2), kThreads, 0, as_stream(stream)>>>(x, mask, keep, n, seed, step, p, 1 / (1 - p));
+    else
+        relu_dropout_forward_kernel<1><<<grid_for(n), kThreads, 0, as_stream(stream)>>>(x, mask, keep, n, seed, step, p, 1 / (1 - p));
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
+extern "C" int drone_relu_dropout_backward_f32(float *grad, const uint8_t *mask, const uint8_t *keep, int64_t n, float p,
+                                               drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(n >= 0 && (n == 0 || (grad && mask && keep)) && p >= 0.0f && p < 1.0f, "operands / probability");
+    if (n == 0) return DRONE_OK;
+    const bool wide = n % 4 == 0 && (reinterpret_cast<uintptr_t>(grad) % 16 == 0) &&
+                      (reinterpret_cast<uintptr_t>(mask) % 4 == 0) && (reinterpret_cast<uintptr_t>(keep) % 4 == 0);
+    if (wide)
+        relu_dropout_backward_kernel<4><<<grid_for(n / 4, 2), kThreads, 0, as_stream(stream)>>>(grad, mask, keep, n, 1 / (1 - p));
+    else
+        relu_dropout_backward_kernel<1><<<grid_for(n), kThreads, 0, as_stream(stream)>>>(grad, mask, keep, n, 1 / (1 - p));
     DRONE_HIP_TRY(hipGetLastError());
     return DRONE_OK;
 }

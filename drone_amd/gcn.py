@@ -128,6 +128,15 @@ def dropout_apply(x, keep, p, stream=0):
     check(lib().drone_dropout_apply_f32(_ptr(x), _ptr(keep), x.numel(), float(p), stream))
 
 
+def relu_dropout_forward(x, mask, keep, seed, step, p, stream=0):
+    check(lib().drone_relu_dropout_forward_f32(_ptr(x), _ptr(mask), _ptr(keep), x.numel(), int(seed), int(step), float(p),
+                                               stream))
+
+
+def relu_dropout_backward(g, mask, keep, p, stream=0):
+    check(lib().drone_relu_dropout_backward_f32(_ptr(g), _ptr(mask), _ptr(keep), g.numel(), float(p), stream))
+
+
 def cross_entropy(logits, truth, classes=None, grad=None, grad_scale=1.0, stream=0):
     """Returns (loss tensor [1], count tensor [1]); fills grad when given."""
     import torch

@@ -291,6 +291,37 @@ public:
     const uint8_t *keep_ptr() const { return keep; }
 };
 
+// ReLU and Dropout on one variable as one module: the same results and masks as the two in a row, one pass over the
+// activations each way instead of two (and no separate pass that draws the mask).
+class ReLUDropout : public Module {
+    Variable *in;
+    float p;
+    uint64_t seed, step = 0;
+    uint8_t *mask = nullptr, *keep = nullptr;
+    drone_stream_t s;
+public:
+    ReLUDropout(Variable *in_, float p_, uint64_t seed_, std::string name, drone_stream_t stream)
+        : in(in_), p(p_), seed(seed_), s(stream)
+    {
+        ModuleName = std::move(name);
+        DRONE_GCN_HIP(hipMalloc(&mask, (size_t)in->rows * in->ld));
+        DRONE_GCN_HIP(hipMalloc(&keep, (size_t)in->rows * in->ld));
+    }
+    ~ReLUDropout() override { (void)hipFree(mask); (void)hipFree(keep); }
+    void forward(bool training) override
+    {
+        const int64_t cnt = (int64_t)in->rows * in->ld;
+        if (training) DRONE_GCN_CHECK(drone_relu_dropout_forward_f32(in->data, mask, keep, cnt, seed, step++, p, s));
+        else DRONE_GCN_CHECK(drone_relu_forward_f32(in->data, mask, cnt, 0, s));
+    }
+    void backward() override
+    {
+        DRONE_GCN_CHECK(drone_relu_dropout_backward_f32(in->grad, mask, keep, (int64_t)in->rows * in->ld, p, s));
+    }
+    const uint8_t *mask_ptr() const { return mask; }
+    const uint8_t *keep_ptr() const { return keep; }
+};
+
 // cuda_module.cu:406-483: writes logits->grad (sum-reduced) when training and the mean loss.
 class CrossEntropyLoss : public Module {
     Variable *logits;
@@ -402,8 +433,8 @@ public:
     const int *mirror2worker = nullptr;    // device [N] (Graph::Mirror2Worker) with replicas, else null
     float *l2_sum = nullptr;               // device scalar: sum of W1^2 (cuda_gcn.cu:254-260)
     CrossEntropyLoss *ce = nullptr;
-    ReLU *relu = nullptr;
-    Dropout *drop = nullptr;
+    ReLU *relu = nullptr;              // layer 1 without dropout
+    ReLUDropout *relu_drop = nullptr;  // layer 1 with dropout
     int *truth = nullptr;   // device [N]: label on rows of the current split, -1 elsewhere
     int truth_split = -1, truth_count = 0;
     int *counts = nullptr;  // device [2]: correct, labelled
@@ -459,11 +490,12 @@ public:
             graphsum1 = new GraphSum(layer1_var1, layer1_var2, adj.get(), p.hidden_dim, "graphSum_layer1", s, r);
             modules.emplace_back(graphsum1);
         }
-        relu = new ReLU(layer1_var2, "Relu", s);
-        modules.emplace_back(relu);
         if (p.use_dropout) {
-            drop = new Dropout(layer1_var2, p.dropout, p.seed, "dropout_layer1", s);
-            modules.emplace_back(drop);
+            relu_drop = new ReLUDropout(layer1_var2, p.dropout, p.seed, "Relu_dropout_layer1", s);
+            modules.emplace_back(relu_drop);
+        } else {
+            relu = new ReLU(layer1_var2, "Relu", s);
+            modules.emplace_back(relu);
         }
         modules.emplace_back(new Matmul(layer1_var2, layer2_weight, layer2_var1, N, p.hidden_dim, p.output_dim, "matmul_layer2", s,
                                         mirror2worker));

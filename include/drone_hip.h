@@ -284,6 +284,14 @@ int drone_relu_backward_f32(float *grad, const uint8_t *mask, int64_t n, drone_s
  * forward activations and the backward gradients. */
 int drone_dropout_mask(uint8_t *keep, int64_t n, uint64_t seed, uint64_t step, float p, drone_stream_t stream);
 int drone_dropout_apply_f32(float *x, const uint8_t *keep, int64_t n, float p, drone_stream_t stream);
+/* The ReLU of layer 1 and the dropout that follows it on the same variable (cuda_gcn.cu:61-64; the dropout line is
+ * commented out there, its module is cuda_module.cu:539-564) in one pass each way: forward = drone_relu_forward_f32 (training), drone_dropout_mask, drone_dropout_apply_f32
+ * in that order, backward = drone_dropout_apply_f32 then drone_relu_backward_f32, element by element the same results
+ * and the same two masks. */
+int drone_relu_dropout_forward_f32(float *x, uint8_t *mask, uint8_t *keep, int64_t n, uint64_t seed, uint64_t step,
+                                   float p, drone_stream_t stream);
+int drone_relu_dropout_backward_f32(float *grad, const uint8_t *mask, const uint8_t *keep, int64_t n, float p,
+                                    drone_stream_t stream);
 /* cuda_kernel.cu:295-379 + cuda_module.cu:406-483.  truth[i] < 0 (or >= classes) = unlabelled.  grad (optional) receives
  * grad_scale * (softmax - onehot) on labelled rows and 0 elsewhere.  grad_scale = 1 is the reference's
  * SUM-reduced gradient (count_grad = 1, cuda_module.cu:452); 1/labelled-count gives the mean-reduced one.

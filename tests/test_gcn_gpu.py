@@ -283,6 +283,34 @@ def test_relu_dropout(T, oracle):
     np.testing.assert_array_equal(xd.cpu().numpy(), oracle.dropout_forward(x, k, 0.5))
 
 
+@pytest.mark.parametrize("shape", [(1000, 37), (999, 128), (1, 1), (513, 44)])
+def test_relu_dropout_in_one_pass(T, oracle, shape):
+    """The one-pass form against the oracle's ReLU and dropout applied in a row, and bit for bit against the three
+    separate entry points (same activations, same two masks, same gradients); element counts that do and do not allow
+    16-byte accesses."""
+    from drone_amd import gcn
+    rng = np.random.default_rng(shape[1])
+    x = rng.normal(size=shape).astype(np.float32)
+    x[rng.random(x.shape) < 0.1] = 0.0
+    g = rng.normal(size=shape).astype(np.float32)
+    a, ma, ka = dev(T, x), T.zeros(shape, dtype=T.uint8, device="cuda"), T.zeros(shape, dtype=T.uint8, device="cuda")
+    gcn.relu_forward(a, ma)
+    gcn.dropout_mask(ka, seed=9, step=3, p=0.4)
+    gcn.dropout_apply(a, ka, 0.4)
+    b, mb, kb = dev(T, x), T.ones(shape, dtype=T.uint8, device="cuda") * 7, T.ones(shape, dtype=T.uint8, device="cuda") * 7
+    gcn.relu_dropout_forward(b, mb, kb, seed=9, step=3, p=0.4)
+    assert T.equal(a, b) and T.equal(ma, mb) and T.equal(ka, kb)
+    y, m = oracle.relu_forward(x)
+    np.testing.assert_array_equal(b.cpu().numpy(), oracle.dropout_forward(y, kb.cpu().numpy(), 0.4))
+    np.testing.assert_array_equal(mb.cpu().numpy(), m)
+    ga, gb = dev(T, g), dev(T, g)
+    gcn.dropout_apply(ga, ka, 0.4)
+    gcn.relu_backward(ga, ma)
+    gcn.relu_dropout_backward(gb, mb, kb, 0.4)
+    assert T.equal(ga, gb)
+    np.testing.assert_array_equal(gb.cpu().numpy(), oracle.relu_backward(oracle.dropout_forward(g, kb.cpu().numpy(), 0.4), m))
+
+
 @pytest.mark.parametrize("classes,ld_pad", [(41, 0), (41, 3), (7, 0), (3, 1), (100, 0)])
 def test_cross_entropy_accuracy_argmax(T, oracle, classes, ld_pad):
     from drone_amd import gcn
