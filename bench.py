@@ -198,7 +198,7 @@ def bench_gcn_step(steps, warmup, cpu_baseline=False):
     plan = gcn.SpmmPlan(rp, ci, val, N, max_k=HID, row_scale=scale, col_scale=scale)
     plain = gcn.SpmmPlan(rp, ci, val, N, max_k=HID)          # what an arbitrary-valued matrix gets: fp32 rectangles
     kernels, plain_ms = [], {}
-    for K, ld in ((HID, HID), (CLS, 44)):
+    for K, ld in ((HID, HID), (CLS, 48)):
         B = torch.rand((N, ld), device="cuda") * 2 - 1
         out = torch.empty((N, ld), device="cuda")
         ms = time_call(lambda: gcn.spmm(plan, rp, ci, val, B[:, :K], K=K, out=out[:, :K]), reps=5)

@@ -245,7 +245,7 @@ def _spmm_checks_config4(torch, gcn, N, HID, CLS, rp, ci, val, A64, degree_scale
     rows = cs[rp[1:].long()] - cs[rp[:-1].long()]
     assert float(((got[:, 0].double() - rows).abs() / rows.abs().clamp(min=1e-30)).max()) <= 1e-4
     # adjointness at K = 41 and 128
-    for K, ld in ((CLS, 44), (HID, HID)):
+    for K, ld in ((CLS, 44), (CLS, 48), (HID, HID)):
         X = (torch.rand((N, ld), device="cuda") * 2 - 1)[:, :K]
         Y = (torch.rand((N, ld), device="cuda") * 2 - 1)[:, :K]
         AX = torch.empty((N, ld), device="cuda")[:, :K]
