@@ -362,6 +362,15 @@ def bench_traverse(cpu_baseline=True):
     w = CCWorkerCUDA(n, us, vs)
     lab = run(w, len(us), "cc")
     w.close()
+    # a path of 20,000 vertices: every hop is a round of its own (one launch runs them while the list stays short)
+    hops = 20000
+    pu = np.arange(hops - 1, dtype=np.int32)
+    w = SSSPWorkerCUDA(hops, pu, pu + 1, startId=0)
+    w.peval()
+    ms = min(timed_ms(w.peval) for _ in range(3))
+    far = float(w.read()[-1])
+    w.close()
+    out["sssp_path"] = {"vertices": hops, "peval_ms": ms, "us_per_hop": ms * 1e3 / (hops - 1), "last_distance": far}
     if cpu_baseline:
         from oracle import oracle
         nl, g2l, l2g, index, dst = oracle.build_graph(n, u, v)
