@@ -163,7 +163,8 @@ int drone_pr_plan_create_ex(drone_pr_plan **plan, int64_t n, int64_t nnz, const 
                             const int32_t *col_idx, const double *inv_outdeg, int flags, drone_stream_t stream);
 int drone_pr_plan_destroy(drone_pr_plan *plan);
 /* Runs `iters` iterations from r_0 = 1/N and writes r_iters to rank_out [n] (device).
- * Asynchronous on `stream`; allocates nothing. */
+ * Asynchronous on `stream`; allocates nothing and launches kernels only (no copies, clears or waits), so a run can be
+ * recorded into a HIP graph and replayed while profiling (drone_pr_profile_enable) is off. */
 int drone_pr_run_f64(drone_pr_plan *plan, double alpha, int iters, double *rank_out,
                      drone_stream_t stream);
 /* Per-iteration timing with HIP events on the launch stream.  When enabled, every iteration inside
@@ -197,7 +198,10 @@ int drone_pr_run_workers_f64(Graph *g, PRValues *values, int workerId, int worke
  * Calls are asynchronous on `stream`.  Apart from plan creation, the transpose (a set-up step) and
  * grow-only scratch kept per (device, stream) by drone_sgemm_rm_f32 (split reductions) and
  * drone_cross_entropy_f32, nothing allocates; calls on different streams may overlap, except that two products with
- * the SAME plan share the plan's partial-row scratch and must not run at the same time. */
+ * the SAME plan share the plan's partial-row scratch and must not run at the same time.  drone_spmm_csr_f32 only
+ * launches kernels and records / waits for events between `stream` and the plan's own side stream, so it can be
+ * recorded into a HIP graph on a capturing stream (drone_sgemm_rm_f32 as well once its scratch has grown to the
+ * shape, drone_sgemm_rm_f32_noalloc always). */
 
 /* cuda_gcn/src/cuda/cuda_kernel.cu:145-155 (launched at cuda_module.cu:163):
  * v[e(u->col)] = 1 / sqrtf(1.0 * out_deg[u] * in_deg[col]) for every entry of row u. */
