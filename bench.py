@@ -28,7 +28,7 @@ def log(*a):
     print("[bench]", *a, file=sys.stderr, flush=True)
 
 
-PR_KERNELS = ("pr_rowblock_kernel<drone::PrF64Epi>", "pr_rowblock_merge_kernel<drone::PrF64Epi>")
+PR_KERNELS = ("pr_rowblock_kernel<drone::PrF64Epi, 6>", "pr_rowblock_merge_kernel<drone::PrF64Epi>")  # the instance a plan of this size launches
 PR_TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "pr_rowblock_pagerank_c2.hbm_traffic.txt")
 
 

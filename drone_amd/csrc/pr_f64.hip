@@ -176,7 +176,9 @@ extern "C" int drone_pr_plan_create_ex(drone_pr_plan **out, int64_t n, int64_t n
             p->units = p->rb.num_blocks;
             // the row-ordered copy is only needed to build the blocks
             relabel_release_csr(&p->rl);
-            DRONE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&pr_rowblock_kernel<PrF64Epi>),
+            DRONE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&pr_rowblock_kernel<PrF64Epi, kRbUnroll>),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, kRbLdsBytes));
+            DRONE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&pr_rowblock_kernel<PrF64Epi, kRbUnrollDeep>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, kRbLdsBytes));
         }
         MergeTiling shape;  // scratch is sized by the number of work units of the active mode
@@ -311,7 +313,9 @@ extern "C" int drone_pr_run_f64(drone_pr_plan *p, double alpha, int iters, doubl
             spmv_merge_kernel<double, int64_t, kPrIpt, PrF64Epi><<<p->mt.num_tiles, kSpmvBlock, 0, s>>>(
                 p->rows, p->nnz, p->mt.tile_row, p->rl.row_ptr, p->rl.col, epi, carry, p->ms.tile_stat);
         } else {
-            pr_rowblock_kernel<PrF64Epi><<<p->rb.num_units, kRbThreads, kRbLdsBytes, s>>>(
+            const auto sweep = p->rb.unroll == kRbUnrollDeep ? &pr_rowblock_kernel<PrF64Epi, kRbUnrollDeep>
+                                                             : &pr_rowblock_kernel<PrF64Epi, kRbUnroll>;
+            sweep<<<p->rb.num_units, kRbThreads, kRbLdsBytes, s>>>(
                 p->rb.block_row, p->rb.block_nnz, p->rb.col, p->rb.lrow, p->rb.stream, p->rb.batch_info, p->rb.block_batch,
                 p->rb.block_wide, p->rb.unit_block, p->rb.block_units, p->rb.block_unit0, p->rb.block_partial,
                 p->rb.partial, epi, carry, p->ms.tile_stat);

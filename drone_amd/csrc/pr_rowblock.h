@@ -34,6 +34,12 @@ constexpr int kRbThreads = 1024;
 constexpr int kRbRows = 16384;       // most rows ending in one block (LDS accumulators: 128 KB)
 constexpr int kRbMaxItems = 1 << 20; // most entries in one block (the plan picks a power of two up to this)
 constexpr int kRbUnroll = 4;    // batches in flight per wavefront; with the compact entries 2 / 3 / 4 / 6 / 8: 0.679 / 0.577 / 0.552 / 0.544 / 0.554 ms
+// Six batches in flight only pay where a work-group sweeps a million entries: fp64 iteration at R-MAT scale 20 / 22 /
+// 23 / 24 with 4 in flight 0.0667 / 0.166 / 0.290 / 0.5515 ms, with 6: 0.0677 / 0.170 / 0.292 / 0.542 ms (the float
+// entry points, whose work-groups sweep half as much: 0.087 / 0.202 / 0.334 / 0.649 against 0.101 / 0.199 / 0.329 /
+// 0.644 ms per superstep, left at 4).  RowBlocks::unroll says which instance the fp64 plan launches.
+constexpr int kRbUnrollDeep = 6;
+constexpr int kRbDeepItems = 1 << 20;  // entries per work-group from which the deep instance is used
 constexpr int kRbSplit = 8;         // most work-groups that share one block of a large matrix
 constexpr int kRbLdsBytes = (kRbRows + 8) * (int)sizeof(double);  // rows ending in a block <= kRbRows + 1, + the open row
 
@@ -71,6 +77,7 @@ struct RowBlocks {
     int num_split = 0;
     int32_t *split_block = nullptr;  // device [num_split]: the blocks with more than one unit
     double *partial = nullptr;       // device: per split block, block_units x (rows + 1) row sums (8-byte values)
+    int unroll = kRbUnroll;          // batches in flight per wavefront that suit these blocks (kRbUnroll or kRbUnrollDeep)
     DeviceArena arena;               // every array above except `stream` is a piece of this one allocation
 };
 
@@ -154,7 +161,7 @@ __device__ __forceinline__ void rb_read(const double *s_acc, const uint32_t *s_f
     out = PushF2{(float)s_acc[i], (float)((s_flag[i & (kRbFlagWords - 1)] >> (i / kRbFlagWords)) & 1u)};
 }
 
-template <bool kWide, typename Epi>
+template <bool kWide, int kU, typename Epi>
 __device__ __forceinline__ void rb_accumulate(int64_t block_begin, int64_t block_end, int share, int shares, int tid,
                                               const int32_t *__restrict__ col, const uint16_t *__restrict__ lrow,
                                               const uint8_t *__restrict__ stream, const int2 *__restrict__ infos,
@@ -179,24 +186,24 @@ __device__ __forceinline__ void rb_accumulate(int64_t block_begin, int64_t block
     // clamped to the block's last entry anyway).
     const int last_batch = __builtin_amdgcn_readfirstlane((int)((last - block_begin) >> 6));
     int batch = __builtin_amdgcn_readfirstlane((int)((s0 - block_begin) >> 6));
-    int2 info[kRbUnroll], info_next[kRbUnroll];
+    int2 info[kU], info_next[kU];
     if (!kWide) {
 #pragma unroll
-        for (int k = 0; k < kRbUnroll; ++k) info[k] = infos[batch + k < last_batch ? batch + k : last_batch];
+        for (int k = 0; k < kU; ++k) info[k] = infos[batch + k < last_batch ? batch + k : last_batch];
     }
-    for (int64_t base = s0; base < s1; base += kWave * kRbUnroll, batch += kRbUnroll) {
-        uint32_t a[kRbUnroll];
-        int32_t g[kRbUnroll];
-        int bits[kRbUnroll];
+    for (int64_t base = s0; base < s1; base += kWave * kU, batch += kU) {
+        uint32_t a[kU];
+        int32_t g[kU];
+        int bits[kU];
         if (!kWide) {
 #pragma unroll
-            for (int k = 0; k < kRbUnroll; ++k) {
-                const int next = batch + kRbUnroll + k;
+            for (int k = 0; k < kU; ++k) {
+                const int next = batch + kU + k;
                 info_next[k] = infos[next < last_batch ? next : last_batch];
             }
         }
 #pragma unroll
-        for (int k = 0; k < kRbUnroll; ++k) {
+        for (int k = 0; k < kU; ++k) {
             int64_t e = base + k * kWave + lane;
             e = e < last ? e : last;
             if (kWide) {
@@ -210,9 +217,9 @@ __device__ __forceinline__ void rb_accumulate(int64_t block_begin, int64_t block
                 bits[k] = 8 * bytes;
             }
         }
-        int c[kRbUnroll], l[kRbUnroll];
+        int c[kU], l[kU];
 #pragma unroll
-        for (int k = 0; k < kRbUnroll; ++k) {
+        for (int k = 0; k < kU; ++k) {
             if (kWide) {
                 c[k] = (int)a[k];
                 l[k] = g[k];
@@ -223,20 +230,20 @@ __device__ __forceinline__ void rb_accumulate(int64_t block_begin, int64_t block
                 l[k] = (int)(v >> offset_bits);
             }
         }
-        Acc v[kRbUnroll];
+        Acc v[kU];
 #pragma unroll
-        for (int k = 0; k < kRbUnroll; ++k) v[k] = epi.load(c[k]);
+        for (int k = 0; k < kU; ++k) v[k] = epi.load(c[k]);
 #pragma unroll
-        for (int k = 0; k < kRbUnroll; ++k)
+        for (int k = 0; k < kU; ++k)
             rb_add(s_acc, s_flag, l[k], base + k * kWave + lane < s1, v[k]);
         if (!kWide) {
 #pragma unroll
-            for (int k = 0; k < kRbUnroll; ++k) info[k] = info_next[k];
+            for (int k = 0; k < kU; ++k) info[k] = info_next[k];
         }
     }
 }
 
-template <typename Epi>
+template <typename Epi, int kU = kRbUnroll>
 __global__ __launch_bounds__(kRbThreads) void pr_rowblock_kernel(const int32_t *__restrict__ block_row,
                                                                  const int64_t *__restrict__ block_nnz,
                                                                  const int32_t *__restrict__ col,
@@ -284,9 +291,9 @@ __global__ __launch_bounds__(kRbThreads) void pr_rowblock_kernel(const int32_t *
     __syncthreads();
 
     if (wide)
-        rb_accumulate<true>(eb, ee, share, shares, tid, col, lrow, stream, infos, epi, s_acc, s_flag);
+        rb_accumulate<true, kU>(eb, ee, share, shares, tid, col, lrow, stream, infos, epi, s_acc, s_flag);
     else
-        rb_accumulate<false>(eb, ee, share, shares, tid, col, lrow, stream, infos, epi, s_acc, s_flag);
+        rb_accumulate<false, kU>(eb, ee, share, shares, tid, col, lrow, stream, infos, epi, s_acc, s_flag);
     __syncthreads();
 
     if (shares > 1) {

@@ -1,5 +1,6 @@
 #include "pr_rowblock.h"
 
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 #include <rocprim/device/device_radix_sort.hpp>
@@ -283,6 +284,11 @@ int row_blocks_create(RowBlocks *rb, int64_t n, int64_t nnz, const int64_t *row_
     // 0.34 / 0.70 with 512 K, - / 0.77 with 1 M (the rule above picks 256 K / 1 M).
     if (uniform_rows && items > 32768) items >>= 1;
     const int unit_items = items;          // entries one work-group sweeps
+    rb->unroll = unit_items >= kRbDeepItems ? kRbUnrollDeep : kRbUnroll;
+    if (const char *depth = getenv("DRONE_PR_SWEEP_DEPTH")) {  // fixes the choice: how small graphs reach the deep instance in tests
+        if (atoi(depth) == kRbUnrollDeep) rb->unroll = kRbUnrollDeep;
+        else if (atoi(depth) == kRbUnroll) rb->unroll = kRbUnroll;
+    }
     // Large matrices get blocks that several work-groups share.  Measured, ms per iteration at R-MAT scale 20 / 22 /
     // 24: with blocks of the weighted split alone and 1 / 2 / 4 / 8 / 16 work-groups per block 0.060 0.063 0.079
     // 0.081 0.087 / 0.175 0.181 0.172 0.216 0.184 / 0.679 0.649 0.617 0.659 0.670 (small matrices lose more to the

@@ -156,7 +156,9 @@ int drone_pr_plan_create(drone_pr_plan **plan, int64_t n, int64_t nnz, const int
 #define DRONE_PR_DETERMINISTIC 1
 /* Tuning overrides of the default mode.  Row blocks of a large matrix (about 50 M entries and more) are shared by up
  * to four work-groups, which then find more entries per cache line of the gather source; small matrices keep one
- * work-group per block.  DRONE_PR_SHARED_BLOCKS forces sharing, DRONE_PR_WHOLE_BLOCKS forbids it. */
+ * work-group per block.  DRONE_PR_SHARED_BLOCKS forces sharing, DRONE_PR_WHOLE_BLOCKS forbids it.  (The sweep keeps
+ * four 64-entry batches in flight per wavefront, six where a work-group sweeps a million entries;
+ * DRONE_PR_SWEEP_DEPTH=4 or 6 in the environment at plan creation fixes that choice.) */
 #define DRONE_PR_SHARED_BLOCKS 2
 #define DRONE_PR_WHOLE_BLOCKS 4
 int drone_pr_plan_create_ex(drone_pr_plan **plan, int64_t n, int64_t nnz, const int64_t *row_ptr,

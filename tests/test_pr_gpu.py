@@ -100,6 +100,24 @@ def test_pull_f64_edge_cases(torch_cuda, oracle, name, iters, det):
     assert abs(got.sum() - 1.0) < 1e-11
 
 
+@pytest.mark.parametrize("det", MODES[:2])
+def test_pull_f64_deep_sweep_instance(torch_cuda, oracle, det, monkeypatch):
+    """Work-groups that sweep a million entries keep six batches in flight instead of four; DRONE_PR_SWEEP_DEPTH
+    brings that instance of the kernel to graphs a CPU can check: every small case and two R-MAT graphs."""
+    from drone_amd import rmat
+    monkeypatch.setenv("DRONE_PR_SWEEP_DEPTH", "6")
+    for name, (n, src, dst) in small_cases().items():
+        rp, ci, inv = in_csr_np(n, src, dst)
+        for iters in (1, 20):
+            got = run_plan(torch_cuda, rp, ci, inv, iters, **mode_kwargs(det))
+            assert_rel(got, oracle.pr_pull_f64(rp, ci, inv, ALPHA, iters), 1e-9)
+    for scale, ef, seed, iters in ((14, 16, 2, 50), (18, 8, 5, 10)):
+        x = rmat.pagerank_inputs_np(scale, ef, seed)
+        got = run_plan(torch_cuda, x["row_ptr"], x["col_idx"], x["inv_outdeg"], iters, **mode_kwargs(det))
+        assert_rel(got, oracle.pr_pull_f64(x["row_ptr"], x["col_idx"], x["inv_outdeg"], ALPHA, iters), 1e-9)
+        assert abs(got.sum() - 1.0) < 1e-11
+
+
 @pytest.mark.parametrize("det", MODES)
 @pytest.mark.parametrize("scale,ef,seed,iters", [(10, 16, 1, 20), (14, 16, 2, 50), (16, 16, 1, 20), (18, 8, 5, 10), (20, 16, 7, 3)])
 def test_pull_f64_rmat(torch_cuda, oracle, scale, ef, seed, iters, det):
