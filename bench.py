@@ -510,8 +510,8 @@ def main():
                          "rocprofv3 byte counters by)")
     ap.add_argument("--suite", default="default", choices=["pr", "default", "full", "gcn", "sweep", "traverse", "exchange"],
                     help="pr: PageRank only (fp64 pull plan, then the reference's PR_PEVal / PR_IncEVal on the same "
-                         "graph); default: + the GCN training step (configs[3]), the GCN layer (configs[2]) and the "
-                         "SpMM sweep (configs[4]); full: + the SSSP / CC jobs and the replica exchange; gcn, sweep, "
+                         "graph); default (= full): + the GCN training step (configs[3]), the GCN layer (configs[2]), "
+                         "the SpMM sweep (configs[4]), the SSSP / CC jobs and the replica exchange; gcn, sweep, "
                          "traverse, exchange: that part alone")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -624,7 +624,6 @@ def main():
         torch.cuda.empty_cache()
         result["spmm_sweep"] = bench_spmm_sweep(cpu_baseline=not args.no_cpu_baseline)
         torch.cuda.empty_cache()
-    if args.suite == "full":
         result["traverse"] = bench_traverse(cpu_baseline=not args.no_cpu_baseline)
         torch.cuda.empty_cache()
         result["exchange"] = bench_exchange()

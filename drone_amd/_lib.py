@@ -121,6 +121,7 @@ SIGNATURES = {
     "drone_sgemm_noalloc_scratch_bytes": (_I64, []),
     "drone_relu_forward_f32": (_I, [_P, _P, _I64, _I, _P]),
     "drone_relu_backward_f32": (_I, [_P, _P, _I64, _P]),
+    "drone_glorot_uniform_f32": (_I, [_P, _I64, _I, _I, _U64, _P]),
     "drone_dropout_mask": (_I, [_P, _I64, _U64, _U64, _F, _P]),
     "drone_dropout_apply_f32": (_I, [_P, _P, _I64, _F, _P]),
     "drone_relu_dropout_forward_f32": (_I, [_P, _P, _P, _I64, _U64, _U64, _F, _P]),

@@ -134,6 +134,19 @@ drone_transport *transport_of(Comm *comm, int workerNum, const char *who)
 
 void drone::routes_release(RouteLists *r)
 {
+    // Ids received in the last phase of a run have not been reported yet (the count travels with the NEXT phase's chunk
+    // counts): read the counter one last time, so that a partition whose tables do not match cannot pass in silence.
+    if (r->chunk_count) {
+        int seen = 0;
+        const size_t most = (size_t)std::max(r->num_chunks[0], r->num_chunks[1]);
+        if (hipDeviceSynchronize() == hipSuccess &&
+            hipMemcpy(&seen, r->chunk_count + most, sizeof(int), hipMemcpyDeviceToHost) == hipSuccess &&
+            seen > r->unknown_reported) {
+            printf("error global id: %d received ids were not on this worker (last exchange phase)\n", seen - r->unknown_reported);
+            set_error(DRONE_ERR_INVALID, "exchange: %d ids received in the last phase are not on this worker",
+                      seen - r->unknown_reported);
+        }
+    }
     if (r->mirror_vertex) (void)hipFree(r->mirror_vertex);
     if (r->master_vertex) (void)hipFree(r->master_vertex);
     if (r->group_off) (void)hipFree(r->group_off);

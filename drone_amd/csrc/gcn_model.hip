@@ -51,7 +51,7 @@ int make_model(struct drone_gcn **out, const drone_gcn_config *cfg, int64_t nnz,
     DRONE_REQUIRE(out && cfg, "null handle / config");
     DRONE_REQUIRE(cfg->n > 0 && cfg->input_dim > 0 && cfg->hidden_dim > 0 && cfg->output_dim > 0, "dimensions");
     DRONE_REQUIRE(nnz >= 0 && nnz < INT32_MAX && rp && (ci || nnz == 0) && in_degree && out_degree, "graph arrays");
-    DRONE_REQUIRE(X && ldx >= cfg->input_dim && label && split && W1 && W2, "feature / label / weight arrays");
+    DRONE_REQUIRE(X && ldx >= cfg->input_dim && label && split, "feature / label arrays");
     DRONE_REQUIRE(cfg->dropout >= 0.0f && cfg->dropout < 1.0f, "dropout probability");
     DRONE_REQUIRE(!(cfg->fold_input_aggregation && rep && rep->workerNum > 1),
                   "fold_input_aggregation needs a single subgraph");

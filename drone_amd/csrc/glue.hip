@@ -53,6 +53,16 @@ __global__ void dropout_mask_kernel(uint8_t *__restrict__ keep, int64_t n, uint6
     }
 }
 
+// cuda_kernel.cu:470-475: data[i] = (u - 0.5) * scale with u uniform in (0, 1], scale = 2 * sqrt(6 / (in + out)).
+__global__ void glorot_kernel(float *__restrict__ w, int64_t n, uint64_t seed, float scale)
+{
+    const uint64_t key = splitmix64_dev(splitmix64_dev(seed) ^ 0x676C6F726F74ull);
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        const float u = (float)((splitmix64_dev(key + (uint64_t)i) >> 40) + 1) * (1.0f / 16777216.0f);
+        w[i] = (u - 0.5f) * scale;
+    }
+}
+
 __global__ void dropout_apply_kernel(float *__restrict__ x, const uint8_t *__restrict__ keep, int64_t n, float scale)
 {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
@@ -351,6 +361,20 @@ extern "C" int drone_dropout_mask(uint8_t *keep, int64_t n, uint64_t seed, uint6
     DRONE_REQUIRE(n >= 0 && (n == 0 || keep) && p >= 0.0f && p < 1.0f, "mask / probability");
     if (n == 0) return DRONE_OK;
     dropout_mask_kernel<<<grid_for(n), kThreads, 0, as_stream(stream)>>>(keep, n, seed, step, p);
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
+// cuda_variable.cu:18-24 (CUDAVariable::glorot): n weights uniform in (-r, r], r = sqrtf(6 / (in_size + out_size)).
+// The reference draws from cuRAND states seeded with 1234 (cuda_kernel.cu:423-426), whose bit stream cannot be
+// reproduced without cuRAND; here element i is a function of (seed, i) alone.
+extern "C" int drone_glorot_uniform_f32(float *w, int64_t n, int in_size, int out_size, uint64_t seed, drone_stream_t stream)
+{
+    clear_error();
+    DRONE_REQUIRE(n >= 0 && (n == 0 || w) && in_size > 0 && out_size > 0, "weights / fan-in / fan-out");
+    if (n == 0) return DRONE_OK;
+    const float range = sqrtf(6.0f / (float)(in_size + out_size));
+    glorot_kernel<<<grid_for(n), kThreads, 0, as_stream(stream)>>>(w, n, seed, range * 2);
     DRONE_HIP_TRY(hipGetLastError());
     return DRONE_OK;
 }

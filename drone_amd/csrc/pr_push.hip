@@ -116,6 +116,8 @@ __global__ __launch_bounds__(kSpmvBlock) void pr_increment_vertex_kernel(
         push[push_slot ? push_slot[id] : id] = out;
     }
     const double total = block_sum_256(part, s_red);
+    // The last work-group reads block_part[] and nothing else the others wrote: only what went through publish_part is
+    // visible to it before the kernel ends (pr[] / push[] above are plain stores and are not).
     unsigned int one = 0;
     if (threadIdx.x == 0) one = publish_part(block_part + blockIdx.x, total);
     if (!last_block_done(ticket, one)) return;

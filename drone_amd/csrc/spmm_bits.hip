@@ -97,6 +97,19 @@ __device__ __forceinline__ bf16x8 expand_bits(unsigned byte)
     return __builtin_bit_cast(bf16x8, v);
 }
 
+// Waits for the loads that bits_mfma_kernel issues by hand.  The registers they fill are in/out operands of the wait,
+// so every later use of them depends on this statement and the compiler can neither move such a use (or a copy or a
+// spill of the register) above it nor reorder it with the loads, which are volatile as well.
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));  // a register quadruple inline asm can take as "+v"
+template <int kPre>
+__device__ __forceinline__ void staged_loads_landed(u32x4 (&pre)[kPre])
+{
+    static_assert(kPre >= 1 && kPre <= 3, "one operand list per count");
+    if constexpr (kPre == 1) asm volatile("s_waitcnt vmcnt(0)" : "+v"(pre[0]) : : "memory");
+    else if constexpr (kPre == 2) asm volatile("s_waitcnt vmcnt(0)" : "+v"(pre[0]), "+v"(pre[1]) : : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" : "+v"(pre[0]), "+v"(pre[1]), "+v"(pre[2]) : : "memory");
+}
+
 // One work-group (8 wavefronts) per unit: T[512 x 32 NT] = bits(512 x [c0, c1)) * split([c0, c1) x 32 NT), the three
 // parts summed.  Wavefront w owns rows 64 w .. + 64 and all NT feature tiles as 2 x NT accumulators of 32 x 32.  The
 // split operand of 32 columns (a stage: 4 groups x 3 parts x NT tiles x 512 bytes) goes through LDS, double buffered,
@@ -130,10 +143,13 @@ __global__ __launch_bounds__(512, 1) void bits_mfma_kernel(const int *__restrict
     const uint4 *w0 = bits + tile_off[tile] + ((size_t)(2 * wave) * blocks + c0 / kBitBlockCols) * 64 + lane;
     const size_t wstep = (size_t)blocks * 64;
     const uint4 *src = split + (size_t)(c0 / 8) * kGroupVecs;
+    // Every lane loads in every slot: a lane past the stage's last word repeats that word (and does not store it).
+    // With the load under `if (tid + 512 * i < kStageVecs)` its destination register would be merged with an older
+    // value after the branch, and the compiler may do that merge before the load has landed.
     int goff[kPre];
 #pragma unroll
     for (int i = 0; i < kPre; ++i) {
-        const int v = tid + 512 * i;
+        const int v = tid + 512 * i < kStageVecs ? tid + 512 * i : kStageVecs - 1;
         const int g = v / (3 * NT * 32), rem = v % (3 * NT * 32);
         goff[i] = g * kGroupVecs + (rem / (NT * 32)) * 4 * 32 + ((rem / 32) % NT) * 32 + rem % 32;
     }
@@ -145,7 +161,7 @@ __global__ __launch_bounds__(512, 1) void bits_mfma_kernel(const int *__restrict
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    uint4 pre[kPre];
+    u32x4 pre[kPre];
     // The work-groups resident at one time share a column range (launch order) and would walk it in step, all asking
     // one L2 channel for the same line at the same moment: every tile starts at its own block of the range and wraps.
     const int rot = (tile * 5) % nblocks;
@@ -155,11 +171,10 @@ __global__ __launch_bounds__(512, 1) void bits_mfma_kernel(const int *__restrict
     {
         const uint4 *first = src + (size_t)rot * 32 * kGroupVecs;
 #pragma unroll
-        for (int i = 0; i < kPre; ++i)
-            if (tid + 512 * i < kStageVecs) pre[i] = first[goff[i]];
+        for (int i = 0; i < kPre; ++i) pre[i] = __builtin_bit_cast(u32x4, first[goff[i]]);
 #pragma unroll
         for (int i = 0; i < kPre; ++i)
-            if (tid + 512 * i < kStageVecs) s_b[0][tid + 512 * i] = pre[i];
+            if (tid + 512 * i < kStageVecs) s_b[0][tid + 512 * i] = __builtin_bit_cast(uint4, pre[i]);
     }
     __syncthreads();
     for (int kb = 0; kb < nblocks; ++kb) {
@@ -178,15 +193,16 @@ __global__ __launch_bounds__(512, 1) void bits_mfma_kernel(const int *__restrict
 #pragma unroll
         for (int st = 0; st < 8; ++st) {
             const bool more = kb + 1 < nblocks || st < 7;
-            if (more) {
+            {
                 // Issued by hand: written as plain loads, the compiler sinks them to the LDS stores at the end of the
                 // stage (or loads twice) and the whole memory latency is waited for, stage after stage.  The matching
-                // wait is the s_waitcnt below; extra loads in flight only make the compiler's own waits stricter.
-                const uint4 *next = src + (size_t)(st < 7 ? block * 8 + st + 1 : block_next * 8) * 4 * kGroupVecs;
+                // wait is staged_loads_landed() below; extra loads in flight only make the compiler's own waits
+                // stricter.  The loads are issued on every path (the last stage of a unit fetches its own words once
+                // more and drops them), so pre[] is written by straight-line code and read only behind the wait.
+                const uint4 *next = src + (size_t)(!more ? block * 8 + st : st < 7 ? block * 8 + st + 1 : block_next * 8) * 4 * kGroupVecs;
 #pragma unroll
                 for (int i = 0; i < kPre; ++i)
-                    if (tid + 512 * i < kStageVecs)
-                        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(pre[i]) : "v"(next + goff[i]) : "memory");
+                    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(pre[i]) : "v"(next + goff[i]) : "memory");
             }
             const uint4 *cur = s_b[st & 1];
 #pragma unroll
@@ -204,11 +220,11 @@ __global__ __launch_bounds__(512, 1) void bits_mfma_kernel(const int *__restrict
                         acc[1][ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A1, bv, acc[1][ct], 0, 0, 0);
                     }
             }
+            staged_loads_landed(pre);
             if (more) {
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
                 for (int i = 0; i < kPre; ++i)
-                    if (tid + 512 * i < kStageVecs) s_b[(st & 1) ^ 1][tid + 512 * i] = pre[i];
+                    if (tid + 512 * i < kStageVecs) s_b[(st & 1) ^ 1][tid + 512 * i] = __builtin_bit_cast(uint4, pre[i]);
             }
             __syncthreads();
         }

@@ -256,16 +256,36 @@ __global__ __launch_bounds__(kSpmvBlock) void spmv_merge_kernel(
 // (on this GPU a fence at device scope writes back a whole L2, once per work-group that executes it: a vertex kernel of
 // 4096 work-groups took twice its time).  Thread 0 of every work-group stores its part with publish_part - an atomic
 // exchange at device scope, performed where all XCDs see it, whose return value is waited for - and then takes a
-// ticket; the work-group that draws the last ticket reads the parts with load_agent.  Nothing else the other
-// work-groups wrote is guaranteed to be visible to it.
+// ticket; the work-group that draws the last ticket reads the parts with load_agent.
+//
+// What this relies on, beyond the HIP memory model: all three steps are RELAXED atomics at agent scope, and relaxed
+// atomics on different addresses are formally unordered.  The order comes from the hardware and from a data dependency:
+// (1) on gfx942 / gfx950 an atomic read-modify-write at agent scope is carried out at the memory side of the L2s (the
+// counters show one fabric transaction per such atomic), which is the one place every XCD observes, and a *returning*
+// atomic does not hand its result to the wavefront before it has been carried out there; (2) the ticket's increment is
+// made to depend on the exchange's result (the empty asm below), so the ticket atomic cannot be issued before the
+// exchange has returned; (3) the reader's loads are agent-scope atomic loads, which are served from that same place and
+// not from its own L1 / L2.  ONLY values that travel through publish_part (or another returning agent-scope atomic) may
+// be read by the last work-group: plain stores of the other work-groups sit in their XCD's L2 until the kernel ends.
+// The formally ordered form (DRONE_HANDOVER_FENCED=1: relaxed store, acq_rel ticket) is kept for comparison; its
+// release is the L2 write-back described above.
+#ifndef DRONE_HANDOVER_FENCED
+#define DRONE_HANDOVER_FENCED 0
+#endif
 __device__ __forceinline__ unsigned int publish_part(double *slot, double v)
 {
+#if DRONE_HANDOVER_FENCED
+    __hip_atomic_store(reinterpret_cast<unsigned long long *>(slot), (unsigned long long)__double_as_longlong(v),
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return 1u;
+#else
     const unsigned long long old =
         __hip_atomic_exchange(reinterpret_cast<unsigned long long *>(slot), (unsigned long long)__double_as_longlong(v),
                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     unsigned int one = 1u;
     asm volatile("" : "+v"(one) : "v"((unsigned int)old));  // the ticket's increment exists once the exchange has returned
     return one;
+#endif
 }
 
 // True in every thread of the work-group whose thread 0 draws the last ticket of the launch.  Tickets are drawn in
@@ -289,11 +309,19 @@ __device__ __forceinline__ bool last_block_done(unsigned int *ticket, unsigned i
         const unsigned int in_group = group + 1 < groups ? kTicketGroup : blocks - group * kTicketGroup;
         unsigned int *mine = ticket + (size_t)(group + 1) * kTicketStride;
         bool last = false;
+#if DRONE_HANDOVER_FENCED
+        if (__hip_atomic_fetch_add(mine, one, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == in_group - 1) {
+            atomicExch(mine, 0u);
+            last = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == groups - 1;
+            if (last) atomicExch(ticket, 0u);
+        }
+#else
         if (atomicAdd(mine, one) == in_group - 1) {  // returns before the next draw is issued
             atomicExch(mine, 0u);
             last = atomicAdd(ticket, 1u) == groups - 1;
             if (last) atomicExch(ticket, 0u);
         }
+#endif
         s_last = last;
     }
     __syncthreads();
@@ -352,6 +380,8 @@ __global__ __launch_bounds__(kSpmvBlock) void spmv_fixup_kernel(
         stat += tile_stat[t];
     }
     const double total = block_sum_256(stat, s_red);
+    // The last work-group reads block_stat[] and nothing else the others wrote (the rows fixed above are plain stores:
+    // not visible across XCDs before the kernel ends).
     unsigned int one = 0;
     if (threadIdx.x == 0) one = publish_part(block_stat + blockIdx.x, total);
     if (!last_block_done(ticket, one)) return;

@@ -299,6 +299,8 @@ __device__ __forceinline__ void frontier_append(bool take, int v, int degree, in
 
 // The last work-group of a launch that built a list hands {count << 32 | edges, largest degree} to the host (pinned
 // memory) and clears the counters for the next launch.  ticket == nullptr: the host copies and clears them.
+// The two counter words are all it reads of the other work-groups' work, and they are only ever updated by returning
+// agent-scope atomics (see publish_part in spmv_merge.h); the list itself is plain stores, read by the next launch.
 __device__ __forceinline__ void publish_counters(unsigned long long *counters, unsigned int *ticket,
                                                  unsigned long long *host)
 {

@@ -120,6 +120,14 @@ def relu_backward(g, mask, stream=0):
     check(lib().drone_relu_backward_f32(_ptr(g), _ptr(mask), g.numel(), stream))
 
 
+def glorot_uniform(w, in_size, out_size, seed=1234, stream=0):
+    """drone_glorot_uniform_f32 (cuda_variable.cu:18-24 CUDAVariable::glorot): w, a contiguous float32 device tensor,
+    is filled with values uniform in (-r, r], r = sqrt(6 / (in_size + out_size))."""
+    assert w.is_contiguous()
+    check(lib().drone_glorot_uniform_f32(_ptr(w), w.numel(), int(in_size), int(out_size), int(seed), stream))
+    return w
+
+
 def dropout_mask(keep, seed, step, p, stream=0):
     check(lib().drone_dropout_mask(_ptr(keep), keep.numel(), int(seed), int(step), float(p), stream))
 
@@ -185,14 +193,19 @@ class GcnModel:
 
     def __init__(self, rp, ci, in_deg, out_deg, X, label, split, W1, W2, dropout=0.5, lr=0.01, weight_decay=5e-4,
                  use_dropout=False, use_adam=True, mean_gradient=False, seed=1234, stream=0, fold_input_aggregation=False,
-                 worker=None):
+                 worker=None, hidden=None, classes=None):
         """worker: None for a whole graph, or dict(g=Graph pointer, comm=Comm, workerId=, workerNum=, semi_batch=False,
         compress=False) for one subgraph of a vertex cut (drone_gcn_create_worker); rp / ci are then ignored (the
-        adjacency is the subgraph's own out-edge CSR) and in_deg / out_deg are the GLOBAL degrees per local vertex."""
+        adjacency is the subgraph's own out-edge CSR) and in_deg / out_deg are the GLOBAL degrees per local vertex.
+        W1 = W2 = None (with hidden= and classes=): the weights start from the reference's glorot initialisation
+        (cuda_gcn.cu:42, :71), drawn from `seed` and `seed + 1`."""
         from ._lib import GcnConfig
         n, input_dim = X.shape
-        hidden, classes = W1.shape[1], W2.shape[1]
-        assert W1.shape[0] == input_dim and W2.shape[0] == hidden and W1.is_contiguous() and W2.is_contiguous()
+        if W1 is None or W2 is None:
+            assert W1 is None and W2 is None and hidden and classes
+        else:
+            hidden, classes = W1.shape[1], W2.shape[1]
+            assert W1.shape[0] == input_dim and W2.shape[0] == hidden and W1.is_contiguous() and W2.is_contiguous()
         assert X.stride(1) == 1
         cfg = GcnConfig(n, input_dim, hidden, classes, dropout, lr, weight_decay, int(use_dropout), int(use_adam),
                         int(mean_gradient), seed, int(fold_input_aggregation))

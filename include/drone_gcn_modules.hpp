@@ -43,9 +43,9 @@ namespace drone_gcn_mod {
         }                                                                                  \
     } while (0)
 
-// cuda_variable.cuh:17-30.  A row-major rows x cols matrix with leading dimension ld >= cols; ld is rounded
-// up to a multiple of 4 floats so that every row starts 16-byte aligned (the 41-class tensors get ld 44).
-// `size` keeps the reference's meaning (rows * cols logical elements).
+// cuda_variable.cuh:17-30.  A row-major rows x cols matrix with leading dimension ld >= cols.  Activations get ld
+// rounded up to a multiple of 16 floats, so that every row starts on a 64-byte boundary (the 41-class tensors get
+// ld 48); weights stay densely packed (ld = cols).  `size` keeps the reference's meaning (rows * cols logical elements).
 struct Variable {
     float *data = nullptr, *grad = nullptr;
     bool requires_grad, is_weight;
@@ -82,6 +82,12 @@ struct Variable {
         if (grad) (void)hipFree(grad);
     }
     size_t bytes() const { return sizeof(float) * (size_t)rows * ld; }
+    // cuda_variable.cu:18-24: uniform in (-r, r], r = sqrt(6 / (in_size + out_size)).  The padding columns of a
+    // variable whose ld exceeds cols are drawn as well; nothing reads them.
+    void glorot(int in_size, int out_size, uint64_t seed = 1234, drone_stream_t stream = nullptr)
+    {
+        DRONE_GCN_CHECK(drone_glorot_uniform_f32(data, (int64_t)rows * ld, in_size, out_size, seed, stream));
+    }
 };
 
 // cuda_module.cuh:31-37
@@ -444,7 +450,9 @@ public:
     const int *label = nullptr, *split = nullptr;  // device, borrowed
     drone_stream_t s;
 
-    // X: device N x input_dim with leading dimension ldx (borrowed).  W1 / W2: device initial weights (copied).
+    // X: device N x input_dim with leading dimension ldx (borrowed).  W1 / W2: device initial weights (copied), or
+    // null for the reference's own initialisation, glorot(input_dim, hidden_dim) / glorot(hidden_dim, output_dim)
+    // (cuda_gcn.cu:42, :71), drawn from params.seed and params.seed + 1.
     // rep: the vertex cut this subgraph belongs to (null: a whole graph).  rp / ci: the subgraph's out-edge CSR
     // (Graph::index / Graph::dst with replicas); in_degree / out_degree: global degrees per local vertex.
     GCN(const GCNParams &p, int64_t nnz, const int *rp, const int *ci, const int *in_degree, const int *out_degree,
@@ -468,8 +476,10 @@ public:
         layer2_var1 = add(new Variable(N, p.output_dim, true, false));
         layer2_weight = add(new Variable(p.hidden_dim, p.output_dim, true, true));
         output = add(new Variable(N, p.output_dim, true, false));
-        DRONE_GCN_HIP(hipMemcpy(layer1_weight->data, W1, layer1_weight->bytes(), hipMemcpyDeviceToDevice));
-        DRONE_GCN_HIP(hipMemcpy(layer2_weight->data, W2, layer2_weight->bytes(), hipMemcpyDeviceToDevice));
+        if (W1) DRONE_GCN_HIP(hipMemcpy(layer1_weight->data, W1, layer1_weight->bytes(), hipMemcpyDeviceToDevice));
+        else layer1_weight->glorot(p.input_dim, p.hidden_dim, p.seed, s);
+        if (W2) DRONE_GCN_HIP(hipMemcpy(layer2_weight->data, W2, layer2_weight->bytes(), hipMemcpyDeviceToDevice));
+        else layer2_weight->glorot(p.hidden_dim, p.output_dim, p.seed + 1, s);
         const int max_dim = p.hidden_dim > p.output_dim ? p.hidden_dim : p.output_dim;
         adj.reset(new Adjacency(N, nnz, rp, ci, in_degree, out_degree, max_dim, s));
         DRONE_GCN_HIP(hipMalloc(&truth, sizeof(int) * (size_t)N));

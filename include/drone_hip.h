@@ -101,7 +101,8 @@ typedef struct PRValues {
 
 /* DRONE/src/cuda/graph.h:45 / graph.cu:30-132.  u, v: host arrays of edgeSize global ids.
  * Local ids are handed out in first-seen order (u[i] then v[i]); rows keep input order.
- * Also builds the in-edge CSR on the device.  workerNum must be 1 in this build (one subgraph). */
+ * Also builds the in-edge CSR on the device.  workerId / workerNum describe the vertex cut this subgraph belongs to;
+ * the routing tables of its replicas are added with addMasterRoute / addMirrorRoute. */
 Graph *build_graph(int globalVertexSize, int edgeSize, int *u, int *v, int workerId, int workerNum,
                    Comm *comm);
 /* DRONE/src/cuda/graph.h:47-48 */
@@ -235,9 +236,13 @@ int drone_spmm_plan_create(drone_spmm_plan **plan, int n_rows, int n_cols, int64
  * makes the two factors).  v is still passed and still used by the band pieces and the short rows; the dense part is
  * then kept as one BIT per cell over a much larger region (any 4096-row x 2048-column chunk where it pays), and
  * multiplied on the matrix cores against col_scale .* B written as the exact sum of three bf16 numbers per element, with
- * fp32 accumulation; rows are scaled by row_scale when the result is added into C.  Creation checks every entry
- * against the scales (relative 4e-6) and every dense cell for holding one entry only; a matrix that fails either
- * check gets the plan drone_spmm_plan_create would have built.  drone_spmm_plan_update_values refuses a plan that
+ * fp32 accumulation; rows are scaled by row_scale when the result is added into C.  Inside the bit region the product
+ * therefore uses row_scale[row] * col_scale[col] IN PLACE OF v[e].  Creation checks every entry for
+ * |v[e] - row_scale[row] * col_scale[col]| <= 4e-6 * |row_scale[row] * col_scale[col]| (about 34 fp32 ulp: 1 / sqrtf(a * b)
+ * and (1 / sqrtf(a)) * (1 / sqrtf(b)) differ by a few ulp), so results inside the region can differ from a v-weighted
+ * product by that much, relative, per entry - well inside the 1e-4 the path is held to.  It also checks every dense
+ * cell for holding one entry only; a matrix that fails either check gets the plan drone_spmm_plan_create would have
+ * built.  drone_spmm_plan_update_values refuses a plan that
  * holds bits.  No counterpart in the reference: cusparseSpMM does not know the values' structure. */
 int drone_spmm_plan_create_scaled(drone_spmm_plan **plan, int n_rows, int n_cols, int64_t nnz, const int *rp,
                                   const int *ci, const float *v, const float *row_scale, const float *col_scale,
@@ -273,8 +278,11 @@ int64_t drone_sgemm_flops(int M, int N, int K);
  * library's code object holds on every GPU it runs on until the process ends, instead of the grow-only scratch.
  * Calls no hipMalloc / hipFree.  The array is sized for the worst case of the split rule (at most 512 work-groups
  * of 128 x 128 outputs); a product whose partial sums (splits * M * N floats) would exceed
- * drone_sgemm_noalloc_scratch_bytes() is refused with DRONE_ERR_INVALID and leaves C untouched.  All calls on one GPU share the array: calls that overlap on one GPU (different streams or
- * threads) race; order them on one stream or with events. */
+ * drone_sgemm_noalloc_scratch_bytes() is refused with DRONE_ERR_INVALID and leaves C untouched.  All calls on one GPU
+ * share the array: calls that overlap on one GPU (different streams or threads) race; order them on one stream or
+ * with events.  The array's device address is looked up once per device (hipGetSymbolAddress), by the first product
+ * that needs it or by drone_sgemm_noalloc_scratch_bytes(): call the latter with the device current BEFORE a stream
+ * capture begins, so that the calls inside the capture only launch kernels. */
 int drone_sgemm_rm_f32_noalloc(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,
                                const float *B, int ldb, float beta, float *C, int ldc, drone_stream_t stream);
 int64_t drone_sgemm_noalloc_scratch_bytes(void);
@@ -285,6 +293,10 @@ int drone_clear_mirror_rows_f32(float *grad, int ld, int rows, int K, const int 
 /* cuda_kernel.cu:384-392 / :394-399: in-place ReLU with a byte mask recorded when training. */
 int drone_relu_forward_f32(float *x, uint8_t *mask, int64_t n, int training, drone_stream_t stream);
 int drone_relu_backward_f32(float *grad, const uint8_t *mask, int64_t n, drone_stream_t stream);
+/* cuda_variable.cu:18-24 CUDAVariable::glorot (kernel cuda_kernel.cu:470-475): w[i] = (u - 0.5) * 2r with u uniform in
+ * (0, 1] and r = sqrtf(6 / (in_size + out_size)), for n consecutive floats on the device.  The reference's cuRAND
+ * stream (states seeded with 1234) is not reproduced: element i depends on (seed, i) only. */
+int drone_glorot_uniform_f32(float *w, int64_t n, int in_size, int out_size, uint64_t seed, drone_stream_t stream);
 /* cuda_kernel.cu:403-420 with the keep-mask explicit (the reference draws it from cuRAND states that
  * cannot be reproduced): keep[i] = u(seed, step, i) >= p, then x *= keep ? 1/(1-p) : 0 for both the
  * forward activations and the backward gradients. */
@@ -326,7 +338,9 @@ int drone_fill_f32(float *x, int64_t n, float value, drone_stream_t stream);
  * drone_gcn_modules.hpp.  The caller hands over device arrays (the reference's file parser is not part
  * of this path): out-edge CSR, global in/out degrees, features X (N x input_dim, leading dimension ldx,
  * borrowed for the handle's lifetime), labels, split ids (1 = train as in cuda_gcn.cu:289), and initial
- * weights W1 (input_dim x hidden) / W2 (hidden x output), which are copied.  Failures inside the module
+ * weights W1 (input_dim x hidden) / W2 (hidden x output), which are copied; a null W1 / W2 asks for the reference's
+ * own initialisation, glorot(input_dim, hidden) / glorot(hidden, output) (cuda_gcn.cu:42, :71), drawn from cfg->seed
+ * and cfg->seed + 1.  Failures inside the module
  * layer print and exit, as the reference does (cuda_kernel.cuh:11-18). */
 typedef struct drone_gcn drone_gcn;
 typedef struct drone_gcn_config {

@@ -354,6 +354,55 @@ def test_sgd_adam(T, oracle):
         np.testing.assert_allclose(wd.cpu().numpy(), wa, rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("in_size,out_size", [(602, 128), (128, 41), (1433, 64)])
+def test_glorot_uniform(T, in_size, out_size):
+    """CUDAVariable::glorot (cuda_variable.cu:18-24, kernel cuda_kernel.cu:470-475): (u - 0.5) * 2r with u in (0, 1] and
+    r = sqrtf(6 / (in + out)).  The cuRAND bit stream is not reproducible, the distribution is: support, mean,
+    variance r^2 / 3 and a Kolmogorov-Smirnov test against the uniform law; a seed fixes the values, seeds differ."""
+    from scipy import stats
+    from drone_amd import gcn
+    r = float(np.sqrt(np.float32(6.0) / np.float32(in_size + out_size)))
+    w = gcn.glorot_uniform(T.empty((in_size, out_size), device="cuda"), in_size, out_size, seed=1234).cpu().numpy()
+    assert w.dtype == np.float32 and w.min() > -r * (1 + 1e-6) and w.max() <= r * (1 + 1e-6)
+    n = w.size
+    assert abs(w.mean()) < 5 * r / np.sqrt(3 * n)                            # five standard errors of the mean
+    assert abs(w.var() / (r * r / 3) - 1) < 5 * np.sqrt(0.8 / n)             # var of u^2 on (-1, 1) is 4/45
+    assert stats.kstest(w.ravel().astype(np.float64), "uniform", args=(-r, 2 * r)).pvalue > 1e-3
+    # no structure along either axis: neighbouring weights are uncorrelated
+    assert abs(np.corrcoef(w[:, :-1].ravel(), w[:, 1:].ravel())[0, 1]) < 5 / np.sqrt(n)
+    assert abs(np.corrcoef(w[:-1].ravel(), w[1:].ravel())[0, 1]) < 5 / np.sqrt(n)
+    again = gcn.glorot_uniform(T.empty((in_size, out_size), device="cuda"), in_size, out_size, seed=1234).cpu().numpy()
+    other = gcn.glorot_uniform(T.empty((in_size, out_size), device="cuda"), in_size, out_size, seed=1235).cpu().numpy()
+    np.testing.assert_array_equal(w, again)
+    assert (w != other).mean() > 0.99
+
+
+def test_model_initialises_weights_with_glorot(T):
+    """A model made without initial weights draws them as CUDAGCN does (cuda_gcn.cu:42, :71): glorot(input, hidden) and
+    glorot(hidden, output), and trains from there."""
+    from drone_amd import gcn, graphs, rmat
+    g = graphs.gcn_graph_np(9, 8, seed=3)
+    n, fin, hid, cls = g["n"], 32, 16, 7
+    X = rmat.normal_f32((n, fin), seed=1)
+    label = rmat.randint_i32(n, seed=4, bound=cls)
+    split = np.ones(n, np.int32)
+    deg = dev(T, g["deg"])
+    m = gcn.GcnModel(dev(T, g["rp"]), dev(T, g["ci"]), deg, deg, dev(T, X), dev(T, label), dev(T, split), None, None,
+                     use_adam=False, mean_gradient=True, lr=0.05, hidden=hid, classes=cls, seed=77)
+    W1, W2 = m.tensor("W1"), m.tensor("W2")
+    for w, (a, b) in ((W1, (fin, hid)), (W2, (hid, cls))):
+        r = float(np.sqrt(np.float32(6.0) / np.float32(a + b)))
+        assert w.shape == (a, b) and np.abs(w).max() <= r * (1 + 1e-6) and w.std() > 0.4 * r
+    np.testing.assert_array_equal(W1, gcn.glorot_uniform(T.empty((fin, hid), device="cuda"), fin, hid, seed=77).cpu().numpy())
+    np.testing.assert_array_equal(W2, gcn.glorot_uniform(T.empty((hid, cls), device="cuda"), hid, cls, seed=78).cpu().numpy())
+    m.set_truth(1)
+    first = m.train_epoch()[0]
+    for _ in range(20):
+        last = m.train_epoch()[0]
+    assert np.isfinite(first) and last < first
+    m.close()
+
+
 def test_split_reductions_on_two_streams_do_not_share_scratch(T):
     """Two weight-gradient GEMMs and two cross-entropies issued back to back on different streams (so they may run
     at the same time) give the results of the serial calls."""
@@ -517,14 +566,44 @@ def test_spmm_scaled_plan_falls_back(T, oracle):
         plan.close()
 
 
-def _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, row_sums, dense=None, scales=None):
+@pytest.mark.parametrize("off,bits", [(2e-6, True), (8e-6, False)])
+def test_spmm_scaled_plan_value_tolerance(T, oracle, off, bits):
+    """A scaled plan is only built when every value lies within 4e-6 (relative) of row_scale * col_scale; the bit
+    region then multiplies by the scales in place of the values.  Values moved by 2e-6 are accepted (and the product
+    agrees with the v-weighted oracle far inside 1e-4), values moved by 8e-6 get the ordinary plan."""
+    from drone_amd import gcn
+    rng = np.random.default_rng(35)
+    n = 9000
+    rp, cols, in_deg, out_deg = _core_graph(rng, n, 5000, 0.7, 30000)
+    d_rp, d_ci = dev(T, rp), dev(T, cols)
+    d_val = gcn.edge_values(d_rp, d_ci, dev(T, in_deg), dev(T, out_deg))
+    r_scale, c_scale = gcn.degree_scales(dev(T, out_deg)), gcn.degree_scales(dev(T, in_deg))
+    sign = T.from_numpy(np.where(rng.random(d_val.numel()) < 0.5, -1.0, 1.0).astype(np.float32)).cuda()
+    exact = (r_scale[T.repeat_interleave(T.arange(n, device="cuda"), T.from_numpy(np.diff(rp).astype(np.int64)).cuda())] *
+             c_scale[d_ci.long()])
+    d_val = (exact * (1.0 + off * sign)).contiguous()          # every entry off by `off`, in either direction
+    plan = gcn.SpmmPlan(d_rp, d_ci, d_val, n, max_k=128, row_scale=r_scale, col_scale=c_scale)
+    assert (plan.bit_core()["cells"] > 0) == bits and plan.info()["dense_nnz"] > 0
+    val = d_val.cpu().numpy()
+    B = rng.uniform(-1, 1, (n, 128)).astype(np.float32)
+    want = oracle.spmm_f64acc(rp, cols, val, B).astype(np.float64)
+    scale = oracle.spmm_f64acc(rp, cols, np.abs(val), np.abs(B)).astype(np.float64)
+    got = gcn.spmm(plan, d_rp, d_ci, d_val, dev(T, B)).cpu().numpy()
+    assert rel_err(got, want, scale) <= (1e-5 if bits else 1e-4)
+    plan.close()
+
+
+def _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, row_sums, dense=None, scales=None, bits=None):
     """Size-independent checks of C = A * B at a benchmark shape: A * 1 against fp64 row sums, adjointness
     <A X, Y> = <X, A^T Y> with the separately built transpose, agreement with the vendor's sparse product on a
     column sample, and a repeatable result.  scales = (row_scale, col_scale) of A: the plans are then the scaled-pattern
-    plans the module layer builds (bits where the matrix is dense enough), with the factors swapped for A^T."""
+    plans the module layer builds (bits where the matrix is dense enough), with the factors swapped for A^T.
+    bits: whether those plans must hold a bit region (the benchmark times the products of plans that do)."""
     rs, cs = scales if scales is not None else (None, None)
     plan = gcn.SpmmPlan(rp, ci, val, N, max_k=K, row_scale=rs, col_scale=cs)
     planT = gcn.SpmmPlan(rpT, ciT, vT, N, max_k=K, row_scale=cs, col_scale=rs)
+    if bits is not None:
+        assert (plan.bit_core()["cells"] > 0) == bits and (planT.bit_core()["cells"] > 0) == bits
     if dense is not None:                      # whether the plans moved part of the matrix to a dense representation
         assert (plan.info()["dense_nnz"] > 0) == dense and (planT.info()["dense_nnz"] > 0) == dense
         assert (plan.bit_core()["cells"] > 0) == (dense and scales is not None)
@@ -544,7 +623,8 @@ def _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, row_
     assert torch.equal(gcn.spmm(plan, rp, ci, val, X), AX)          # fixed summation order
     # vendor sparse product in fp64 on four columns
     A64 = torch.sparse_csr_tensor(rp.long(), ci.long(), val.double(), size=(N, N))
-    cols = [0, 1, K // 2, K - 1]
+    from column_sample import sample_columns
+    cols = sample_columns(K, seed=K)
     ref = torch.sparse.mm(A64, X[:, cols].double().contiguous())
     err = (AX[:, cols].double() - ref).abs().max(dim=0).values / ref.abs().max(dim=0).values
     assert float(err.max()) <= 1e-4
@@ -576,7 +656,7 @@ def test_full_size_properties_config3(T):
     row_sums = cs[rp[1:].long()] - cs[rp[:-1].long()]
     _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, 128, row_sums)
     scale = gcn.degree_scales(deg)
-    _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, 128, row_sums, scales=(scale, scale))
+    _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, 128, row_sums, scales=(scale, scale), bits=True)
 
 
 @pytest.mark.parametrize("K", [16, 64, 256])
@@ -596,7 +676,8 @@ def test_full_size_properties_config5(T, K):
     rpT, ciT, vT = gcn.csr_transpose(N, N, rp, ci, val)
     assert int(rpT[-1]) == x["nnz"] and int((ciT[1:] < ciT[:-1]).sum()) <= N          # rows ascending inside
     _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, (cnt > 0).double(), dense=(K == 256))
-    if K != 16:                                                     # the same with the plans told that val = 1/count[row] * 1
-        inv = (1.0 / cnt.clamp(min=1).float()).contiguous()
-        _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, (cnt > 0).double(),
-                                   scales=(inv, torch.ones(N, device="cuda")))
+    # the same with the plans told that val = 1/count[row] * 1: at every width (16 included, where 16 of the 64 tile
+    # columns are live) these are the plans the benchmark times, and each of them holds a bit region
+    inv = (1.0 / cnt.clamp(min=1).float()).contiguous()
+    _spmm_full_size_properties(torch, gcn, N, rp, ci, val, rpT, ciT, vT, K, (cnt > 0).double(),
+                               scales=(inv, torch.ones(N, device="cuda")), bits=True)

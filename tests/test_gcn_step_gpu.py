@@ -259,9 +259,10 @@ def _spmm_checks_config4(torch, gcn, N, HID, CLS, rp, ci, val, A64, degree_scale
         again = torch.empty((N, ld), device="cuda")[:, :K]       # same leading dimension -> same lane layout
         gcn.spmm(plan, rp, ci, val, X, K=K, out=again)
         assert torch.equal(again, AX)                          # fixed summation order
-        # element-wise: the vendor's sparse product in fp64 on four columns, every element against its own sum of
+        # element-wise: the vendor's sparse product in fp64 on a column sample, every element against its own sum of
         # |a||b| (the values are positive, so that is A * |X|)
-        cols = [0, 1, K // 2, K - 1]
+        from column_sample import sample_columns
+        cols = sample_columns(K, seed=K + ld)                    # one column in every 32-wide matrix-core tile
         ref = torch.sparse.mm(A64, X[:, cols].double().contiguous())
         mag = torch.sparse.mm(A64, X[:, cols].double().abs().contiguous())
         assert float(((AX[:, cols].double() - ref).abs() / mag.clamp(min=1e-30)).max()) <= 1e-4
@@ -313,3 +314,72 @@ def test_full_size_properties_config4(T):
         m.close()
     assert np.isfinite(losses[0][0]) and abs(losses[0][0] - np.log(CLS)) < 0.5
     assert losses[0] == losses[1]
+
+
+@pytest.mark.parametrize("fold", [False, True])
+def test_full_size_step_config4_against_fp64(T, fold):
+    """The composed training step of the fourth configuration at full size, as the benchmark runs it (module list, and
+    with the first layer's aggregation folded): logits, hidden activations and both weight gradients against the same
+    step carried out in fp64 (the vendor's sparse product and matmul, this model's own dropout and ReLU masks), every
+    element within 1e-4 of its own scale - the step recomputed on absolute values, softmax derivative included - and
+    arg-max predictions equal to the fp64 ones except where the two largest fp64 logits of a row lie within 2e-4 of the
+    row's largest magnitude of each other (cuda_gcn.cu:226-246)."""
+    torch = T
+    from drone_amd import gcn, graphs, rmat
+    N, FIN, HID, CLS, p = 232965, 602, 128, 41, 0.5
+    g = graphs.gcn_graph_torch(18, 0, seed=4, n=N, n_edges=221_000_000)
+    rp, ci, deg = g["rp"], g["ci"], g["deg"]
+    val = gcn.edge_values(rp, ci, deg, deg)                     # symmetric graph: A^T = A
+    A = torch.sparse_csr_tensor(rp.long(), ci.long(), val.double(), size=(N, N))
+    Xf = torch.from_numpy(rmat.normal_f32((N, FIN), seed=4)).cuda()
+    W1 = torch.from_numpy(rmat.uniform_f32((FIN, HID), seed=41, lo=-0.09, hi=0.09)).cuda()
+    W2 = torch.from_numpy(rmat.uniform_f32((HID, CLS), seed=42, lo=-0.18, hi=0.18)).cuda()
+    label = torch.from_numpy(rmat.randint_i32(N, seed=43, bound=CLS)).cuda()
+    split = torch.from_numpy(np.where(rmat.uniform_f32(N, seed=44, lo=0, hi=1) < 0.66, 1, 2).astype(np.int32)).cuda()
+    m = gcn.GcnModel(rp, ci, deg, deg, Xf, label, split, W1.clone(), W2.clone(), dropout=p, lr=0.01, use_dropout=True,
+                     use_adam=False, mean_gradient=True, seed=4, fold_input_aggregation=fold)
+    m.set_truth(1)
+    m.train_step_async()                                        # forward + backward + SGD, as timed
+    m.read_metrics()
+    got = {k: torch.from_numpy(m.tensor(k)).cuda().double() for k in ("Z", "H1", "dW1", "dW2")}
+    keep = torch.from_numpy(m.tensor("keep1")).cuda().double() / (1.0 - p)
+    relu = torch.from_numpy(m.tensor("relu_mask")).cuda().double()
+    truth = torch.from_numpy(m.tensor("truth")).cuda().long()
+    m.close()
+    lab = truth >= 0
+    count = int(lab.sum())
+    assert 0.6 * N < count < 0.72 * N
+    X64, W1d, W2d = Xf.double(), W1.double(), W2.double()
+    gate = relu * keep
+    H1 = torch.sparse.mm(A, X64 @ W1d) * gate
+    Z = torch.sparse.mm(A, H1 @ W2d)
+    prob = torch.softmax(Z, dim=1)
+    dZ = prob.clone()
+    rows = torch.nonzero(lab).squeeze(1)
+    dZ[rows, truth[rows]] -= 1.0
+    dZ = dZ * lab[:, None] / count
+    dT2 = torch.sparse.mm(A, dZ)
+    dW2 = H1.T @ dT2
+    dT1 = torch.sparse.mm(A, (dT2 @ W2d.T) * gate)
+    dW1 = X64.T @ dT1
+    # scales: the same step on absolute values (no ReLU mask)
+    aX, aW1, aW2 = X64.abs(), W1d.abs(), W2d.abs()
+    sH1 = torch.sparse.mm(A, aX @ aW1) * keep
+    sZ = torch.sparse.mm(A, sH1 @ aW2)
+    sdZ = (dZ.abs() * count + prob * (sZ + (prob * sZ).sum(1, keepdim=True))) * lab[:, None] / count
+    sdT2 = torch.sparse.mm(A, sdZ)
+    sdT1 = torch.sparse.mm(A, (sdT2 @ aW2.T) * keep)
+    want = {"Z": (Z, sZ), "H1": (H1, sH1), "dW2": (dW2, sH1.T @ sdT2), "dW1": (dW1, aX.T @ sdT1)}
+    for name, (ref, scale) in want.items():
+        err = float(((got[name] - ref).abs() / scale.clamp(min=1e-30)).max())
+        assert err <= 1e-4, f"{name}: error {err:.3e} of the element's scale (fold={fold})"
+        top = float((got[name] - ref).abs().max() / ref.abs().max())
+        assert top <= 1e-4, f"{name}: error {top:.3e} of the tensor's maximum"
+    # predictions: equal to the fp64 arg-max wherever the fp64 winner leads by more than the tolerance, taken relative
+    # to the row's largest logit (not to the much larger sum of absolute values)
+    pred, pred64 = got["Z"].argmax(1), Z.argmax(1)
+    top2 = torch.topk(Z, 2, dim=1).values
+    clear = (top2[:, 0] - top2[:, 1]) > 2e-4 * Z.abs().max(dim=1).values
+    assert float(clear.double().mean()) > 0.99                  # the tie clause excuses next to nothing
+    assert bool((pred[clear] == pred64[clear]).all())
+    assert int((pred != pred64).sum()) <= int((~clear).sum())

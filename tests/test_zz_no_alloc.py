@@ -68,3 +68,26 @@ def test_noalloc_gemm_worst_case_fills_the_scratch_exactly(T):
     out = T.zeros((M, N), device="cuda")
     gcn.sgemm(1, 0, A, B, out=out, noalloc=True)
     assert float(out.min()) == K == float(out.max())
+
+
+def test_noalloc_gemm_leaves_free_device_memory_unchanged(T):
+    """The entry point's claim itself: with the operands in place and the array's address resolved
+    (drone_sgemm_noalloc_scratch_bytes), a split product of a shape no earlier call has seen takes no device memory,
+    while the allocating entry point grows its scratch for the same shape."""
+    from drone_amd import gcn
+    from drone_amd._lib import lib
+    M, N, K = 96, 80, 262_144 + 4096                      # 1 tile -> the reduction is split; a shape used nowhere else
+    A = T.rand((K, M), device="cuda")
+    B = T.rand((K, N), device="cuda")
+    out = T.empty((M, N), device="cuda")
+    want = T.empty((M, N), device="cuda")
+    assert lib().drone_sgemm_noalloc_scratch_bytes() > 0  # resolves the address for this device
+    T.cuda.synchronize()
+    free0 = T.cuda.mem_get_info()[0]
+    for _ in range(3):
+        gcn.sgemm(1, 0, A, B, out=out, noalloc=True)
+    T.cuda.synchronize()
+    assert T.cuda.mem_get_info()[0] == free0
+    gcn.sgemm(1, 0, A, B, out=want)                       # the allocating form on a fresh stream-scratch size
+    T.cuda.synchronize()
+    assert T.equal(out, want)
