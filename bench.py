@@ -30,6 +30,8 @@ def log(*a):
 
 PR_KERNELS = ("pr_rowblock_kernel<drone::PrF64Epi, 6>", "pr_rowblock_merge_kernel<drone::PrF64Epi>")  # the instance a plan of this size launches
 PR_TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "pr_rowblock_pagerank_c2.hbm_traffic.txt")
+SPMM_TRAFFIC_PROFILE_NAME = "profiles/spmm_gcn_layer_c3__spmm_sweep_c5.hbm_traffic.txt"
+SPMM_TRAFFIC_PROFILE = os.path.join(ROOT, *SPMM_TRAFFIC_PROFILE_NAME.split("/"))
 
 
 def pr_traffic_from_profile(path=PR_TRAFFIC_PROFILE):
@@ -125,14 +127,34 @@ def time_call(fn, reps, warmup=1):
     return t.stop_ms() / reps
 
 
-def spmm_report(name, n, nnz, K, ms):
+def spmm_traffic_from_profile(label, path=SPMM_TRAFFIC_PROFILE):
+    """Fabric bytes one product moves (all of its kernels), from the committed rocprofv3 counter summary: the line
+    `product <label> ... fetch_bytes F write_bytes W` (already scaled by the 1 GiB copy kernel of the same run).
+    None when the file is missing or has no such line."""
+    try:
+        for line in open(path):
+            w = line.split()
+            if len(w) > 2 and w[0] == "product" and w[1] == label and "fetch_bytes" in w and "write_bytes" in w:
+                return float(w[w.index("fetch_bytes") + 1]) + float(w[w.index("write_bytes") + 1])
+    except (OSError, ValueError):
+        pass
+    return None
+
+
+def spmm_report(name, n, nnz, K, ms, traffic_label=None):
     from drone_amd._lib import lib
     b = lib().drone_spmm_bytes(n, nnz, K)
     gbs = b / (ms * 1e-3) / 1e9
     gather = (8 * nnz + 4 * nnz * K + 4 * n * K) / (ms * 1e-3) / 1e9
-    return {"kernel": name, "K": K, "ms": ms, "algorithmic_bytes": b, "achieved_GBps": gbs,
-            "frac_of_hbm_peak": gbs / HBM_PEAK_GBS, "gather_inclusive_GBps": gather,
-            "gflops": 2.0 * nnz * K / (ms * 1e-3) / 1e9}
+    out = {"kernel": name, "K": K, "ms": ms, "algorithmic_bytes": b, "achieved_GBps": gbs,
+           "frac_of_hbm_peak": gbs / HBM_PEAK_GBS, "gather_inclusive_GBps": gather,
+           "gflops": 2.0 * nnz * K / (ms * 1e-3) / 1e9}
+    if traffic_label:
+        t = spmm_traffic_from_profile(traffic_label)
+        out["traffic"] = t          # rocprofv3 FETCH_SIZE + WRITE_SIZE per product, None if not profiled
+        out["traffic_over_algorithmic"] = t / b if t else None
+        out["traffic_source"] = SPMM_TRAFFIC_PROFILE_NAME
+    return out
 
 
 def bench_gcn_step(steps, warmup, cpu_baseline=False):
@@ -287,13 +309,14 @@ def bench_gcn_layer(cpu_baseline=False):
     log(f"GCN layer (configs[2]): {ms:.2f} ms, SpMM {ms_spmm:.2f} ms, GEMM {ms_gemm:.2f} ms" +
         (f"; CPU SpMM {cpu['value']:.0f} ms on {cpu['cores']} threads" if cpu else ""))
     return {"workload": f"GCN layer forward (configs[2]): R-MAT scale 20 undirected + self-loops, N={N}, nnz={nnz}, K=128",
-            "layer_ms": ms, "spmm": spmm_report("spmm (rows + band pieces + bit core) K=128", N, nnz, K, ms_spmm),
+            "layer_ms": ms, "spmm": spmm_report("spmm (rows + band pieces + bit core) K=128", N, nnz, K, ms_spmm,
+                                                traffic_label="c3_K128"),
             "spmm_plan": plan_info,
             "gemm_ms": ms_gemm, "gemm_tflops": 2.0 * N * K * K / (ms_gemm * 1e-3) / 1e12,
             "gemm_frac_of_fp32_mfma_peak": 2.0 * N * K * K / (ms_gemm * 1e-3) / 1e12 / 157.3, "cpu_baseline_spmm": cpu}
 
 
-def bench_spmm_sweep(cpu_baseline=False):
+def bench_spmm_sweep(cpu_baseline=False, widths=(16, 64, 256)):
     """configs[4]: skew-stress SpMM sweep, R-MAT scale 22 ef 32 a/b/c = .70/.12/.12, row-normalised, K in 16/64/256,
     forward (A*H) and transpose (A^T*G)."""
     import torch
@@ -308,7 +331,7 @@ def bench_spmm_sweep(cpu_baseline=False):
     inv_deg, ones = (1.0 / deg.float()).contiguous(), torch.ones(N, device="cuda")   # val = inv_deg[row] * 1
     out = {"workload": f"SpMM sweep (configs[4]): R-MAT scale 22 ef 32 skewed, N={N}, nnz={nnz}, max row "
                        f"{int((rp[1:]-rp[:-1]).max())}, max transposed row {int((rpT[1:]-rpT[:-1]).max())}", "kernels": []}
-    for K in (16, 64, 256):
+    for K in widths:
         H = torch.rand((N, K), device="cuda") * 2 - 1
         C_ = torch.empty((N, K), device="cuda")
         for name, (a, b, c, rs, cs) in (("forward A*H", (rp, ci, val, inv_deg, ones)),
@@ -317,11 +340,11 @@ def bench_spmm_sweep(cpu_baseline=False):
             ms = time_call(lambda: gcn.spmm(plan, a, b, c, H, out=C_), reps=5)
             info = dict(plan.info(), bit_core=plan.bit_core())
             plan.close()
-            out["kernels"].append(dict(spmm_report(f"{name} K={K}", N, nnz, K, ms), plan=info))
+            out["kernels"].append(dict(spmm_report(f"{name} K={K}", N, nnz, K, ms, traffic_label=f"c5_K{K}"), plan=info))
             log(f"SpMM sweep (configs[4]) {name} K={K}: {ms:.2f} ms = {out['kernels'][-1]['frac_of_hbm_peak']*100:.1f} % of "
                 f"the HBM roofline")
         del H, C_
-    if cpu_baseline:
+    if cpu_baseline and 64 in widths:
         out["cpu_baseline_spmm"] = cpu_spmm_baseline(rp, ci, val, N, 64, nnz)
         out["cpu_baseline_spmm"]["gpu_ms"] = [k["ms"] for k in out["kernels"] if k["K"] == 64][0]
         log(f"cpu baseline SpMM K=64 forward: {out['cpu_baseline_spmm']['value']:.0f} ms")
@@ -508,10 +531,11 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="launch the 1 GiB stream-copy kernel exactly once (a dispatch of known traffic to scale "
                          "rocprofv3 byte counters by)")
-    ap.add_argument("--suite", default="default", choices=["pr", "default", "full", "gcn", "sweep", "traverse", "exchange"],
+    ap.add_argument("--widths", default="16,64,256", help="feature widths of --suite sweep (a profiling run takes one)")
+    ap.add_argument("--suite", default="default", choices=["pr", "default", "full", "gcn", "layer", "sweep", "traverse", "exchange"],
                     help="pr: PageRank only (fp64 pull plan, then the reference's PR_PEVal / PR_IncEVal on the same "
                          "graph); default (= full): + the GCN training step (configs[3]), the GCN layer (configs[2]), "
-                         "the SpMM sweep (configs[4]), the SSSP / CC jobs and the replica exchange; gcn, sweep, "
+                         "the SpMM sweep (configs[4]), the SSSP / CC jobs and the replica exchange; gcn, layer, sweep, "
                          "traverse, exchange: that part alone")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -535,13 +559,17 @@ def main():
     del a, b
     torch.cuda.empty_cache()
 
-    if args.suite in ("gcn", "sweep", "traverse", "exchange"):      # profiling helpers: one part alone, no headline line
+    if args.suite in ("gcn", "layer", "sweep", "traverse", "exchange"):      # profiling helpers: one part alone, no headline line
         if args.suite == "exchange":
             part = bench_exchange()
         elif args.suite == "traverse":
             part = bench_traverse(cpu_baseline=not args.no_cpu_baseline)
+        elif args.suite == "layer":
+            part = bench_gcn_layer()
+        elif args.suite == "sweep":
+            part = bench_spmm_sweep(widths=tuple(int(k) for k in args.widths.split(",")))
         else:
-            part = bench_gcn_step(steps=max(3, args.steps), warmup=max(1, args.warmup)) if args.suite == "gcn" else bench_spmm_sweep()
+            part = bench_gcn_step(steps=max(3, args.steps), warmup=max(1, args.warmup))
         print(json.dumps(part), flush=True)
         return
 

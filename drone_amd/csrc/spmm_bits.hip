@@ -380,12 +380,15 @@ int bit_core_products(const BitCore *bc, const unsigned *col_order, const float 
         const int width = std::min(K - pass * 128, 128);
         const uint4 *split = bc->split + (size_t)pass * groups * kGroupVecs;
         float *partial = bc->partial + (size_t)pass * bc->num_units * kBitTileRows * kPartialLd;
-        if (width <= 64)
-            bits_mfma_kernel<2><<<bc->num_units, 512, 0, s>>>(bc->unit_tile, bc->unit_c0, bc->unit_c1, bc->unit_slot,
-                                                             bc->tile_blocks, bc->tile_off, bc->bits, split, partial);
-        else
-            bits_mfma_kernel<4><<<bc->num_units, 512, 0, s>>>(bc->unit_tile, bc->unit_c0, bc->unit_c1, bc->unit_slot,
-                                                             bc->tile_blocks, bc->tile_off, bc->bits, split, partial);
+        // as many 32-column feature tiles as the pass holds (the plan's cost model prices the cells per such tile)
+        const auto launch = [&](auto kernel) {
+            kernel<<<bc->num_units, 512, 0, s>>>(bc->unit_tile, bc->unit_c0, bc->unit_c1, bc->unit_slot, bc->tile_blocks,
+                                                 bc->tile_off, bc->bits, split, partial);
+        };
+        if (width <= 32) launch(bits_mfma_kernel<1>);
+        else if (width <= 64) launch(bits_mfma_kernel<2>);
+        else if (width <= 96) launch(bits_mfma_kernel<3>);
+        else launch(bits_mfma_kernel<4>);
     }
     DRONE_HIP_TRY(hipGetLastError());
     return DRONE_OK;
