@@ -218,18 +218,177 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             }
 }
 
-// C = alpha * sum_z partial[z] + beta * C, z ascending
-__global__ void sgemm_reduce_kernel(int M, int N, int splits, const float *__restrict__ partial, float alpha,
-                                    float beta, float *__restrict__ C, int ldc)
+// Weight gradients with a small output: C(M x N) = A^T * B with M <= 128, N <= 64 and a reduction over hundreds of
+// thousands of rows (H1^T * dT2 of the 2-layer model: 128 x 41 over 232,965 vertices).  The whole output is eight
+// 32 x 32 accumulators, so ONE wavefront holds it, and with A stored K x M and B stored K x N both operands of
+// v_mfma_f32_32x32x2_f32 come straight from rows of the inputs: no LDS staging, no loader wavefronts, every wavefront
+// streams its own share of the reduction into registers, kSkinnyDepth k-pairs ahead.  A lane reads FOUR consecutive
+// floats of A's row and TWO of B's with one load each (lane r of a half-wavefront: columns 4r .. 4r + 3 and 2r, 2r + 1),
+// and its four / two values go to the four / two tiles: tile i holds the output rows 4r + i, tile j the output columns
+// 2r + j - a renumbering that only the epilogue sees.  (With one dword per lane and tile, six loads per k-pair instead
+// of two, the address unit spends 16 clocks per 256 bytes and the same product took 57 us instead of the figure below;
+// splitting the output rows over the wavefronts instead of the reduction - 32 registers of accumulators, 16 k-pairs in
+// flight - reads B four times and took 70 us.)  The four wavefronts of a work-group add their tiles in wavefront order
+// through LDS; the work-groups' tiles go to the split scratch and are summed in a fixed order by sgemm_reduce_kernel
+// (bitwise repeatable).  Through the tiled kernel the same product ran at 23 TFLOP/s: 227 work-groups with one
+// 128 x 64 tile each, every one paying the LDS pipeline's fill and drain for 1,024 reduction steps.
+#ifndef DRONE_SKINNY_DEPTH
+#define DRONE_SKINNY_DEPTH 4
+#endif
+#ifndef DRONE_SKINNY_SPLITS
+#define DRONE_SKINNY_SPLITS 512
+#endif
+constexpr int kSkinnyDepth = DRONE_SKINNY_DEPTH;   // k-pairs fetched per step and wavefront
+constexpr int kSkinnyWaves = 4;
+struct alignas(4) Float2U {
+    float v[2];
+};
+__global__ __launch_bounds__(kSkinnyWaves * kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void sgemm_tn_skinny_kernel(
+    int M, int N, int K, const float *__restrict__ A, int lda, const float *__restrict__ B, int ldb, int k_chunk,
+    float *__restrict__ partial)
 {
+    constexpr int TM = 4, TN = 2;
+    __shared__ float s_tile[128 * 64];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int lr = lane & 31, lk = lane >> 5;
+    const int kb = blockIdx.x * k_chunk;
+    const int ke = kb + k_chunk < K ? kb + k_chunk : K;
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+    // Every load is unconditional: a lane outside the output reads a valid place of the row (the caller guarantees
+    // lda >= M rounded up to 4 and ldb >= N rounded up to 2) and the bits it gets are masked to zero.  (A load whose
+    // value is only selected under a per-lane condition is sunk into a branch of its own by the compiler; the mask keeps
+    // it needed on every path and cannot turn a stray NaN into one.)  Rows are addressed as a wavefront-uniform base plus
+    // a 32-bit lane offset in bytes, the form that costs one register per load.
+    unsigned keep_m[TM], keep_n[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) keep_m[i] = 4 * lr + i < M ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) keep_n[j] = 2 * lr + j < N ? 0xFFFFFFFFu : 0u;
+    const unsigned lane_a = 4u * (unsigned)(lk * lda + (4 * lr < M ? 4 * lr : 0));
+    const unsigned lane_b = 4u * (unsigned)(lk * ldb + (2 * lr < N ? 2 * lr : 0));
+    const int step = 2 * kSkinnyWaves * kSkinnyDepth;
+    const int ke_pairs = kb + ((ke - kb) & ~1);  // whole k-pairs end here; an odd last row is added after the loop
+    // Two register sets with fixed names take turns (a set chosen by a run-time index would live in scratch memory).
+    float a0[kSkinnyDepth][TM], b0[kSkinnyDepth][TN], a1[kSkinnyDepth][TM], b1[kSkinnyDepth][TN];
+    const auto fetch = [&](float (&a)[kSkinnyDepth][TM], float (&b)[kSkinnyDepth][TN], int k_first) {
+        const int k0 = __builtin_amdgcn_readfirstlane(k_first);
+#pragma unroll
+        for (int u = 0; u < kSkinnyDepth; ++u) {
+            const int k = k0 + 2 * kSkinnyWaves * u;               // the pair's first row: uniform
+            const bool live = k < ke_pairs;
+            const unsigned keep_k = live ? 0xFFFFFFFFu : 0u;       // a pair past the end reads rows kb, kb + 1: zeros
+            const char *ra = reinterpret_cast<const char *>(A + (size_t)(live ? k : kb) * lda);
+            const char *rb = reinterpret_cast<const char *>(B + (size_t)(live ? k : kb) * ldb);
+            const Float4U qa = *reinterpret_cast<const Float4U *>(ra + lane_a);
+            const Float2U qb = *reinterpret_cast<const Float2U *>(rb + lane_b);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) a[u][i] = __uint_as_float(__float_as_uint(qa.v[i]) & keep_m[i] & keep_k);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) b[u][j] = __uint_as_float(__float_as_uint(qb.v[j]) & keep_n[j] & keep_k);
+        }
+    };
+    const auto multiply = [&](const float (&a)[kSkinnyDepth][TM], const float (&b)[kSkinnyDepth][TN]) {
+#pragma unroll
+        for (int u = 0; u < kSkinnyDepth; ++u)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u][i], b[u][j], acc[i][j], 0, 0, 0);
+    };
+    int k0 = kb + 2 * wave;
+    if (k0 < ke_pairs) {  // the same for the whole wavefront
+        fetch(a0, b0, k0);
+        for (;;) {
+            fetch(a1, b1, k0 + step);
+            multiply(a0, b0);
+            k0 += step;
+            if (k0 >= ke_pairs) break;
+            fetch(a0, b0, k0 + step);
+            multiply(a1, b1);
+            k0 += step;
+            if (k0 >= ke_pairs) break;
+        }
+    }
+    if (wave == 0 && ke_pairs < ke) {  // the odd last row of the range: a pair whose second row is zero
+        const unsigned keep_k = lk == 0 ? 0xFFFFFFFFu : 0u;
+        const Float4U qa = *reinterpret_cast<const Float4U *>(A + (size_t)ke_pairs * lda + (4 * lr < M ? 4 * lr : 0));
+        const Float2U qb = *reinterpret_cast<const Float2U *>(B + (size_t)ke_pairs * ldb + (2 * lr < N ? 2 * lr : 0));
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(__float_as_uint(qa.v[i]) & keep_m[i] & keep_k),
+                                                                 __uint_as_float(__float_as_uint(qb.v[j]) & keep_n[j] & keep_k),
+                                                                 acc[i][j], 0, 0, 0);
+    }
+    // The wavefronts' tiles, added in wavefront order.  Register v of lane l of tile (i, j) is row 8*(v/4) + 4*(l/32) +
+    // v%4 and column l%32 of the tile, i.e. output row 4 * that row + i and output column 2 * (l%32) + j.
+    for (int w = 0; w < kSkinnyWaves; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int row = 4 * (8 * (v / 4) + 4 * lk + (v % 4)) + i, col = 2 * lr + j;
+                        float *cell = s_tile + row * 64 + col;
+                        *cell = w == 0 ? acc[i][j][v] : *cell + acc[i][j][v];
+                    }
+        }
+        __syncthreads();
+    }
+    float *out = partial + (size_t)blockIdx.x * M * N;
+    for (int idx = threadIdx.x; idx < M * N; idx += kSkinnyWaves * kWave) {
+        const int row = idx / N, col = idx - row * N;
+        out[idx] = s_tile[row * 64 + col];
+    }
+}
+
+// C = alpha * sum_z partial[z] + beta * C.  A work-group of 256 lanes owns 32 consecutive outputs; lane (o, g) adds the
+// partials z = g, g + 8, ... of output o (eight independent loads in flight), and the eight sums of an output are added
+// in g order - a fixed order, so the result is repeatable.  (One lane per output adding all the splits in turn took
+// 31 ... 108 us for 227 ... 512 splits of a few thousand outputs: a chain of dependent round trips on a few dozen CUs.)
+constexpr int kReduceOutputs = 32, kReduceGroups = 8;
+__global__ __launch_bounds__(kReduceOutputs * kReduceGroups) void sgemm_reduce_kernel(
+    int M, int N, int splits, const float *__restrict__ partial, float alpha, float beta, float *__restrict__ C, int ldc)
+{
+    __shared__ float s_sum[kReduceGroups][kReduceOutputs];
     const int64_t total = (int64_t)M * N;
-    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+    const int o = threadIdx.x % kReduceOutputs, g = threadIdx.x / kReduceOutputs;
+    for (int64_t base = (int64_t)blockIdx.x * kReduceOutputs; base < total; base += (int64_t)gridDim.x * kReduceOutputs) {
+        const int64_t idx = base + o;
         float s = 0.0f;
-        for (int z = 0; z < splits; ++z) s += partial[(size_t)z * total + idx];
-        const int row = (int)(idx / N), col = (int)(idx % N);
-        float r = alpha * s;
-        if (beta != 0.0f) r += beta * C[(size_t)row * ldc + col];
-        C[(size_t)row * ldc + col] = r;
+        if (idx < total) {
+            int z = g;
+            for (; z + 7 * kReduceGroups < splits; z += 8 * kReduceGroups) {
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[u] = partial[(size_t)(z + u * kReduceGroups) * total + idx];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) s += v[u];
+            }
+            for (; z < splits; z += kReduceGroups) s += partial[(size_t)z * total + idx];
+        }
+        s_sum[g][o] = s;
+        __syncthreads();
+        if (g == 0 && idx < total) {
+            float sum = s_sum[0][o];
+#pragma unroll
+            for (int k = 1; k < kReduceGroups; ++k) sum += s_sum[k][o];
+            const int row = (int)(idx / N), col = (int)(idx % N);
+            float r = alpha * sum;
+            if (beta != 0.0f) r += beta * C[(size_t)row * ldc + col];
+            C[(size_t)row * ldc + col] = r;
+        }
+        __syncthreads();
     }
 }
 
@@ -304,6 +463,48 @@ int static_scratch(float **out)
     return DRONE_OK;
 }
 
+void launch_reduce(int M, int N, int splits, const float *partial, float alpha, float beta, float *C, int ldc, hipStream_t s)
+{
+    int blocks = (int)ceil_div((int64_t)M * N, kReduceOutputs);
+    if (blocks > 8192) blocks = 8192;
+    sgemm_reduce_kernel<<<blocks, kReduceOutputs * kReduceGroups, 0, s>>>(M, N, splits, partial, alpha, beta, C, ldc);
+}
+
+// Scratch for `floats` partial sums: the stream's grow-only buffer, or the fixed array of the entry point that may not
+// allocate.
+int split_scratch(bool may_allocate, size_t floats, hipStream_t s, int M, int N, int K, int splits, float **partial)
+{
+    if (may_allocate) return workspace(sizeof(float) * floats, s, partial);
+    if (floats > kStaticScratchFloats) {
+        set_error(DRONE_ERR_INVALID,
+                  "drone_sgemm_rm_f32_noalloc: %d x %d x %d splits the reduction %d ways and needs %zu bytes of "
+                  "partial sums, the fixed scratch holds %zu; use drone_sgemm_rm_f32",
+                  M, N, K, splits, floats * sizeof(float), kStaticScratchFloats * sizeof(float));
+        return DRONE_ERR_INVALID;
+    }
+    return static_scratch(partial);
+}
+
+// C = alpha * A^T * B + beta * C for a small output and a long reduction (see sgemm_tn_skinny_kernel).
+int sgemm_tn_skinny(bool may_allocate, int M, int N, int K, float alpha, const float *A, int lda, const float *B, int ldb,
+                    float beta, float *C, int ldc, hipStream_t s)
+{
+    // two work-groups of four wavefronts per CU, each wavefront at least 16 steps of the reduction deep
+    int splits = DRONE_SKINNY_SPLITS;
+    const int deepest = (int)ceil_div(K, 2 * kSkinnyWaves * kSkinnyDepth * 16);
+    if (splits > deepest) splits = deepest;
+    if (splits < 1) splits = 1;
+    int k_chunk = (int)ceil_div(ceil_div(K, splits), 2 * kSkinnyWaves) * 2 * kSkinnyWaves;
+    splits = (int)ceil_div(K, k_chunk);
+    float *partial = nullptr;
+    const int rc = split_scratch(may_allocate, (size_t)splits * M * N, s, M, N, K, splits, &partial);
+    if (rc != DRONE_OK) return rc;
+    sgemm_tn_skinny_kernel<<<splits, kSkinnyWaves * kWave, 0, s>>>(M, N, K, A, lda, B, ldb, k_chunk, partial);
+    launch_reduce(M, N, splits, partial, alpha, beta, C, ldc, s);
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
 int sgemm_entry(bool may_allocate, int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,
                 const float *B, int ldb, float beta, float *C, int ldc, drone_stream_t stream)
 {
@@ -314,6 +515,9 @@ int sgemm_entry(bool may_allocate, int transA, int transB, int M, int N, int K, 
     if (M == 0 || N == 0) return DRONE_OK;
     DRONE_REQUIRE(C != nullptr && (K == 0 || (A && B)), "null operand");
     hipStream_t s = as_stream(stream);
+    // (the skinny kernel's lanes read four floats of A's row and two of B's at once, also the lanes past M and N)
+    if (transA && !transB && M <= 128 && N <= 64 && K >= 8192 && lda >= (M + 3) / 4 * 4 && ldb >= (N + 1) / 2 * 2)
+        return sgemm_tn_skinny(may_allocate, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, s);
     const bool narrow = N <= 64;
     const int bn = narrow ? 64 : 128;
     const int tiles = (int)(ceil_div(M, BM) * ceil_div(N, bn));
@@ -336,30 +540,14 @@ int sgemm_entry(bool may_allocate, int transA, int transB, int M, int N, int K, 
     if (splits > 1) {
         // every (tile, split) work-group stores its whole tile, so the partials need no clearing
         const size_t floats = (size_t)splits * M * N;
-        if (may_allocate) {
-            int rc = workspace(sizeof(float) * floats, s, &partial);
-            if (rc != DRONE_OK) return rc;
-        } else {
-            if (floats > kStaticScratchFloats) {
-                set_error(DRONE_ERR_INVALID,
-                          "drone_sgemm_rm_f32_noalloc: %d x %d x %d splits the reduction %d ways and needs %zu bytes of "
-                          "partial sums, the fixed scratch holds %zu; use drone_sgemm_rm_f32",
-                          M, N, K, splits, floats * sizeof(float), kStaticScratchFloats * sizeof(float));
-                return DRONE_ERR_INVALID;
-            }
-            int rc = static_scratch(&partial);
-            if (rc != DRONE_OK) return rc;
-        }
+        const int rc = split_scratch(may_allocate, floats, s, M, N, K, splits, &partial);
+        if (rc != DRONE_OK) return rc;
     }
     dim3 grid((unsigned)ceil_div(N, bn), (unsigned)ceil_div(M, BM), (unsigned)splits);
     DRONE_REQUIRE(grid.y <= 65535u * 32u, "M too large for the launch grid");
     if (narrow) launch<64>(transA != 0, transB != 0, grid, s, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
     else launch<128>(transA != 0, transB != 0, grid, s, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
-    if (splits > 1) {
-        int blocks = (int)ceil_div((int64_t)M * N, 256);
-        if (blocks > 4096) blocks = 4096;
-        sgemm_reduce_kernel<<<blocks, 256, 0, s>>>(M, N, splits, partial, alpha, beta, C, ldc);
-    }
+    if (splits > 1) launch_reduce(M, N, splits, partial, alpha, beta, C, ldc, s);
     DRONE_HIP_TRY(hipGetLastError());
     return DRONE_OK;
 }

@@ -217,6 +217,32 @@ def test_sgemm_against_oracle(T, oracle, tA, tB, M, N, K):
         np.testing.assert_allclose(got, oracle.sgemm_f32(0, 0, A, B), rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("M,N,K", [(128, 41, 20001), (100, 64, 9000), (33, 7, 8192), (1, 1, 10000), (128, 64, 65537),
+                                   (97, 33, 8193), (64, 64, 8200)])
+@pytest.mark.parametrize("pad", [0, 5])
+def test_sgemm_small_output_long_reduction(T, M, N, K, pad):
+    """C = A^T * B with at most 128 x 64 outputs and a reduction of 8,192 steps or more takes the register-only kernel
+    (one wavefront holds the whole output; operands stream straight from memory): odd reduction lengths, outputs that
+    do not fill the 32 x 32 tiles, padded leading dimensions, alpha / beta, and a repeatable result."""
+    from drone_amd import gcn
+    rng = np.random.default_rng(M + 3 * N + K + pad)
+    A = rng.uniform(-1, 1, (K, M + pad)).astype(np.float32)
+    B = rng.uniform(-1, 1, (K, N + pad)).astype(np.float32)
+    C0 = rng.uniform(-1, 1, (M, N + pad)).astype(np.float32)
+    dA, dB = dev(T, A)[:, :M], dev(T, B)[:, :N]
+    out = dev(T, C0)
+    gcn.sgemm(1, 0, dA, dB, out=out[:, :N], alpha=0.75, beta=-0.5)
+    got = out.cpu().numpy()
+    opA, opB = A[:, :M].T.astype(np.float64), B[:, :N].astype(np.float64)
+    want = 0.75 * (opA @ opB) - 0.5 * C0[:, :N]
+    scale = 0.75 * (np.abs(opA) @ np.abs(opB)) + 0.5 * np.abs(C0[:, :N])
+    assert rel_err(got[:, :N], want, scale) <= 1e-4
+    np.testing.assert_array_equal(got[:, N:], C0[:, N:])             # padding columns untouched
+    again = dev(T, C0)
+    gcn.sgemm(1, 0, dA, dB, out=again[:, :N], alpha=0.75, beta=-0.5)
+    assert T.equal(again, out)
+
+
 def test_sgemm_identity_alpha_beta_ld_and_split_reduction(T):
     from drone_amd import gcn
     rng = np.random.default_rng(3)
