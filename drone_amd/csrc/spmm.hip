@@ -400,9 +400,20 @@ __global__ void spmm_combine_kernel(int num_long, const int *__restrict__ long_r
     const int i = blockIdx.x;
     if (i >= num_long) return;
     const int r = long_row[i];
+    const int s0 = first_slot[i], s1 = first_slot[i + 1];
     for (int k = threadIdx.x; k < K; k += blockDim.x) {
+        // eight loads in flight, added in slot order (one load at a time made a row a chain of a dozen round trips:
+        // 0.12 ... 0.20 ms per product on the 232,965-vertex graph for 0.34 GB of partial rows)
         float s = 0.0f;
-        for (int slot = first_slot[i]; slot < first_slot[i + 1]; ++slot) s += partial[(size_t)slot * ldp + k];
+        int slot = s0;
+        for (; slot + 8 <= s1; slot += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = partial[(size_t)(slot + u) * ldp + k];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += v[u];
+        }
+        for (; slot < s1; ++slot) s += partial[(size_t)slot * ldp + k];
         float out = alpha * s;
         if (beta != 0.0f) out += beta * C[(size_t)r * ldc + k];
         C[(size_t)r * ldc + k] = out;

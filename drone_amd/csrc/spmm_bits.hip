@@ -257,9 +257,18 @@ __global__ __launch_bounds__(256) void bits_combine_kernel(int rows, const int *
         const float scale = alpha * row_scale[row];
         for (int k = lane; k < K; k += kWave) {
             const float *src = partial + ((size_t)(k / 128) * num_units * kBitTileRows + rr % kBitTileRows) * kPartialLd + k % 128;
+            const float before = C[(size_t)row * ldc + k];  // in flight with the tile sums
             float sum = 0.0f;
-            for (int u = u0; u < u1; ++u) sum += src[(size_t)u * kBitTileRows * kPartialLd];
-            C[(size_t)row * ldc + k] += scale * sum;
+            int u = u0;
+            for (; u + 4 <= u1; u += 4) {                   // four loads in flight, added in unit order
+                float v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = src[(size_t)(u + j) * kBitTileRows * kPartialLd];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) sum += v[j];
+            }
+            for (; u < u1; ++u) sum += src[(size_t)u * kBitTileRows * kPartialLd];
+            C[(size_t)row * ldc + k] = before + scale * sum;
         }
     }
 }
