@@ -221,8 +221,10 @@ extern "C" int drone_gcn_tensor(struct drone_gcn *h, const char *name, void **pt
     for (const Entry &e : table)
         if (strcmp(e.name, name) == 0 && e.v != nullptr) {
             *ptr = e.grad ? e.v->grad : e.v->data;
-            if (rows) *rows = e.v->rows;
-            if (cols) *cols = e.v->cols;
+            // layer 1's inner dimension is padded inside the model: report the logical extent
+            const bool inner_is_cols = e.v == m->input || e.v == m->aggregated_input, inner_is_rows = e.v == m->layer1_weight;
+            if (rows) *rows = inner_is_rows ? m->params.input_dim : e.v->rows;
+            if (cols) *cols = inner_is_cols ? m->params.input_dim : e.v->cols;
             if (ld) *ld = e.v->ld;
             return DRONE_OK;
         }

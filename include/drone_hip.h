@@ -337,7 +337,9 @@ int drone_fill_f32(float *x, int64_t n, float value, drone_stream_t stream);
  * epoch loop of gcn.cu:96-106 / cuda_gcn.cu:287-318,356-379) over the C++ module layer in
  * drone_gcn_modules.hpp.  The caller hands over device arrays (the reference's file parser is not part
  * of this path): out-edge CSR, global in/out degrees, features X (N x input_dim, leading dimension ldx,
- * borrowed for the handle's lifetime), labels, split ids (1 = train as in cuda_gcn.cu:289), and initial
+ * borrowed for the handle's lifetime; when input_dim is not a multiple of 128 - or of 32, whichever adds at most an
+ * eighth - or ldx is not a multiple of 4, the model works on its own zero-padded copy of X made at creation, N x the
+ * rounded width, so that layer 1's two products see whole aligned tiles: later changes to X are then not seen), labels, split ids (1 = train as in cuda_gcn.cu:289), and initial
  * weights W1 (input_dim x hidden) / W2 (hidden x output), which are copied; a null W1 / W2 asks for the reference's
  * own initialisation, glorot(input_dim, hidden) / glorot(hidden, output) (cuda_gcn.cu:42, :71), drawn from cfg->seed
  * and cfg->seed + 1.  Failures inside the module
