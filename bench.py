@@ -230,16 +230,38 @@ def bench_gcn_step(steps, warmup, cpu_baseline=False):
     plain.close()
     spmm_ms = 2 * sum(k["ms"] for k in kernels[:2])
     spmm_bytes = 2 * sum(k["algorithmic_bytes"] for k in kernels[:2])
+    # The five dense products of the step, launched as the model launches them: activations at the module layer's row
+    # pitch (16-float multiples: 48 for the 41-column tensors), layer 1's inner dimension padded on the model's copy of
+    # X (602 -> 640 columns; the forward product runs over 608 of them); flops are counted on the logical shapes.
+    pitch = lambda c: (c + 15) // 16 * 16
+    FINP = FIN
+    for unit in (128, 32):
+        if (FIN + unit - 1) // unit * unit - FIN <= FIN // 8:
+            FINP = (FIN + unit - 1) // unit * unit
+            break
+    FINF = min(FINP, (FIN + 31) // 32 * 32)
+    Xp = torch.zeros((N, FINP), device="cuda")
+    Xp[:, :FIN] = X
+    W1p = torch.zeros((FINP, HID), device="cuda")
+    W1p[:FIN] = W1
+    H1 = torch.rand((N, pitch(HID)), device="cuda")[:, :HID]
+    dT1 = torch.rand((N, pitch(HID)), device="cuda")[:, :HID]
+    dT2 = torch.rand((N, pitch(CLS)), device="cuda")[:, :CLS]
+    T1 = torch.empty((N, pitch(HID)), device="cuda")[:, :HID]
+    T2 = torch.empty((N, pitch(CLS)), device="cuda")[:, :CLS]
+    dW1p, dW2 = torch.empty((FINP, HID), device="cuda"), torch.empty((HID, CLS), device="cuda")
     gemms = []
-    for (tA, tB, M, Nn, Kk, what) in ((0, 0, N, HID, FIN, "X*W1"), (0, 0, N, CLS, HID, "H1*W2"), (0, 1, N, HID, CLS, "dT2*W2^T"),
-                                      (1, 0, HID, CLS, N, "H1^T*dT2"), (1, 0, FIN, HID, N, "X^T*dT1")):
-        A = torch.rand((Kk, M) if tA else (M, Kk), device="cuda")
-        Bm = torch.rand((Nn, Kk) if tB else (Kk, Nn), device="cuda")
-        out = torch.empty((M, Nn), device="cuda")
-        ms = time_call(lambda: gcn.sgemm(tA, tB, A, Bm, out=out), reps=5)
+    for what, (M, Nn, Kk), call in (
+            ("X*W1", (N, HID, FIN), lambda: gcn.sgemm(0, 0, Xp, W1p, out=T1, K=FINF)),
+            ("H1*W2", (N, CLS, HID), lambda: gcn.sgemm(0, 0, H1, W2, out=T2)),
+            ("dT2*W2^T", (N, HID, CLS), lambda: gcn.sgemm(0, 1, dT2, W2, out=T1)),
+            ("H1^T*dT2", (HID, CLS, N), lambda: gcn.sgemm(1, 0, H1, dT2, out=dW2)),
+            ("X^T*dT1", (FIN, HID, N), lambda: gcn.sgemm(1, 0, Xp, dT1, out=dW1p))):
+        ms = time_call(call, reps=5)
         fl = 2.0 * M * Nn * Kk
         gemms.append({"gemm": what, "M": M, "N": Nn, "K": Kk, "ms": ms, "tflops": fl / (ms * 1e-3) / 1e12,
                       "frac_of_fp32_mfma_peak": fl / (ms * 1e-3) / 1e12 / 157.3})
+    del Xp, W1p, H1, dT1, dT2, T1, T2
     # CPU baseline: the oracle's CSR SpMM of identical semantics (OpenMP, all host cores) on the same matrix, K=128
     cpu = None
     if cpu_baseline:
