@@ -392,6 +392,146 @@ __global__ __launch_bounds__(kReduceOutputs * kReduceGroups) void sgemm_reduce_k
     }
 }
 
+// C (M x N) = alpha * A (M x K) * op(B) + beta * C for a tall A with short rows (K <= 128) and a small op(B)
+// (N <= 128): the layer products H * W and dZ * W^T of the model, 700 bytes of A and C per row for 10 K multiply-adds.
+// A wavefront owns a run of consecutive rows and takes them 16 at a time: it fetches the 16 rows with whole-line loads
+// (consecutive lanes, consecutive 16-byte pieces of a row), parks them in its own strip of LDS, and reads them back in
+// the layout v_mfma_f32_16x16x4_f32 wants (lane = row + 16 kk holds k = 16 q + 4 kk + j in component j of its q-th
+// 16-byte read; a row pitch of K + 4 floats keeps these reads free of bank conflicts).  The next 16 rows are in flight
+// in registers meanwhile, op(B) sits in LDS in the order the lanes read it, and the 16 x N result goes through the
+// strip once more so that it leaves in 16-byte pieces of consecutive lanes.  A strip belongs to one wavefront, whose
+// LDS accesses execute in order, so the loop has no barrier.  Values of A past K are replaced by zeros, whatever the
+// padding of the rows holds.
+// Measured on 232,965 rows (us; the general kernel / this one): 128 -> 41 columns 65 / 40, 41 -> 128 columns 74 / 37
+// (the matrix instructions and LDS traffic alone take 30, the loads alone 19, the stores alone 20 - 25).
+// What did not work: loading the operand layout straight from memory, every lane its own row, costs a cache lookup
+// per lane (64 per instruction): 19 us for the 119 MB of H even when all of it hits L1, 48 - 56 us in all; storing the
+// accumulators as they lie (64-byte pieces of four rows per instruction) 41 / 46.
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+constexpr int kTallWaves = 12, kTallRows = 16, kTallGroups = 256;
+template <int KQ, int NT, bool TB>
+__global__ __launch_bounds__(kTallWaves * kWave) void sgemm_tall_kernel(int M, int N, int K, float alpha,
+                                                                        const float *__restrict__ A, int lda,
+                                                                        const float *__restrict__ B, int ldb, float beta,
+                                                                        float *__restrict__ C, int ldc)
+{
+    constexpr int KP = 16 * KQ, PITCH = KP + 4, PIECES = KP / 4;  // a row of A in the strip
+    constexpr int CP = 16 * NT + 4, CPIECES = 4 * NT;              // a row of C in the strip
+    constexpr int kStrip = kTallRows * (PITCH > CP ? PITCH : CP) / 4;
+    __shared__ floatx4 s_b[KQ * NT * kWave];
+    __shared__ floatx4 s_strip[kTallWaves][kStrip];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int lr = lane & 15, kk = lane >> 4;
+    // the 16-row steps of the matrix are dealt out evenly: wavefront w of W takes steps [w S / W, (w + 1) S / W)
+    const int64_t all_steps = ((int64_t)M + kTallRows - 1) / kTallRows, waves = (int64_t)gridDim.x * kTallWaves;
+    const int64_t w = (int64_t)blockIdx.x * kTallWaves + wave;
+    const int step0 = (int)(w * all_steps / waves), steps = (int)((w + 1) * all_steps / waves) - step0;
+    float *mine = reinterpret_cast<float *>(s_strip[wave]);
+    // load c of a step: this lane's piece is 16-byte piece number 64 c + lane of the 16 rows
+    int piece_row[KQ], piece_k[KQ];
+#pragma unroll
+    for (int c = 0; c < KQ; ++c) {
+        piece_row[c] = (kWave * c + lane) / PIECES;
+        piece_k[c] = 4 * ((kWave * c + lane) % PIECES);
+    }
+    // store c of a step: 16-byte piece number 64 c + lane of the 16 rows of C
+    int out_row[NT], out_col[NT];
+#pragma unroll
+    for (int c = 0; c < NT; ++c) {
+        out_row[c] = (kWave * c + lane) / CPIECES;
+        out_col[c] = 4 * ((kWave * c + lane) % CPIECES);
+    }
+    floatx4 pre[KQ];
+    auto fetch = [&](int step) {
+#pragma unroll
+        for (int c = 0; c < KQ; ++c) {
+            int row = (step0 + step) * kTallRows + piece_row[c];
+            row = row < M ? row : M - 1;
+            pre[c] = *reinterpret_cast<const floatx4 *>(A + (size_t)row * lda + piece_k[c]);
+        }
+    };
+    if (steps > 0) fetch(0);  // in flight while op(B) is staged
+    // op(B)(k, n) with k = 16 q + 4 kk + j, n = 16 tile + lr  ->  s_b[(q NT + tile) 64 + 16 kk + lr][j]
+    for (int e = threadIdx.x; e < KQ * NT * kWave; e += kTallWaves * kWave) {
+        const int l = e % kWave, tile = (e / kWave) % NT, q = e / (kWave * NT);
+        const int n = 16 * tile + (l & 15), k0 = 16 * q + 4 * (l >> 4);
+        floatx4 v;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int k = k0 + j;
+            v[j] = (k < K && n < N) ? (TB ? B[(size_t)n * ldb + k] : B[(size_t)k * ldb + n]) : 0.0f;
+        }
+        s_b[e] = v;
+    }
+    __syncthreads();
+    for (int step = 0; step < steps; ++step) {
+#pragma unroll
+        for (int c = 0; c < KQ; ++c) {
+            floatx4 v = pre[c];
+            if (KP != K) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = piece_k[c] + j < K ? v[j] : 0.0f;
+            }
+            *reinterpret_cast<floatx4 *>(mine + piece_row[c] * PITCH + piece_k[c]) = v;
+        }
+        if (step + 1 < steps) fetch(step + 1);
+        floatx4 acc[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+        // the wavefronts that have matrix instructions to issue go first: those fetching or storing wait anyway
+        __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+        for (int q = 0; q < KQ; ++q) {
+            const floatx4 a = *reinterpret_cast<const floatx4 *>(mine + lr * PITCH + 16 * q + 4 * kk);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const floatx4 b = s_b[(q * NT + t) * kWave + lane];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j], b[j], acc[t], 0, 0, 0);
+            }
+        }
+        __builtin_amdgcn_s_setprio(0);
+        // Through the strip again, so that C is written in whole 16-byte pieces of consecutive lanes: the lane holds
+        // C(row = 4 kk + i, column = lr) of every 16 x 16 tile.
+        const int row_base = (step0 + step) * kTallRows;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) mine[(4 * kk + i) * CP + 16 * t + lr] = alpha * acc[t][i];
+        floatx4 out[NT];
+#pragma unroll
+        for (int c = 0; c < NT; ++c) out[c] = *reinterpret_cast<const floatx4 *>(mine + out_row[c] * CP + out_col[c]);
+        if (beta != 0.0f) {
+#pragma unroll
+            for (int c = 0; c < NT; ++c) {
+                const int row = row_base + out_row[c];
+                if (row >= M) continue;
+                const float *old = C + (size_t)row * ldc + out_col[c];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (out_col[c] + j < N) out[c][j] += beta * old[j];
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < NT; ++c) {
+            const int row = row_base + out_row[c];
+            if (row < M && out_col[c] + 4 <= N) *reinterpret_cast<floatx4 *>(C + (size_t)row * ldc + out_col[c]) = out[c];
+        }
+        if (N % 4 != 0) {
+#pragma unroll
+            for (int c = 0; c < NT; ++c) {
+                const int row = row_base + out_row[c];
+                if (row < M && out_col[c] < N && out_col[c] + 4 > N) {
+                    float *dst = C + (size_t)row * ldc + out_col[c];
+#pragma unroll
+                    for (int j = 0; j < 3; ++j)
+                        if (out_col[c] + j < N) dst[j] = out[c][j];
+                }
+            }
+        }
+    }
+}
+
 // Grow-only scratch for split-K partials, one per (device, stream): calls on one stream are ordered, so they can
 // share a buffer; calls on different streams may overlap and get their own.
 struct SplitScratch {
@@ -505,6 +645,42 @@ int sgemm_tn_skinny(bool may_allocate, int M, int N, int K, float alpha, const f
     return DRONE_OK;
 }
 
+// C = alpha * A * op(B) + beta * C for a tall A with rows of at most 128 values (see sgemm_tall_kernel); false when no
+// instance of the kernel covers the shape.
+template <int KQ, int NT, bool TB>
+void launch_tall(int M, int N, int K, float alpha, const float *A, int lda, const float *B, int ldb, float beta, float *C,
+                 int ldc, hipStream_t s)
+{
+    // one work-group per CU, as many as there are 16-row steps for every wavefront
+    const int64_t all_steps = ceil_div(M, kTallRows);
+    const unsigned grid = (unsigned)std::min<int64_t>(kTallGroups, ceil_div(all_steps, kTallWaves));
+    sgemm_tall_kernel<KQ, NT, TB><<<grid, kTallWaves * kWave, 0, s>>>(M, N, K, alpha, A, lda, B, ldb, beta, C, ldc);
+}
+bool sgemm_tall(int transB, int M, int N, int K, float alpha, const float *A, int lda, const float *B, int ldb, float beta,
+                float *C, int ldc, hipStream_t s)
+{
+    const int kq = (K + 15) / 16, nt = N <= 48 ? 3 : N <= 64 ? 4 : 8;
+    // the lanes read whole 16-byte pieces of A's rows up to column 16 kq, and write C's rows in 16-byte pieces
+    if (M < 8192 || K < 1 || N > 128 || lda < 16 * kq || lda % 4 != 0 || (reinterpret_cast<uintptr_t>(A) & 15) != 0 ||
+        ldc % 4 != 0 || (reinterpret_cast<uintptr_t>(C) & 15) != 0)
+        return false;
+#define DRONE_TALL(KQ_, NT_, TB_)                                                            \
+    if (kq == KQ_ && nt == NT_ && (transB != 0) == TB_) {                                    \
+        launch_tall<KQ_, NT_, TB_>(M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, s);         \
+        return true;                                                                         \
+    }
+    DRONE_TALL(8, 3, false)
+    DRONE_TALL(8, 4, false)
+    DRONE_TALL(4, 3, false)
+    DRONE_TALL(4, 4, false)
+    DRONE_TALL(3, 8, true)
+    DRONE_TALL(4, 8, true)
+    DRONE_TALL(3, 4, true)
+    DRONE_TALL(4, 4, true)
+#undef DRONE_TALL
+    return false;
+}
+
 int sgemm_entry(bool may_allocate, int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,
                 const float *B, int ldb, float beta, float *C, int ldc, drone_stream_t stream)
 {
@@ -518,6 +694,10 @@ int sgemm_entry(bool may_allocate, int transA, int transB, int M, int N, int K, 
     // (the skinny kernel's lanes read four floats of A's row and two of B's at once, also the lanes past M and N)
     if (transA && !transB && M <= 128 && N <= 64 && K >= 8192 && lda >= (M + 3) / 4 * 4 && ldb >= (N + 1) / 2 * 2)
         return sgemm_tn_skinny(may_allocate, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, s);
+    if (!transA && K <= 128 && sgemm_tall(transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, s)) {
+        DRONE_HIP_TRY(hipGetLastError());
+        return DRONE_OK;
+    }
     const bool narrow = N <= 64;
     const int bn = narrow ? 64 : 128;
     const int tiles = (int)(ceil_div(M, BM) * ceil_div(N, bn));

@@ -243,6 +243,46 @@ def test_sgemm_small_output_long_reduction(T, M, N, K, pad):
     assert T.equal(again, out)
 
 
+@pytest.mark.parametrize("tB,M,N,K", [(0, 20011, 41, 128), (0, 8192, 48, 120), (0, 9001, 64, 128), (0, 8200, 50, 113),
+                                      (0, 12345, 41, 64), (0, 8193, 33, 49), (0, 10000, 64, 60), (0, 8207, 1, 128),
+                                      (1, 20011, 128, 41), (1, 8192, 100, 33), (1, 9001, 128, 64), (1, 8200, 64, 48),
+                                      (1, 12345, 60, 50), (1, 8193, 65, 1)])
+@pytest.mark.parametrize("beta", [0.0, -0.5])
+def test_sgemm_tall_short_rows(T, tB, M, N, K, beta):
+    """C = A * op(B) for at least 8,192 rows of at most 128 values and at most 128 output columns takes the kernel that
+    streams A through per-wavefront LDS strips (the layer products H * W and dZ * W^T): every instance of it, row counts
+    that do not fill the 16-row steps, reductions that do not fill the 16-value pieces (A's padding holds NaN, which
+    must not reach the result), outputs that do not fill the 16-byte pieces (C's padding must stay), alpha / beta
+    (with beta = 0 C starts as NaN), a repeatable result, and agreement with the general kernel (unaligned A)."""
+    from drone_amd import gcn
+    rng = np.random.default_rng(M + 3 * N + K + tB)
+    lda, ldc = (K + 15) // 16 * 16 + 4, (N + 3) // 4 * 4 + 4
+    A = np.full((M, lda), np.nan, dtype=np.float32)
+    A[:, :K] = rng.uniform(-1, 1, (M, K))
+    B = rng.uniform(-1, 1, (N, K) if tB else (K, N)).astype(np.float32)
+    C0 = rng.uniform(-1, 1, (M, ldc)).astype(np.float32)
+    start = C0.copy()
+    if beta == 0.0:
+        start[:, :N] = np.nan
+    dA, dB, out = dev(T, A)[:, :K], dev(T, B), dev(T, start)
+    gcn.sgemm(0, tB, dA, dB, out=out[:, :N], alpha=0.75, beta=beta)
+    got = out.cpu().numpy()
+    opA, opB = A[:, :K].astype(np.float64), (B.T if tB else B).astype(np.float64)
+    want = 0.75 * (opA @ opB) + beta * C0[:, :N]
+    scale = 0.75 * (np.abs(opA) @ np.abs(opB)) + abs(beta) * np.abs(C0[:, :N])
+    assert rel_err(got[:, :N], want, scale) <= 1e-4
+    np.testing.assert_array_equal(got[:, N:], C0[:, N:])             # padding columns untouched
+    again = dev(T, start)
+    gcn.sgemm(0, tB, dA, dB, out=again[:, :N], alpha=0.75, beta=beta)
+    assert T.equal(again[:, :N], out[:, :N])
+    # the same product through the general kernel: A one float off the 16-byte grid
+    shifted = T.empty((M * lda + 1,), dtype=T.float32, device="cuda")[1:].view(M, lda)
+    shifted.copy_(dev(T, A))
+    other = dev(T, start)
+    gcn.sgemm(0, tB, shifted[:, :K], dB, out=other[:, :N], alpha=0.75, beta=beta)
+    assert rel_err(other.cpu().numpy()[:, :N], want, scale) <= 1e-4
+
+
 def test_sgemm_identity_alpha_beta_ld_and_split_reduction(T):
     from drone_amd import gcn
     rng = np.random.default_rng(3)
