@@ -377,11 +377,14 @@ def test_relu_dropout_in_one_pass(T, oracle, shape):
     np.testing.assert_array_equal(gb.cpu().numpy(), oracle.relu_backward(oracle.dropout_forward(g, kb.cpu().numpy(), 0.4), m))
 
 
-@pytest.mark.parametrize("classes,ld_pad", [(41, 0), (41, 3), (7, 0), (3, 1), (100, 0)])
+@pytest.mark.parametrize("classes,ld_pad", [(41, 0), (41, 3), (7, 0), (3, 1), (100, 0), (1, 0), (16, 1), (20, 0), (64, 0),
+                                            (65, 2), (129, 0), (256, 0), (300, 1)])
 def test_cross_entropy_accuracy_argmax(T, oracle, classes, ld_pad):
+    """Every lanes-per-row instance of the two kernels (4 ... 64 lanes, a lane holding up to four classes in registers), the
+    64-lane instance's loop over more than 256 classes, and row counts that do not fill the last group of rows."""
     from drone_amd import gcn
     rng = np.random.default_rng(classes)
-    n = 3000
+    n = 3000 + classes % 7
     z = (rng.normal(size=(n, classes)) * 3).astype(np.float32)
     z[5] = 1.0                                                      # a fully tied row
     truth = rng.integers(0, classes, n).astype(np.int32)
