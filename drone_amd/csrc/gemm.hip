@@ -408,13 +408,20 @@ __global__ __launch_bounds__(kReduceOutputs * kReduceGroups) void sgemm_reduce_k
 // per lane (64 per instruction): 19 us for the 119 MB of H even when all of it hits L1, 48 - 56 us in all; storing the
 // accumulators as they lie (64-byte pieces of four rows per instruction) 41 / 46.
 typedef float floatx4 __attribute__((ext_vector_type(4)));
-constexpr int kTallWaves = 12, kTallRows = 16, kTallGroups = 256;
+constexpr int kTallRows = 16, kTallGroups = 256;
+// Wavefronts per work-group: 12 where op(B) and 12 strips fit the 160 KB of LDS, else 8.
+constexpr int tall_waves(int kq, int nt)
+{
+    const int pitch = 16 * kq + 4, cp = 16 * nt + 4;
+    return kq * nt * 1024 + 12 * kTallRows * (pitch > cp ? pitch : cp) * 4 <= 160 * 1024 ? 12 : 8;
+}
 template <int KQ, int NT, bool TB>
-__global__ __launch_bounds__(kTallWaves * kWave) void sgemm_tall_kernel(int M, int N, int K, float alpha,
+__global__ __launch_bounds__(tall_waves(KQ, NT) * kWave) void sgemm_tall_kernel(int M, int N, int K, float alpha,
                                                                         const float *__restrict__ A, int lda,
                                                                         const float *__restrict__ B, int ldb, float beta,
                                                                         float *__restrict__ C, int ldc)
 {
+    constexpr int kTallWaves = tall_waves(KQ, NT);
     constexpr int KP = 16 * KQ, PITCH = KP + 4, PIECES = KP / 4;  // a row of A in the strip
     constexpr int CP = 16 * NT + 4, CPIECES = 4 * NT;              // a row of C in the strip
     constexpr int kStrip = kTallRows * (PITCH > CP ? PITCH : CP) / 4;
@@ -653,6 +660,7 @@ void launch_tall(int M, int N, int K, float alpha, const float *A, int lda, cons
 {
     // one work-group per CU, as many as there are 16-row steps for every wavefront
     const int64_t all_steps = ceil_div(M, kTallRows);
+    constexpr int kTallWaves = tall_waves(KQ, NT);
     const unsigned grid = (unsigned)std::min<int64_t>(kTallGroups, ceil_div(all_steps, kTallWaves));
     sgemm_tall_kernel<KQ, NT, TB><<<grid, kTallWaves * kWave, 0, s>>>(M, N, K, alpha, A, lda, B, ldb, beta, C, ldc);
 }
@@ -673,6 +681,10 @@ bool sgemm_tall(int transB, int M, int N, int K, float alpha, const float *A, in
     DRONE_TALL(8, 4, false)
     DRONE_TALL(4, 3, false)
     DRONE_TALL(4, 4, false)
+    DRONE_TALL(8, 8, false)
+    DRONE_TALL(4, 8, false)
+    DRONE_TALL(8, 8, true)
+    DRONE_TALL(8, 4, true)
     DRONE_TALL(3, 8, true)
     DRONE_TALL(4, 8, true)
     DRONE_TALL(3, 4, true)

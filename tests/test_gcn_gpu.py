@@ -246,7 +246,8 @@ def test_sgemm_small_output_long_reduction(T, M, N, K, pad):
 @pytest.mark.parametrize("tB,M,N,K", [(0, 20011, 41, 128), (0, 8192, 48, 120), (0, 9001, 64, 128), (0, 8200, 50, 113),
                                       (0, 12345, 41, 64), (0, 8193, 33, 49), (0, 10000, 64, 60), (0, 8207, 1, 128),
                                       (1, 20011, 128, 41), (1, 8192, 100, 33), (1, 9001, 128, 64), (1, 8200, 64, 48),
-                                      (1, 12345, 60, 50), (1, 8193, 65, 1)])
+                                      (1, 12345, 60, 50), (1, 8193, 65, 1), (0, 9001, 128, 128), (0, 8200, 100, 64),
+                                      (1, 8200, 128, 128), (1, 9001, 64, 120)])
 @pytest.mark.parametrize("beta", [0.0, -0.5])
 def test_sgemm_tall_short_rows(T, tB, M, N, K, beta):
     """C = A * op(B) for at least 8,192 rows of at most 128 values and at most 128 output columns takes the kernel that
