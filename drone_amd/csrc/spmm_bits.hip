@@ -243,6 +243,125 @@ __global__ __launch_bounds__(512, 1) void bits_mfma_kernel(const int *__restrict
             }
 }
 
+// The same product for at most 48 feature columns, on 16-row x 16-column tiles (v_mfma_f32_16x16x32_bf16): 41 columns
+// fill three 16-wide tiles, where the 32-wide tiles of bits_mfma_kernel<2> multiply 64.  A wavefront still owns 64 rows
+// (four row tiles) and all CT feature tiles.  The bits stay in the layout above; the instruction wants lane
+// r + 16 q to hold row r's columns 32 s + 8 q .. + 8 of step s, and that byte sits in lane (r + 16 p) + 32 (q & 1),
+// byte 2 s + (q >> 1), of the 32-row group that holds row tile 2 i + p - so sixteen ds_bpermute per 256-column block
+// (one per group, p and dword) regroup them, against 288 matrix instructions.  A stage is 64 ranked columns (two
+// steps): 8 groups x 3 parts x 16 CT features, fetched and handed over exactly as in bits_mfma_kernel.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+template <int CT>
+__global__ __launch_bounds__(512, 1) void bits_mfma16_kernel(const int *__restrict__ unit_tile,
+                                                             const int *__restrict__ unit_c0,
+                                                             const int *__restrict__ unit_c1,
+                                                             const int *__restrict__ unit_slot,
+                                                             const int *__restrict__ tile_blocks,
+                                                             const int64_t *__restrict__ tile_off,
+                                                             const uint4 *__restrict__ bits,
+                                                             const uint4 *__restrict__ split, float *__restrict__ partial)
+{
+    constexpr int kF = 16 * CT, kStageGroups = 8, kStageVecs = kStageGroups * 3 * kF;
+    constexpr int kPre = (kStageVecs + 511) / 512;
+    __shared__ uint4 s_b[2][kStageVecs];
+    const int u = blockIdx.x, tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int tile = unit_tile[u], c0 = unit_c0[u], c1 = unit_c1[u];
+    const int blocks = tile_blocks[tile], nblocks = (c1 - c0) / kBitBlockCols;
+    const uint4 *w0 = bits + tile_off[tile] + ((size_t)(2 * wave) * blocks + c0 / kBitBlockCols) * 64 + lane;
+    const size_t wstep = (size_t)blocks * 64;
+    const uint4 *src = split + (size_t)(c0 / 8) * kGroupVecs;
+    int goff[kPre];  // every lane loads in every slot, see bits_mfma_kernel
+#pragma unroll
+    for (int i = 0; i < kPre; ++i) {
+        const int v = tid + 512 * i < kStageVecs ? tid + 512 * i : kStageVecs - 1;
+        const int g = v / (3 * kF), rem = v % (3 * kF);
+        goff[i] = g * kGroupVecs + (rem / kF) * 4 * 32 + rem % kF;
+    }
+    f32x4 acc[4][CT];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < CT; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    const int r16 = lane & 15, kq = lane >> 4;
+    const int pull[2] = {4 * (r16 + 32 * (kq & 1)), 4 * (16 + r16 + 32 * (kq & 1))};
+    const int shift = 8 * (kq >> 1);
+
+    u32x4 pre[kPre];
+    const int rot = (tile * 5) % nblocks;
+    uint4 a[2], an[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) a[i] = w0[i * wstep + (size_t)rot * 64];
+    {
+        const uint4 *first = src + (size_t)rot * 32 * kGroupVecs;
+#pragma unroll
+        for (int i = 0; i < kPre; ++i) pre[i] = __builtin_bit_cast(u32x4, first[goff[i]]);
+#pragma unroll
+        for (int i = 0; i < kPre; ++i)
+            if (tid + 512 * i < kStageVecs) s_b[0][tid + 512 * i] = __builtin_bit_cast(uint4, pre[i]);
+    }
+    __syncthreads();
+    for (int kb = 0; kb < nblocks; ++kb) {
+        const int block = kb + rot < nblocks ? kb + rot : kb + rot - nblocks;
+        const int block_next = block + 1 < nblocks ? block + 1 : 0;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) an[i] = w0[i * wstep + (size_t)block_next * 64];
+        unsigned aw[2][2][4];  // [32-row group][row tile of the group][dword]: this lane's bytes in the 16-row layout
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const unsigned word[4] = {a[i].x, a[i].y, a[i].z, a[i].w};
+#pragma unroll
+            for (int p = 0; p < 2; ++p)
+#pragma unroll
+                for (int w = 0; w < 4; ++w) aw[i][p][w] = (unsigned)__builtin_amdgcn_ds_bpermute(pull[p], (int)word[w]);
+        }
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            const bool more = kb + 1 < nblocks || st < 3;
+            {
+                const uint4 *next = src + (size_t)(!more ? block * 4 + st : st < 3 ? block * 4 + st + 1 : block_next * 4) * kStageGroups * kGroupVecs;
+#pragma unroll
+                for (int i = 0; i < kPre; ++i)
+                    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(pre[i]) : "v"(next + goff[i]) : "memory");
+            }
+            const uint4 *cur = s_b[st & 1];
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                bf16x8 A[4];
+#pragma unroll
+                for (int rt = 0; rt < 4; ++rt) A[rt] = expand_bits((aw[rt / 2][rt % 2][st] >> (16 * ks + shift)) & 0xFFu);
+#pragma unroll
+                for (int part = 0; part < 3; ++part)
+#pragma unroll
+                    for (int ct = 0; ct < CT; ++ct) {
+                        const uint4 raw = cur[((4 * ks + kq) * 3 + part) * kF + 16 * ct + r16];
+                        const bf16x8 bv = __builtin_bit_cast(bf16x8, raw);
+#pragma unroll
+                        for (int rt = 0; rt < 4; ++rt)
+                            acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[rt], bv, acc[rt][ct], 0, 0, 0);
+                    }
+            }
+            staged_loads_landed(pre);
+            if (more) {
+#pragma unroll
+                for (int i = 0; i < kPre; ++i)
+                    if (tid + 512 * i < kStageVecs) s_b[(st & 1) ^ 1][tid + 512 * i] = __builtin_bit_cast(uint4, pre[i]);
+            }
+            __syncthreads();
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) a[i] = an[i];
+    }
+    // 16 x 16 accumulator layout: register v of lane l holds row 4 (l / 16) + v, column l % 16
+    float *out = partial + (size_t)unit_slot[u] * kBitTileRows * kPartialLd;
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                out[(size_t)(64 * wave + 16 * rt + 4 * kq + v) * kPartialLd + 16 * ct + r16] = acc[rt][ct][v];
+}
+
 // One wavefront per ranked row: adds the units' tile sums of the row, scales and adds into C.
 __global__ __launch_bounds__(256) void bits_combine_kernel(int rows, const int *__restrict__ tile_unit0,
                                                            const float *__restrict__ partial, int num_units, int passes,
@@ -394,7 +513,9 @@ int bit_core_products(const BitCore *bc, const unsigned *col_order, const float 
             kernel<<<bc->num_units, 512, 0, s>>>(bc->unit_tile, bc->unit_c0, bc->unit_c1, bc->unit_slot, bc->tile_blocks,
                                                  bc->tile_off, bc->bits, split, partial);
         };
-        if (width <= 32) launch(bits_mfma_kernel<1>);
+        if (width <= 16) launch(bits_mfma16_kernel<1>);
+        else if (width <= 32) launch(bits_mfma_kernel<1>);
+        else if (width <= 48) launch(bits_mfma16_kernel<3>);
         else if (width <= 64) launch(bits_mfma_kernel<2>);
         else if (width <= 96) launch(bits_mfma_kernel<3>);
         else launch(bits_mfma_kernel<4>);
