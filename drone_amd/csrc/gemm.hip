@@ -30,6 +30,7 @@ namespace drone {
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int BM = 128;
 constexpr int BK = 32;
@@ -352,6 +353,142 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) __attribute__((amdgpu_waves_p
     }
 }
 
+// The same product on 16 x 16 tiles (v_mfma_f32_16x16x4_f32) for outputs of at most 128 x 16 NT: 41 columns fill three
+// 16-wide tiles where the 32-wide tiles above multiply 64.  Lane m + 16 q of a wavefront reads, from row k + q of a
+// group of four rows, four consecutive floats of A at columns 4 m and 64 + 4 m (the eight tiles along M: tile (h, i)
+// holds the output rows 64 h + 4 m + i) and NT consecutive floats of B at column NT m (tile j: output columns
+// NT m + j) - three loads per four rows and 8 NT matrix instructions.  Loads are unconditional and masked, rows are
+// addressed as a wavefront-uniform base plus a 32-bit lane offset, two register sets of kSmallDepth groups take turns,
+// and the four wavefronts add their tiles in wavefront order through LDS, all as in sgemm_tn_skinny_kernel.
+template <int W> struct alignas(4) FloatNU {
+    float v[W];
+};
+// One group of four rows per fetch: deeper steps (2 / 3 / 4 groups) measured 50 / 68 / 66 us against 47 for the 128 x 41
+// gradient over 232,965 rows (a wavefront's share of a work-group's 455 rows is then cut into coarser steps, and the
+// matrix instructions of a long step leave the next step's loads less time to land).
+constexpr int kSmallDepth = 1, kSmallWaves = 4;
+template <int NT>
+__global__ __launch_bounds__(kSmallWaves * kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void sgemm_tn_small_kernel(
+    int M, int N, int K, const float *__restrict__ A, int lda, const float *__restrict__ B, int ldb, int k_chunk,
+    float *__restrict__ partial)
+{
+    constexpr int CP = 16 * NT;
+    __shared__ float s_tile[2 * 128 * CP];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int lm = lane & 15, lk = lane >> 4;
+    const int kb = blockIdx.x * k_chunk;
+    const int ke = kb + k_chunk < K ? kb + k_chunk : K;
+    floatx4 acc[2][4][NT];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j) acc[h][i][j] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    unsigned keep_m[2][4], keep_n[NT];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) keep_m[h][i] = 64 * h + 4 * lm + i < M ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) keep_n[j] = NT * lm + j < N ? 0xFFFFFFFFu : 0u;
+    unsigned lane_a[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) lane_a[h] = 4u * (unsigned)(lk * lda + (64 * h + 4 * lm < M ? 64 * h + 4 * lm : 0));
+    const unsigned lane_b = 4u * (unsigned)(lk * ldb + (NT * lm < N ? NT * lm : 0));
+    const int step = 4 * kSmallWaves * kSmallDepth;
+    const int ke_groups = kb + ((ke - kb) & ~3);  // whole groups of four rows end here; the last 1 - 3 rows follow the loop
+    float a0[kSmallDepth][2][4], b0[kSmallDepth][NT], a1[kSmallDepth][2][4], b1[kSmallDepth][NT];
+    const auto fetch = [&](float (&a)[kSmallDepth][2][4], float (&b)[kSmallDepth][NT], int k_first) {
+        const int k0 = __builtin_amdgcn_readfirstlane(k_first);
+#pragma unroll
+        for (int u = 0; u < kSmallDepth; ++u) {
+            const int k = k0 + 4 * kSmallWaves * u;                // the group's first row: uniform
+            const bool live = k < ke_groups;
+            const unsigned keep_k = live ? 0xFFFFFFFFu : 0u;       // a group past the end reads rows kb .. kb + 3: zeros
+            const char *ra = reinterpret_cast<const char *>(A + (size_t)(live ? k : kb) * lda);
+            const char *rb = reinterpret_cast<const char *>(B + (size_t)(live ? k : kb) * ldb);
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const Float4U qa = *reinterpret_cast<const Float4U *>(ra + lane_a[h]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) a[u][h][i] = __uint_as_float(__float_as_uint(qa.v[i]) & keep_m[h][i] & keep_k);
+            }
+            const FloatNU<NT> qb = *reinterpret_cast<const FloatNU<NT> *>(rb + lane_b);
+#pragma unroll
+            for (int j = 0; j < NT; ++j) b[u][j] = __uint_as_float(__float_as_uint(qb.v[j]) & keep_n[j] & keep_k);
+        }
+    };
+    const auto multiply = [&](const float (&a)[kSmallDepth][2][4], const float (&b)[kSmallDepth][NT]) {
+#pragma unroll
+        for (int u = 0; u < kSmallDepth; ++u)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < NT; ++j)
+                        acc[h][i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u][h][i], b[u][j], acc[h][i][j], 0, 0, 0);
+    };
+    int k0 = kb + 4 * wave;
+    if (k0 < ke_groups) {  // the same for the whole wavefront
+        fetch(a0, b0, k0);
+        for (;;) {
+            fetch(a1, b1, k0 + step);
+            multiply(a0, b0);
+            k0 += step;
+            if (k0 >= ke_groups) break;
+            fetch(a0, b0, k0 + step);
+            multiply(a1, b1);
+            k0 += step;
+            if (k0 >= ke_groups) break;
+        }
+    }
+    if (wave == 0 && ke_groups < ke) {  // the last 1 - 3 rows of the range: a group whose other rows are zero
+        const bool live = ke_groups + lk < ke;
+        const unsigned keep_k = live ? 0xFFFFFFFFu : 0u;
+        const size_t row = (size_t)(live ? ke_groups + lk : ke_groups);
+        const FloatNU<NT> qb = *reinterpret_cast<const FloatNU<NT> *>(B + row * ldb + (NT * lm < N ? NT * lm : 0));
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const Float4U qa = *reinterpret_cast<const Float4U *>(A + row * lda + (64 * h + 4 * lm < M ? 64 * h + 4 * lm : 0));
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < NT; ++j)
+                    acc[h][i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                        __uint_as_float(__float_as_uint(qa.v[i]) & keep_m[h][i] & keep_k),
+                        __uint_as_float(__float_as_uint(qb.v[j]) & keep_n[j] & keep_k), acc[h][i][j], 0, 0, 0);
+        }
+    }
+    // The wavefronts' tiles, added in a fixed order: wavefronts 0 and 1 store theirs side by side, 2 and 3 add theirs on
+    // top, and the two sums are added on the way out.  Register v of lane l of tile (h, i, j) is row 4 (l / 16) + v and
+    // column l % 16 of the tile, i.e. output row 64 h + 4 * that row + i and output column NT * (l % 16) + j.
+    static_assert(kSmallWaves == 4, "two rounds of two wavefronts");
+    for (int round = 0; round < 2; ++round) {
+        if (wave / 2 == round) {
+            float *mine = s_tile + (wave & 1) * 128 * CP;
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < NT; ++j)
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) {
+                            float *cell = mine + (64 * h + 4 * (4 * lk + v) + i) * CP + NT * lm + j;
+                            *cell = round == 0 ? acc[h][i][j][v] : *cell + acc[h][i][j][v];
+                        }
+        }
+        __syncthreads();
+    }
+    float *out = partial + (size_t)blockIdx.x * M * N;
+    for (int idx = threadIdx.x; idx < M * N; idx += kSmallWaves * kWave) {
+        const int row = idx / N, col = idx - row * N;
+        out[idx] = s_tile[row * CP + col] + s_tile[128 * CP + row * CP + col];
+    }
+}
+
 // C = alpha * sum_z partial[z] + beta * C.  A work-group of 256 lanes owns 32 consecutive outputs; lane (o, g) adds the
 // partials z = g, g + 8, ... of output o (eight independent loads in flight), and the eight sums of an output are added
 // in g order - a fixed order, so the result is repeatable.  (One lane per output adding all the splits in turn took
@@ -407,7 +544,6 @@ __global__ __launch_bounds__(kReduceOutputs * kReduceGroups) void sgemm_reduce_k
 // What did not work: loading the operand layout straight from memory, every lane its own row, costs a cache lookup
 // per lane (64 per instruction): 19 us for the 119 MB of H even when all of it hits L1, 48 - 56 us in all; storing the
 // accumulators as they lie (64-byte pieces of four rows per instruction) 41 / 46.
-typedef float floatx4 __attribute__((ext_vector_type(4)));
 constexpr int kTallRows = 16, kTallGroups = 256;
 // Wavefronts per work-group: 12 where op(B) and 12 strips fit the 160 KB of LDS, else 8.
 constexpr int tall_waves(int kq, int nt)
@@ -632,21 +768,30 @@ int split_scratch(bool may_allocate, size_t floats, hipStream_t s, int M, int N,
     return static_scratch(partial);
 }
 
-// C = alpha * A^T * B + beta * C for a small output and a long reduction (see sgemm_tn_skinny_kernel).
+// C = alpha * A^T * B + beta * C for a small output and a long reduction (see sgemm_tn_skinny_kernel and
+// sgemm_tn_small_kernel, which takes the outputs whose rows of B can be read in whole pieces).
 int sgemm_tn_skinny(bool may_allocate, int M, int N, int K, float alpha, const float *A, int lda, const float *B, int ldb,
                     float beta, float *C, int ldc, hipStream_t s)
 {
+    const int nt = (N + 15) / 16;
+    const bool small = ldb >= (N + nt - 1) / nt * nt;  // a lane reads nt consecutive floats of B's row, also past N
     // two work-groups of four wavefronts per CU, each wavefront at least 16 steps of the reduction deep
+    const int rows_per_step = small ? 4 * kSmallWaves * kSmallDepth : 2 * kSkinnyWaves * kSkinnyDepth;
+    const int align = small ? 4 * kSmallWaves : 2 * kSkinnyWaves;
     int splits = DRONE_SKINNY_SPLITS;
-    const int deepest = (int)ceil_div(K, 2 * kSkinnyWaves * kSkinnyDepth * 16);
+    const int deepest = (int)ceil_div(K, rows_per_step * 16);
     if (splits > deepest) splits = deepest;
     if (splits < 1) splits = 1;
-    int k_chunk = (int)ceil_div(ceil_div(K, splits), 2 * kSkinnyWaves) * 2 * kSkinnyWaves;
+    int k_chunk = (int)ceil_div(ceil_div(K, splits), align) * align;
     splits = (int)ceil_div(K, k_chunk);
     float *partial = nullptr;
     const int rc = split_scratch(may_allocate, (size_t)splits * M * N, s, M, N, K, splits, &partial);
     if (rc != DRONE_OK) return rc;
-    sgemm_tn_skinny_kernel<<<splits, kSkinnyWaves * kWave, 0, s>>>(M, N, K, A, lda, B, ldb, k_chunk, partial);
+    if (!small) sgemm_tn_skinny_kernel<<<splits, kSkinnyWaves * kWave, 0, s>>>(M, N, K, A, lda, B, ldb, k_chunk, partial);
+    else if (nt == 1) sgemm_tn_small_kernel<1><<<splits, kSmallWaves * kWave, 0, s>>>(M, N, K, A, lda, B, ldb, k_chunk, partial);
+    else if (nt == 2) sgemm_tn_small_kernel<2><<<splits, kSmallWaves * kWave, 0, s>>>(M, N, K, A, lda, B, ldb, k_chunk, partial);
+    else if (nt == 3) sgemm_tn_small_kernel<3><<<splits, kSmallWaves * kWave, 0, s>>>(M, N, K, A, lda, B, ldb, k_chunk, partial);
+    else sgemm_tn_small_kernel<4><<<splits, kSmallWaves * kWave, 0, s>>>(M, N, K, A, lda, B, ldb, k_chunk, partial);
     launch_reduce(M, N, splits, partial, alpha, beta, C, ldc, s);
     DRONE_HIP_TRY(hipGetLastError());
     return DRONE_OK;
