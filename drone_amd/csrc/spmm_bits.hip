@@ -392,6 +392,60 @@ __global__ __launch_bounds__(256) void bits_combine_kernel(int rows, const int *
     }
 }
 
+// The same with 16-byte accesses: L lanes per ranked row (4 L >= K, K <= 256), 64 / L rows per wavefront.  wide_c: C's rows
+// can be read and written in aligned 16-byte pieces; the piece that holds column K - 1 goes float by float when K is not
+// a multiple of four (the tile sums' own rows are 128 floats long, so reading them past K is harmless).
+template <int L>
+__global__ __launch_bounds__(256) void bits_combine4_kernel(int rows, const int *__restrict__ tile_unit0,
+                                                            const float *__restrict__ partial, int num_units,
+                                                            const int *__restrict__ dense_row,
+                                                            const float *__restrict__ row_scale, float *__restrict__ C,
+                                                            int ldc, int K, float alpha, bool wide_c)
+{
+    constexpr int R = kWave / L;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int li = lane % L, sub = lane / L, k = 4 * li;
+    const int rr = (blockIdx.x * (256 / kWave) + wave) * R + sub;
+    if (rr >= rows || k >= K) return;
+    const int tile = rr / kBitTileRows, u0 = tile_unit0[tile], u1 = tile_unit0[tile + 1];
+    const int row = dense_row[rr];
+    const float scale = alpha * row_scale[row];
+    const float *src = partial + ((size_t)(k / 128) * num_units * kBitTileRows + rr % kBitTileRows) * kPartialLd + k % 128;
+    float *dst = C + (size_t)row * ldc + k;
+    const bool whole = wide_c && k + 4 <= K;
+    f32x4 before = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (whole) {
+        before = *reinterpret_cast<const f32x4 *>(dst);  // in flight with the tile sums
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (k + j < K) before[j] = dst[j];
+    }
+    f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+    // four loads in flight, added in unit order; a step past the tile's last unit repeats it and counts as zero
+    for (int u = u0; u < u1; u += 4) {
+        f32x4 v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int at = u + j < u1 ? u + j : u1 - 1;
+            v[j] = *reinterpret_cast<const f32x4 *>(src + (size_t)at * kBitTileRows * kPartialLd);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+            sum += u + j < u1 ? v[j] : zero;
+        }
+    }
+    const f32x4 out = before + scale * sum;
+    if (whole) {
+        *reinterpret_cast<f32x4 *>(dst) = out;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (k + j < K) dst[j] = out[j];
+    }
+}
+
 }  // namespace
 
 int bit_core_create(BitCore *bc, int rows, const std::vector<int> &width_of_row, const int *seg_begin, const int *seg_end,
@@ -531,8 +585,21 @@ int bit_core_add(const BitCore *bc, const int *dense_row, const float *row_scale
     const int passes = (int)ceil_div(K, 128);
     int grid = (int)ceil_div(bc->rows, 4);
     if (grid > 65536) grid = 65536;
-    bits_combine_kernel<<<grid, 256, 0, s>>>(bc->rows, bc->tile_unit0, bc->partial, bc->num_units, passes, dense_row,
-                                             row_scale, C, ldc, K, alpha);
+    if (K <= 256) {
+        const bool wide_c = ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0;
+        const auto launch = [&](auto kernel, int lanes) {
+            kernel<<<(int)ceil_div(bc->rows, 4 * (kWave / lanes)), 256, 0, s>>>(bc->rows, bc->tile_unit0, bc->partial, bc->num_units,
+                                                                               dense_row, row_scale, C, ldc, K, alpha, wide_c);
+        };
+        if (K <= 16) launch(bits_combine4_kernel<4>, 4);
+        else if (K <= 32) launch(bits_combine4_kernel<8>, 8);
+        else if (K <= 64) launch(bits_combine4_kernel<16>, 16);
+        else if (K <= 128) launch(bits_combine4_kernel<32>, 32);
+        else launch(bits_combine4_kernel<64>, 64);
+    } else {
+        bits_combine_kernel<<<grid, 256, 0, s>>>(bc->rows, bc->tile_unit0, bc->partial, bc->num_units, passes, dense_row,
+                                                 row_scale, C, ldc, K, alpha);
+    }
     DRONE_HIP_TRY(hipGetLastError());
     return DRONE_OK;
 }
