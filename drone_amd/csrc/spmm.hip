@@ -1237,10 +1237,15 @@ extern "C" int drone_spmm_csr_f32(const drone_spmm_plan *plan, const int *rp, co
     hipStream_t s = as_stream(stream);
     // The bit core's products run on the plan's side stream beside the gathers below (matrix cores and LDS there, the
     // L2 -> L1 path here): 2.75 against 2.88 ms at 128 feature columns, 1.35 against 1.45 at 41 on the 229 M-entry graph.
+    // (The split of B takes 0.2 ms there instead of 0.03 alone; run on the caller's stream before the fork it lets the
+    // products start that much earlier, but they then share the CUs with the gathers for longer: 8.78 ... 8.81 against
+    // 8.75 ... 9.07 ms per training step, 1.18 against 1.16 ms per 41-wide product - no gain, left beside the products.)
     if (plan->bits.tiles > 0) {
         DRONE_HIP_TRY(hipEventRecord(plan->bits.fork, s));
         DRONE_HIP_TRY(hipStreamWaitEvent(plan->bits.side, plan->bits.fork, 0));
-        const int st = bit_core_products(&plan->bits, plan->col_order, plan->col_scale, B, ldb, K, plan->bits.side);
+        int st = bit_core_split(&plan->bits, plan->col_order, plan->col_scale, B, ldb, K, plan->bits.side);
+        if (st != DRONE_OK) return st;
+        st = bit_core_products(&plan->bits, K, plan->bits.side);
         if (st != DRONE_OK) return st;
         DRONE_HIP_TRY(hipEventRecord(plan->bits.join, plan->bits.side));
     }

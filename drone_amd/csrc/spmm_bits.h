@@ -47,11 +47,13 @@ int bit_core_create(BitCore *bc, int rows, const std::vector<int> &width_of_row,
                     const int *cols, const int *col_rank, int max_k, hipStream_t s, bool *has_duplicates);
 void bit_core_destroy(BitCore *bc);
 
-// Two steps, so that the first can run beside the gathers of the rest of the matrix:
-// bit_core_products: T[rr, 0..K) = sum over ranked row rr's dense cells of col_scale[col] * B[col, 0..K), kept in the core's
-// scratch (col_order: rank -> column); bit_core_add: C[dense_row[rr], 0..K) += alpha * row_scale[dense_row[rr]] * T[rr, :].
-int bit_core_products(const BitCore *bc, const unsigned *col_order, const float *col_scale, const float *B, int ldb,
-                      int K, hipStream_t s);
+// Three steps, so that the second can run beside the gathers of the rest of the matrix:
+// bit_core_split: the scaled operand col_scale .* B in its three bf16 parts, for the ranked columns (col_order: rank ->
+// column); bit_core_products: T[rr, 0..K) = sum over ranked row rr's dense cells of that operand, kept in the core's
+// scratch; bit_core_add: C[dense_row[rr], 0..K) += alpha * row_scale[dense_row[rr]] * T[rr, :].
+int bit_core_split(const BitCore *bc, const unsigned *col_order, const float *col_scale, const float *B, int ldb, int K,
+                   hipStream_t s);
+int bit_core_products(const BitCore *bc, int K, hipStream_t s);
 int bit_core_add(const BitCore *bc, const int *dense_row, const float *row_scale, float *C, int ldc, int K, float alpha,
                  hipStream_t s);
 

@@ -550,19 +550,28 @@ void bit_core_destroy(BitCore *bc)
     *bc = BitCore();
 }
 
-int bit_core_products(const BitCore *bc, const unsigned *col_order, const float *col_scale, const float *B, int ldb,
-                      int K, hipStream_t s)
+int bit_core_split(const BitCore *bc, const unsigned *col_order, const float *col_scale, const float *B, int ldb, int K,
+                   hipStream_t s)
 {
     if (bc->tiles == 0) return DRONE_OK;
     DRONE_REQUIRE(K > 0 && K <= bc->max_k, "K exceeds the plan's feature width");
     const int groups = bc->wmax / 8, passes = (int)ceil_div(K, 128);
     bits_split_kernel<<<dim3((unsigned)ceil_div(groups, 2), (unsigned)passes), 256, 0, s>>>(groups, col_order, col_scale, B,
                                                                                            ldb, K, bc->split);
+    DRONE_HIP_TRY(hipGetLastError());
+    return DRONE_OK;
+}
+
+int bit_core_products(const BitCore *bc, int K, hipStream_t s)
+{
+    if (bc->tiles == 0) return DRONE_OK;
+    DRONE_REQUIRE(K > 0 && K <= bc->max_k, "K exceeds the plan's feature width");
+    const int groups = bc->wmax / 8, passes = (int)ceil_div(K, 128);
     for (int pass = 0; pass < passes; ++pass) {
         const int width = std::min(K - pass * 128, 128);
         const uint4 *split = bc->split + (size_t)pass * groups * kGroupVecs;
         float *partial = bc->partial + (size_t)pass * bc->num_units * kBitTileRows * kPartialLd;
-        // as many 32-column feature tiles as the pass holds (the plan's cost model prices the cells per such tile)
+        // as many feature tiles as the pass holds (the plan's cost model prices the cells per 32-column tile)
         const auto launch = [&](auto kernel) {
             kernel<<<bc->num_units, 512, 0, s>>>(bc->unit_tile, bc->unit_c0, bc->unit_c1, bc->unit_slot, bc->tile_blocks,
                                                  bc->tile_off, bc->bits, split, partial);
