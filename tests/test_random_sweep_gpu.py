@@ -143,7 +143,7 @@ def test_scaled_pattern_spmm_random(T, case, monkeypatch):
     rng = np.random.default_rng(5000 + case)
     n_rows = int(rng.choice([600, 1100, 4096, 4100, 5000, 9000]))
     n_cols = int(rng.choice([2048, 2049, 4095, 4100, 6500, 9000]))
-    K = int(rng.choice([1, 7, 32, 33, 41, 64, 65, 100, 128, 129, 200, 256]))
+    K = int(rng.choice([1, 7, 16, 17, 32, 33, 41, 48, 49, 64, 65, 100, 128, 129, 144, 200, 256]))
     ld_pad = int(rng.choice([0, 0, 3, 4]))
     long_rows = int(rng.choice([1, 40, 511, 512, 513, 700, 3000])) if n_rows > 700 else int(rng.choice([1, 40, 300]))
     long_rows = min(long_rows, n_rows)
