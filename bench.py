@@ -642,7 +642,9 @@ def main():
                      "traffic": pr_traffic_from_profile() if (args.scale == 24 and n == 16777216) else None,
                      "traffic_source": "profiles/pr_rowblock_pagerank_c2.hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / "
                                        "WRITE_SIZE of this command, scaled by the 1 GiB copy kernel)",
-                     "kernel": "one iteration: " + " + ".join(PR_KERNELS) + " + row fix-up (whose last work-group reduces the dangling mass)",
+                     "kernel": "one iteration: " + " + ".join(PR_KERNELS if (args.scale == 24 and n == 16777216) else
+                                                             ("pr_rowblock_kernel<drone::PrF64Epi, 4 or 6>", "pr_rowblock_merge_kernel<drone::PrF64Epi>"))
+                               + " + row fix-up (whose last work-group reduces the dangling mass)",
                      "algorithmic_bytes_per_launch": bytes_iter, "mean_launch_ms": prof["mean_ms"],
                      "launches_timed": prof["launches"]},
         "plan_ms_one_off": plan_s * 1e3,
